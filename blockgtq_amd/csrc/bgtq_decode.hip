@@ -1,0 +1,417 @@
+// Fused unpack + dequant + split-T decode attention, the partition merge, and
+// the dense fp16 window partial, for gfx950.
+//
+// decode_generic_kernel is the layout-agnostic path: any segment table, both K
+// layouts, both V layouts, any row stride.  One work-group of 256 threads owns
+// one partition of one (batch row, KV head).  Per 256-token tile the packed K
+// rows, K norms, packed V rows and V norms are staged into LDS with coalesced
+// loads; thread t then scores token t against all query heads of the group
+// (codes pulled out of the staged record with shift/mask, codebooks and the
+// rotated queries read from LDS), the tile maximum is reduced across the
+// work-group, and thread (d, half) accumulates output dim d for one half of
+// the query heads over the tile's tokens.
+#include "bgtq_common.h"
+
+namespace {
+
+constexpr int D = BGTQ_D;
+constexpr int GT = 256;          // threads == tokens per tile of the generic kernel
+constexpr int ROW_PAD = 4;       // slack bytes so a 2-byte window never leaves the tile
+
+struct DecodeArgs {
+    const bgtq_head_plan* plans;
+    const uint16_t* q;  int64_t q_sb, q_sh;
+    const uint8_t* kp;  int64_t kp_sb, kp_sh, kp_st;
+    const uint16_t* kn; int64_t kn_sb, kn_sh, kn_st;
+    const uint8_t* vp;  int64_t vp_sb, vp_sh, vp_st;
+    const uint16_t* vn; int64_t vn_sb, vn_sh, vn_st;
+    const int32_t* seq_lens; int T;
+    int B, n_kv, gqa, n_splits;
+    float* part_out; float* part_lse;
+    int k_layout, v_layout;
+    float scale;
+    int k_row_width;       // widest K record over the heads (LDS sizing)
+    int v_row_width;
+};
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// code of width `bw` at absolute bit `bit` of a staged record
+__device__ inline unsigned take_bits(const uint8_t* row, int bit, int bw) {
+    int byte = bit >> 3;
+    unsigned w = (unsigned)row[byte] | ((unsigned)row[byte + 1] << 8);
+    return (w >> (bit & 7)) & ((1u << bw) - 1u);
+}
+
+template <int GQA_MAX>
+__global__ __launch_bounds__(GT) void decode_generic_kernel(DecodeArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x;
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const bgtq_head_plan& P = a.plans[h];
+    const int gqa = a.gqa;
+
+    const int T = a.seq_lens ? a.seq_lens[b] : a.T;
+    const int chunk = (T + a.n_splits - 1) / a.n_splits;
+    const int t0 = min(c * chunk, T);
+    const int t1 = min(t0 + chunk, T);
+
+    // ---- LDS carve-up ------------------------------------------------------
+    const int krow = (a.k_row_width + ROW_PAD + 3) & ~3;
+    const int vrow = (a.v_row_width + ROW_PAD + 3) & ~3;
+    float* q_s = (float*)smem;                               // [GQA_MAX][D]
+    float* cb_s = q_s + GQA_MAX * D;                         // [8][256]
+    float* vlut_s = cb_s + BGTQ_MAX_SEGMENTS * BGTQ_MAX_CENTROIDS;  // [16]
+    float* p_s = vlut_s + 16;                                // [GQA_MAX][GT]
+    float* red_s = p_s + GQA_MAX * GT;                       // [GQA_MAX][4]
+    float* alpha_s = red_s + GQA_MAX * 4;                    // [GQA_MAX] rescale of the tile
+    float* fin_s = alpha_s + GQA_MAX;                        // [2][GQA_MAX] final m, l
+    float* kn_s = fin_s + 2 * GQA_MAX;                       // [GT][8]
+    float* vn_s = kn_s + GT * BGTQ_MAX_SEGMENTS;             // [GT]
+    uint32_t* dim_s = (uint32_t*)(vn_s + GT);                // [D] bit | bw<<16 | seg<<24
+    uint8_t* krow_s = (uint8_t*)(dim_s + D);                 // [GT][krow]
+    uint8_t* vrow_s = krow_s + (size_t)GT * krow;            // [GT][vrow]
+
+    // ---- static tables -----------------------------------------------------
+    for (int i = tid; i < gqa * D; i += GT) {
+        int hq = i / D, d = i - hq * D;
+        q_s[i] = bgtq_h2f(a.q[b * a.q_sb + (h * gqa + hq) * a.q_sh + d]);
+    }
+    for (int i = tid; i < BGTQ_MAX_SEGMENTS * BGTQ_MAX_CENTROIDS; i += GT)
+        cb_s[i] = bgtq_h2f(P.k_codebook_f16[i >> 8][i & 255]);
+    if (tid < 16) vlut_s[tid] = bgtq_h2f(P.v_lut_f16[tid]);
+    if (tid < D) {
+        int g = P.group_of[tid];
+        uint32_t e = 0xFFFFFFFFu;
+        if (g >= 0) {
+            int bw = P.seg_bw[g], rel = tid - P.seg_start[g];
+            int bit, xbw;
+            if (a.k_layout == BGTQ_K_MIXED) {
+                if (bw <= 4) { bit = (tid - P.n_zero_dims) * 4; xbw = 4; }
+                else         { bit = (P.seg_mixed_off[g] + rel) * 8; xbw = 8; }
+            } else {
+                if (bw <= 4) { bit = P.seg_pack_off[g] * 8 + rel * bw; xbw = bw; }
+                else         { bit = (P.seg_pack_off[g] + rel) * 8; xbw = 8; }
+            }
+            e = (uint32_t)bit | ((uint32_t)xbw << 16) | ((uint32_t)g << 24);
+        }
+        dim_s[tid] = e;
+    }
+    const int n_seg = P.n_seg;
+    const int kbytes = min((a.k_layout == BGTQ_K_MIXED) ? P.k_mixed_bytes : P.k_row_bytes,
+                           a.k_row_width);
+    const int vbw = (a.v_layout == BGTQ_V_NIBBLE) ? 4 : P.v_bits;
+    const int vbytes = min(bgtq_seg_bytes(vbw, D), a.v_row_width);
+
+    const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
+    const uint16_t* kn_base = a.kn + b * a.kn_sb + h * a.kn_sh;
+    const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
+    const uint16_t* vn_base = a.vn + b * a.vn_sb + h * a.vn_sh;
+
+    // running softmax state (replicated in every thread) and output accumulators
+    float m_run[GQA_MAX], l_run[GQA_MAX];
+    const int hhalf = (GQA_MAX + 1) / 2;         // heads per PV thread
+    float acc[(GQA_MAX + 1) / 2];
+#pragma unroll
+    for (int i = 0; i < GQA_MAX; i++) { m_run[i] = -INFINITY; l_run[i] = 0.f; }
+#pragma unroll
+    for (int i = 0; i < hhalf; i++) acc[i] = 0.f;
+    const int pv_d = tid & (D - 1);
+    const int pv_h0 = (tid >> 7) * hhalf;
+
+    for (int tile = t0; tile < t1; tile += GT) {
+        const int nt = min(GT, t1 - tile);
+        __syncthreads();   // previous tile fully consumed (also orders the static tables)
+        // ---- stage the tile -----------------------------------------------
+        for (int i = tid; i < nt * kbytes; i += GT) {
+            int t = i / kbytes, o = i - t * kbytes;
+            krow_s[t * krow + o] = kp_base[(int64_t)(tile + t) * a.kp_st + o];
+        }
+        for (int i = tid; i < nt * vbytes; i += GT) {
+            int t = i / vbytes, o = i - t * vbytes;
+            vrow_s[t * vrow + o] = vp_base[(int64_t)(tile + t) * a.vp_st + o];
+        }
+        for (int i = tid; i < nt * n_seg; i += GT) {
+            int t = i / n_seg, g = i - t * n_seg;
+            kn_s[t * BGTQ_MAX_SEGMENTS + g] = bgtq_h2f(kn_base[(int64_t)(tile + t) * a.kn_st + g]);
+        }
+        if (tid < nt) vn_s[tid] = bgtq_h2f(vn_base[(int64_t)(tile + tid) * a.vn_st]);
+        __syncthreads();
+
+        // ---- scores: thread = token ------------------------------------------
+        float logit[GQA_MAX];
+#pragma unroll
+        for (int i = 0; i < GQA_MAX; i++) logit[i] = -INFINITY;
+        if (tid < nt) {
+            const uint8_t* row = krow_s + tid * krow;
+            float tot[GQA_MAX], part[GQA_MAX];
+#pragma unroll
+            for (int i = 0; i < GQA_MAX; i++) { tot[i] = 0.f; part[i] = 0.f; }
+            int cur = -1;
+            for (int d = P.n_zero_dims; d < D; d++) {
+                uint32_t e = dim_s[d];
+                int g = (int)(e >> 24);
+                if (g != cur) {
+                    if (cur >= 0) {
+                        float n = kn_s[tid * BGTQ_MAX_SEGMENTS + cur];
+#pragma unroll
+                        for (int i = 0; i < GQA_MAX; i++) { tot[i] += part[i] * n; part[i] = 0.f; }
+                    }
+                    cur = g;
+                }
+                unsigned code = take_bits(row, (int)(e & 0xFFFFu), (int)((e >> 16) & 0xFFu));
+                float cv = cb_s[g * BGTQ_MAX_CENTROIDS + code];
+#pragma unroll
+                for (int i = 0; i < GQA_MAX; i++)
+                    if (i < gqa) part[i] += q_s[i * D + d] * cv;
+            }
+            if (cur >= 0) {
+                float n = kn_s[tid * BGTQ_MAX_SEGMENTS + cur];
+#pragma unroll
+                for (int i = 0; i < GQA_MAX; i++) tot[i] += part[i] * n;
+            }
+#pragma unroll
+            for (int i = 0; i < GQA_MAX; i++) logit[i] = tot[i] * a.scale;
+        }
+
+        // ---- tile maximum per head (work-group reduce) -------------------------
+#pragma unroll
+        for (int i = 0; i < GQA_MAX; i++) {
+            float m = wave_max(logit[i]);
+            if ((tid & 63) == 0) red_s[i * 4 + (tid >> 6)] = m;
+        }
+        __syncthreads();
+        float alpha[GQA_MAX];
+#pragma unroll
+        for (int i = 0; i < GQA_MAX; i++) {
+            float m = fmaxf(fmaxf(red_s[i * 4], red_s[i * 4 + 1]),
+                            fmaxf(red_s[i * 4 + 2], red_s[i * 4 + 3]));
+            float m_new = fmaxf(m_run[i], m);
+            alpha[i] = (m_run[i] == -INFINITY) ? 0.f : __expf(m_run[i] - m_new);
+            m_run[i] = m_new;
+            float p = (tid < nt && i < gqa) ? __expf(logit[i] - m_new) : 0.f;
+            p_s[i * GT + tid] = p * ((tid < nt) ? vn_s[tid] : 0.f);   // V norm folded into p
+            logit[i] = p;
+            if (tid == 0) alpha_s[i] = alpha[i];
+        }
+        __syncthreads();   // red_s consumed, p_s visible
+#pragma unroll
+        for (int i = 0; i < GQA_MAX; i++) {
+            float s = wave_sum(logit[i]);
+            if ((tid & 63) == 0) red_s[i * 4 + (tid >> 6)] = s;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < GQA_MAX; i++) {
+            float s = red_s[i * 4] + red_s[i * 4 + 1] + red_s[i * 4 + 2] + red_s[i * 4 + 3];
+            l_run[i] = l_run[i] * alpha[i] + s;
+        }
+
+        // ---- values: thread = (dim, half of the heads) ------------------------
+#pragma unroll
+        for (int i = 0; i < hhalf; i++)
+            if (pv_h0 + i < GQA_MAX) acc[i] *= alpha_s[pv_h0 + i];
+        for (int t = 0; t < nt; t++) {
+            unsigned code = take_bits(vrow_s + t * vrow, pv_d * vbw, vbw);
+            float val = vlut_s[code];
+#pragma unroll
+            for (int i = 0; i < hhalf; i++)
+                if (pv_h0 + i < GQA_MAX) acc[i] += p_s[(pv_h0 + i) * GT + t] * val;
+        }
+    }
+
+    // ---- partition result --------------------------------------------------------
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int i = 0; i < GQA_MAX; i++) { fin_s[i] = m_run[i]; fin_s[GQA_MAX + i] = l_run[i]; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < hhalf; i++) {
+        int hq = pv_h0 + i;
+        if (hq < gqa) {
+            float l = fin_s[GQA_MAX + hq];
+            float o = (t1 > t0) ? acc[i] / l : 0.f;
+            size_t row = ((size_t)b * a.n_kv * gqa + (size_t)h * gqa + hq) * a.n_splits + c;
+            a.part_out[row * D + pv_d] = o;
+        }
+    }
+    if (tid < gqa) {
+        float lse = (t1 > t0) ? fin_s[tid] + __logf(fin_s[GQA_MAX + tid]) : -INFINITY;
+        size_t row = ((size_t)b * a.n_kv * gqa + (size_t)h * gqa + tid) * a.n_splits + c;
+        a.part_lse[row] = lse;
+    }
+}
+
+size_t generic_smem_bytes(int gqa_max, int krow_bytes, int vrow_bytes) {
+    size_t krow = (size_t)((krow_bytes + ROW_PAD + 3) & ~3);
+    size_t vrow = (size_t)((vrow_bytes + ROW_PAD + 3) & ~3);
+    size_t f = (size_t)gqa_max * D + BGTQ_MAX_SEGMENTS * BGTQ_MAX_CENTROIDS + 16 +
+               (size_t)gqa_max * GT + (size_t)gqa_max * 7 + (size_t)GT * BGTQ_MAX_SEGMENTS + GT + D;
+    return f * 4 + (size_t)GT * (krow + vrow) + 16;
+}
+
+template <int GQA_MAX>
+int launch_generic(const DecodeArgs& a, hipStream_t st) {
+    size_t smem = generic_smem_bytes(GQA_MAX, a.k_row_width, a.v_row_width);
+    auto kern = decode_generic_kernel<GQA_MAX>;
+    if (smem > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return (int)e;
+    }
+    dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)a.B);
+    hipLaunchKernelGGL(kern, grid, dim3(GT), smem, st, a);
+    return bgtq_launch_status();
+}
+
+// ---- partition merge + V un-rotation ------------------------------------------
+__global__ __launch_bounds__(D) void lse_reduce_kernel(
+    const bgtq_head_plan* plans, const float* part_out, const float* part_lse, int n_splits,
+    const float* extra_out, const float* extra_lse, int n_extra,
+    int n_q, int gqa, int unrotate, uint16_t* out, int64_t o_sb, int64_t o_sh, float* lse_out) {
+    __shared__ float vec[D];
+    const int j = threadIdx.x;
+    const int hq = blockIdx.x, b = blockIdx.y;
+    const size_t row = (size_t)b * n_q + hq;
+    const float* pl = part_lse + row * n_splits;
+    const float* el = extra_lse ? extra_lse + row * n_extra : nullptr;
+
+    float m = -INFINITY;
+    for (int c = 0; c < n_splits; c++) m = fmaxf(m, pl[c]);
+    for (int c = 0; c < n_extra; c++) m = fmaxf(m, el[c]);
+    if (m == -INFINITY) {                      // nothing visible at all
+        out[b * o_sb + hq * o_sh + j] = 0;
+        if (lse_out && j == 0) lse_out[row] = -INFINITY;
+        return;
+    }
+    float den = 0.f, accp = 0.f, acce = 0.f;
+    for (int c = 0; c < n_splits; c++) {
+        float l = pl[c];
+        if (l == -INFINITY) continue;          // empty partition: its vector is undefined
+        float w = __expf(l - m);
+        den += w;
+        accp += w * part_out[(row * n_splits + c) * D + j];
+    }
+    for (int c = 0; c < n_extra; c++) {
+        float l = el[c];
+        if (l == -INFINITY) continue;
+        float w = __expf(l - m);
+        den += w;
+        acce += w * extra_out[(row * n_extra + c) * D + j];
+    }
+    float res = accp;
+    if (unrotate) {
+        vec[j] = accp;
+        __syncthreads();
+        const float* R = plans[hq / gqa].v_rot;
+        float r = 0.f;
+        for (int k = 0; k < D; k++) r += vec[k] * R[k * D + j];
+        res = r;
+    }
+    out[b * o_sb + hq * o_sh + j] = bgtq_f2h((res + acce) / den);
+    if (lse_out && j == 0) lse_out[row] = m + __logf(den);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t bgtq_workspace_bytes(int B, int n_q, int n_splits) {
+    if (B <= 0 || n_q <= 0 || n_splits <= 0) return 0;
+    return (size_t)B * n_q * n_splits * (D + 1) * sizeof(float);
+}
+
+int bgtq_default_splits(int B, int n_kv, int max_T) {
+    // Enough partitions to put several work-groups on each of the 256 CUs, but
+    // never fewer than 256 tokens per partition.
+    if (B <= 0 || n_kv <= 0 || max_T <= 0) return 1;
+    int by_tokens = (max_T + 255) / 256;
+    int want = (1024 + B * n_kv - 1) / (B * n_kv);
+    int s = want < by_tokens ? want : by_tokens;
+    if (s < 1) s = 1;
+    if (s > BGTQ_MAX_SPLITS) s = BGTQ_MAX_SPLITS;
+    return s;
+}
+
+int bgtq_decode_attn(const bgtq_head_plan* plans,
+                     const void* q_rot, int64_t q_sb, int64_t q_sh,
+                     const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                     const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                     const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                     const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                     const int32_t* seq_lens, int T,
+                     int B, int n_kv, int gqa, int n_splits,
+                     float* partial_out, float* partial_lse,
+                     int k_layout, int v_layout, float scale, void* stream) {
+    BGTQ_CHECK_ARG(plans && q_rot && k_packed && k_norms && v_packed && v_norms);
+    BGTQ_CHECK_ARG(partial_out && partial_lse);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && T >= 0);
+    BGTQ_CHECK_ARG(gqa >= 1 && gqa <= BGTQ_MAX_GQA);
+    BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
+    BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
+    if (n_splits > BGTQ_MAX_SPLITS) return BGTQ_ELIMIT;
+    BGTQ_CHECK_ARG(n_splits >= 1);
+    if (B == 0 || n_kv == 0) return BGTQ_OK;
+    DecodeArgs a{};
+    a.plans = plans;
+    a.q = (const uint16_t*)q_rot; a.q_sb = q_sb; a.q_sh = q_sh;
+    a.kp = (const uint8_t*)k_packed; a.kp_sb = kp_sb; a.kp_sh = kp_sh; a.kp_st = kp_st;
+    a.kn = (const uint16_t*)k_norms; a.kn_sb = kn_sb; a.kn_sh = kn_sh; a.kn_st = kn_st;
+    a.vp = (const uint8_t*)v_packed; a.vp_sb = vp_sb; a.vp_sh = vp_sh; a.vp_st = vp_st;
+    a.vn = (const uint16_t*)v_norms; a.vn_sb = vn_sb; a.vn_sh = vn_sh; a.vn_st = vn_st;
+    a.seq_lens = seq_lens; a.T = T;
+    a.B = B; a.n_kv = n_kv; a.gqa = gqa; a.n_splits = n_splits;
+    a.part_out = partial_out; a.part_lse = partial_lse;
+    a.k_layout = k_layout; a.v_layout = v_layout; a.scale = scale;
+    BGTQ_CHECK_ARG(k_row_width >= 1 && k_row_width <= BGTQ_D);
+    BGTQ_CHECK_ARG(v_row_width >= 1 && v_row_width <= BGTQ_D / 2);
+    a.k_row_width = k_row_width; a.v_row_width = v_row_width;
+    hipStream_t st = (hipStream_t)stream;
+    if (gqa <= 4) return launch_generic<4>(a, st);
+    if (gqa <= 8) return launch_generic<8>(a, st);
+    return launch_generic<16>(a, st);
+}
+
+int bgtq_lse_reduce(const bgtq_head_plan* plans,
+                    const float* partial_out, const float* partial_lse, int n_splits,
+                    const float* extra_out, const float* extra_lse, int n_extra,
+                    int B, int n_kv, int gqa, int unrotate,
+                    void* out, int64_t o_sb, int64_t o_sh,
+                    float* lse_out, void* stream) {
+    BGTQ_CHECK_ARG(plans && partial_out && partial_lse && out);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && gqa >= 1 && n_splits >= 1 && n_extra >= 0);
+    BGTQ_CHECK_ARG(n_extra == 0 || (extra_out && extra_lse));
+    if (B == 0 || n_kv == 0) return BGTQ_OK;
+    dim3 grid((unsigned)(n_kv * gqa), (unsigned)B);
+    hipLaunchKernelGGL(lse_reduce_kernel, grid, dim3(D), 0, (hipStream_t)stream,
+                       plans, partial_out, partial_lse, n_splits,
+                       n_extra ? extra_out : nullptr, n_extra ? extra_lse : nullptr, n_extra,
+                       n_kv * gqa, gqa, unrotate, (uint16_t*)out, o_sb, o_sh, lse_out);
+    return bgtq_launch_status();
+}
+
+size_t bgtq_plan_sizeof(void) { return sizeof(bgtq_head_plan); }
+int bgtq_abi_version(void) { return 1; }
+
+const char* bgtq_strerror(int code) {
+    switch (code) {
+    case BGTQ_OK: return "ok";
+    case BGTQ_EINVAL: return "invalid argument";
+    case BGTQ_EUNSUPPORTED: return "not supported by this build";
+    case BGTQ_ELIMIT: return "size beyond a documented maximum";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}
+
+}  // extern "C"

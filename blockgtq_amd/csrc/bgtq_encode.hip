@@ -1,0 +1,388 @@
+// K / V quantise-and-pack kernels and the query rotation for gfx950.
+//
+// Arithmetic contract (what "bit-exact" means for the packed bytes): every
+// reduction over coordinates is a chain of fused multiply-adds in ascending
+// packed-dim order starting from +0, square roots and divisions are IEEE
+// correctly rounded, and the rotation of coordinate j of a group spanning dims
+// [s, e) is fma(xhat[k], R_T[k][j], acc) for k = s .. e-1 (skipped altogether,
+// y = xhat, when the group's rotation block is the identity).  This file is
+// compiled with floating-point contraction off so nothing else fuses.
+//
+// One work-group of 128 threads encodes ROWS token rows of one KV head:
+// thread j owns packed dim j during normalise / rotate / quantise and output
+// byte j while packing.  The rotation matrix is read once per work-group
+// (coalesced across j, served from L2) and reused for all ROWS rows out of
+// registers; rows are staged in LDS so the k-loop reads them as broadcasts.
+#include "bgtq_common.h"
+
+namespace {
+
+constexpr int D = BGTQ_D;
+constexpr int NT = 128;  // threads per work-group
+
+struct EncodeArgs {
+    const bgtq_head_plan* plans;
+    const uint16_t* x;          // fp16 [B][n_kv][S][128]
+    int64_t x_sb, x_sh, x_ss;
+    int B, n_kv, S;
+    uint8_t* packed;            // cache records, or nullptr
+    int64_t p_sb, p_sh, p_st;
+    int row_width;
+    uint16_t* norms;            // fp16 cache norms, or nullptr
+    int64_t n_sb, n_sh, n_st;
+    int norm_width;
+    const int32_t* t_pos;
+    int t_pos_scalar;
+    int layout;
+    int quant_mode;
+    uint8_t* codes_out;         // [N][128] unpacked codes, or nullptr
+    float* norms_f32_out;       // K: [N][norm_width] fp32; or nullptr
+    int corrected;              // K codes path: emit corrected norms
+};
+
+// LSB-first stream of bw-bit codes -> byte `idx`; codes past `len` read as 0.
+__device__ inline unsigned stream_byte(const uint8_t* codes, int len, int bw, int idx) {
+    unsigned out = 0;
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        int bit = idx * 8 + b;
+        int ci = bit / bw;
+        unsigned c = ci < len ? codes[ci] : 0u;
+        out |= ((c >> (bit - ci * bw)) & 1u) << b;
+    }
+    return out;
+}
+
+template <int ROWS, bool IS_V>
+__global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
+    __shared__ float xs[ROWS][D];
+    __shared__ float nrm[ROWS][BGTQ_MAX_SEGMENTS];
+    __shared__ float nrm_out[ROWS][BGTQ_MAX_SEGMENTS];
+    __shared__ uint8_t cds[ROWS][D];
+
+    const int j = threadIdx.x;
+    const int h = blockIdx.y;
+    const bgtq_head_plan& P = a.plans[h];
+    const int64_t N = (int64_t)a.B * a.S;
+    const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+
+    // ---- per-thread static data -------------------------------------------
+    const int n_seg = IS_V ? 1 : P.n_seg;
+    const int g = IS_V ? 0 : P.group_of[j];
+    int gs = 0, ge = D, ident = 0;
+    if (!IS_V) {
+        if (g >= 0) { gs = P.seg_start[g]; ge = gs + P.seg_len[g]; ident = P.seg_identity[g]; }
+        else        { gs = 0; ge = 0; }
+    }
+    const float* RT = IS_V ? P.v_rot_T : P.k_rot_T;
+    const int src_dim = IS_V ? j : P.head_perm[j];
+
+    // ---- 1. load (gather by head_perm for K), fp16 -> fp32 -----------------
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        int64_t n = row0 + r;
+        float v = 0.f;
+        if (n < N) {
+            int64_t b = n / a.S, s = n - b * a.S;
+            v = bgtq_h2f(a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + src_dim]);
+        }
+        xs[r][j] = v;
+    }
+    __syncthreads();
+
+    // ---- 2. group norms: thread (r, grp) runs one sequential chain ---------
+    if (j < ROWS * BGTQ_MAX_SEGMENTS) {
+        int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
+        float n = 0.f;
+        if (gg < n_seg) {
+            int s = IS_V ? 0 : P.seg_start[gg];
+            int e = IS_V ? D : s + P.seg_len[gg];
+            float ss = 0.f;
+            for (int k = s; k < e; k++) ss = __builtin_fmaf(xs[r][k], xs[r][k], ss);
+            n = __builtin_sqrtf(ss + 1e-30f);
+        }
+        nrm[r][gg] = n;
+    }
+    __syncthreads();
+
+    // ---- 3. normalise -------------------------------------------------------
+    float xh[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        float v = 0.f;
+        if (g >= 0) {
+            float n = nrm[r][g];
+            float safe = (n > (IS_V ? 1e-8f : 1e-10f)) ? n : 1.0f;
+            v = xs[r][j] / safe;
+        }
+        xh[r] = v;
+        xs[r][j] = v;     // only this thread ever touched xs[r][j] since the barrier
+    }
+    __syncthreads();
+
+    // ---- 4. rotate ------------------------------------------------------------
+    float y[ROWS];
+    if (ident || g < 0) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) y[r] = xh[r];
+    } else {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) y[r] = 0.f;
+        for (int k = gs; k < ge; k++) {
+            float rt = RT[k * D + j];
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][k], rt, y[r]);
+        }
+    }
+
+    // ---- 5. scalar quantise ---------------------------------------------------
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        int code = 0;
+        if (IS_V) {
+            int nb = (1 << P.v_bits) - 1;
+            for (int b = 0; b < nb; b++) code += (y[r] > P.v_boundaries[b]) ? 1 : 0;
+        } else if (g >= 0) {
+            if (a.quant_mode == BGTQ_QUANT_EXACT) {
+                int nb = (1 << P.seg_bw[g]) - 1;
+                for (int b = 0; b < nb; b++) code += (P.k_boundaries[g][b] < y[r]) ? 1 : 0;
+            } else {
+                float t = (y[r] - P.lut_offset[j]) * P.lut_inv_scale[j];
+                t = fminf(fmaxf(t, 0.0f), (float)(BGTQ_LUT_BINS - 1));
+                code = P.code_lut[g][(int)t];
+            }
+        }
+        cds[r][j] = (uint8_t)code;
+    }
+    __syncthreads();
+
+    // ---- 6. norms to store (raw or divided by ||centroids[codes]||) ---------
+    if (j < ROWS * BGTQ_MAX_SEGMENTS) {
+        int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
+        float out = 0.f;
+        if (gg < n_seg) {
+            float n = nrm[r][gg];
+            if (IS_V) {
+                float cs = 0.f;
+                for (int k = 0; k < D; k++) {
+                    float c = P.v_centroids[cds[r][k]];
+                    cs = __builtin_fmaf(c, c, cs);
+                }
+                float cn = __builtin_sqrtf(cs + 1e-20f);
+                out = n / (cn > 1e-10f ? cn : 1.0f);
+            } else if (a.layout == BGTQ_K_MIXED || a.corrected) {
+                int s = P.seg_start[gg], e = s + P.seg_len[gg];
+                float cs = 0.f;
+                for (int k = s; k < e; k++) {
+                    float c = P.k_centroids[gg][cds[r][k]];
+                    cs = __builtin_fmaf(c, c, cs);
+                }
+                out = n / fmaxf(__builtin_sqrtf(cs), 1e-10f);
+            } else {
+                out = n;
+            }
+        }
+        nrm_out[r][gg] = out;
+    }
+    __syncthreads();
+
+    // ---- 7a. unpacked outputs (codes path) ------------------------------------
+    if (a.codes_out) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            int64_t n = row0 + r;
+            if (n < N) a.codes_out[n * D + j] = cds[r][j];
+        }
+        if (IS_V) {
+            if (j < ROWS && row0 + j < N && a.norms)
+                a.norms[row0 + j] = bgtq_f2h(nrm_out[j][0]);
+        } else if (a.norms_f32_out && j < ROWS * BGTQ_MAX_SEGMENTS) {
+            int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
+            if (row0 + r < N && gg < a.norm_width)
+                a.norms_f32_out[(row0 + r) * a.norm_width + gg] = nrm_out[r][gg];
+        }
+        return;
+    }
+
+    // ---- 7b. cache norms --------------------------------------------------------
+    if (j < ROWS * BGTQ_MAX_SEGMENTS) {
+        int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
+        int64_t n = row0 + r;
+        int width = IS_V ? 1 : a.norm_width;
+        if (n < N && gg < width) {
+            int64_t b = n / a.S, s = n - b * a.S;
+            int64_t t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            a.norms[b * a.n_sb + h * a.n_sh + t * a.n_st + gg] = bgtq_f2h(nrm_out[r][gg]);
+        }
+    }
+
+    // ---- 8. pack: thread j produces output byte j of every row ---------------
+    if (j >= a.row_width) return;
+    int mode = 0;        // 0: zero fill, 1: bit stream, 2: raw byte copy
+    int c0 = 0, clen = 0, bw = 1, idx = 0;
+    if (IS_V) {
+        bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : P.v_bits;
+        if (j < bgtq_seg_bytes(bw, D)) { mode = 1; c0 = 0; clen = D; idx = j; }
+    } else if (a.layout == BGTQ_K_MIXED) {
+        int z = P.n_zero_dims;
+        int nib = (P.nopack_start - z) >> 1;
+        if (j < nib)                     { mode = 1; bw = 4; c0 = z; clen = P.nopack_start - z; idx = j; }
+        else if (j < nib + P.nopack_len) { mode = 2; c0 = P.nopack_start + (j - nib); }
+    } else {
+        for (int s = 0; s < P.n_seg; s++) {
+            int off = P.seg_pack_off[s], sb = P.seg_bw[s], sl = P.seg_len[s];
+            if (j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
+                if (sb >= 5) { mode = 2; c0 = P.seg_start[s] + (j - off); }
+                else         { mode = 1; bw = sb; c0 = P.seg_start[s]; clen = sl; idx = j - off; }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        int64_t n = row0 + r;
+        if (n >= N) break;
+        int64_t b = n / a.S, s = n - b * a.S;
+        int64_t t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+        unsigned v = 0;
+        if (mode == 1)      v = stream_byte(&cds[r][c0], clen, bw, idx);
+        else if (mode == 2) v = cds[r][c0];
+        a.packed[b * a.p_sb + h * a.p_sh + t * a.p_st + j] = (uint8_t)v;
+    }
+}
+
+template <bool IS_V>
+int launch_encode(const EncodeArgs& a, hipStream_t st) {
+    int64_t N = (int64_t)a.B * a.S;
+    if (N == 0 || a.n_kv == 0) return BGTQ_OK;
+    // Few rows (decode append): small tiles so every row gets its own work-group
+    // and the step stays latency-bound; many rows (prefill): 16-row tiles so the
+    // rotation matrix is amortised.
+    if (N <= 64) {
+        dim3 grid((unsigned)((N + 1) / 2), (unsigned)a.n_kv);
+        hipLaunchKernelGGL((encode_kernel<2, IS_V>), grid, dim3(NT), 0, st, a);
+    } else {
+        dim3 grid((unsigned)((N + 15) / 16), (unsigned)a.n_kv);
+        hipLaunchKernelGGL((encode_kernel<16, IS_V>), grid, dim3(NT), 0, st, a);
+    }
+    return bgtq_launch_status();
+}
+
+// ---- query permute + rotate ---------------------------------------------------
+__global__ __launch_bounds__(NT) void rotate_q_kernel(
+    const bgtq_head_plan* plans, const uint16_t* q, int64_t q_sr, int64_t q_sh,
+    uint16_t* q_rot, int64_t qr_sr, int64_t qr_sh, int gqa) {
+    __shared__ float xs[D];
+    const int j = threadIdx.x;
+    const int hq = blockIdx.y;
+    const int64_t row = blockIdx.x;
+    const bgtq_head_plan& P = plans[hq / gqa];
+    xs[j] = bgtq_h2f(q[row * q_sr + hq * q_sh + P.head_perm[j]]);
+    __syncthreads();
+    const int g = P.group_of[j];
+    float acc = 0.f;
+    if (g >= 0) {
+        if (P.seg_identity[g]) {
+            acc = xs[j];
+        } else {
+            int s = P.seg_start[g], e = s + P.seg_len[g];
+            for (int k = s; k < e; k++) acc = __builtin_fmaf(xs[k], P.k_rot_T[k * D + j], acc);
+        }
+    }
+    q_rot[row * qr_sr + hq * qr_sh + j] = bgtq_f2h(acc);
+}
+
+}  // namespace
+
+extern "C" {
+
+int bgtq_encode_k(const bgtq_head_plan* plans,
+                  const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                  int B, int n_kv, int S,
+                  void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                  void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
+                  const int32_t* t_pos, int t_pos_scalar,
+                  int k_layout, int quant_mode, void* stream) {
+    BGTQ_CHECK_ARG(plans && k && k_packed && k_norms);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
+    BGTQ_CHECK_ARG(k_row_width >= 0 && k_row_width <= NT);
+    BGTQ_CHECK_ARG(norm_width >= 0 && norm_width <= BGTQ_MAX_SEGMENTS);
+    BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
+    BGTQ_CHECK_ARG(quant_mode == BGTQ_QUANT_LUT256 || quant_mode == BGTQ_QUANT_EXACT);
+    BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
+    EncodeArgs a{};
+    a.plans = plans; a.x = (const uint16_t*)k; a.x_sb = k_sb; a.x_sh = k_sh; a.x_ss = k_ss;
+    a.B = B; a.n_kv = n_kv; a.S = S;
+    a.packed = (uint8_t*)k_packed; a.p_sb = kp_sb; a.p_sh = kp_sh; a.p_st = kp_st;
+    a.row_width = k_row_width;
+    a.norms = (uint16_t*)k_norms; a.n_sb = kn_sb; a.n_sh = kn_sh; a.n_st = kn_st;
+    a.norm_width = norm_width;
+    a.t_pos = t_pos; a.t_pos_scalar = t_pos_scalar;
+    a.layout = k_layout; a.quant_mode = quant_mode;
+    return launch_encode<false>(a, (hipStream_t)stream);
+}
+
+int bgtq_encode_v(const bgtq_head_plan* plans,
+                  const void* v, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                  int B, int n_kv, int S,
+                  void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                  void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                  const int32_t* t_pos, int t_pos_scalar,
+                  int v_layout, void* stream) {
+    BGTQ_CHECK_ARG(plans && v && v_packed && v_norms);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
+    BGTQ_CHECK_ARG(v_row_width >= 0 && v_row_width <= NT);
+    BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
+    BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
+    EncodeArgs a{};
+    a.plans = plans; a.x = (const uint16_t*)v; a.x_sb = v_sb; a.x_sh = v_sh; a.x_ss = v_ss;
+    a.B = B; a.n_kv = n_kv; a.S = S;
+    a.packed = (uint8_t*)v_packed; a.p_sb = vp_sb; a.p_sh = vp_sh; a.p_st = vp_st;
+    a.row_width = v_row_width;
+    a.norms = (uint16_t*)v_norms; a.n_sb = vn_sb; a.n_sh = vn_sh; a.n_st = vn_st;
+    a.norm_width = 1;
+    a.t_pos = t_pos; a.t_pos_scalar = t_pos_scalar;
+    a.layout = v_layout;
+    return launch_encode<true>(a, (hipStream_t)stream);
+}
+
+int bgtq_compress_k_codes(const bgtq_head_plan* plan, const void* k, int64_t N,
+                          void* codes, float* norms, int norm_width,
+                          int corrected, int quant_mode, void* stream) {
+    BGTQ_CHECK_ARG(plan && k && codes && norms);
+    BGTQ_CHECK_ARG(N >= 0 && N < (int64_t)1 << 31);
+    BGTQ_CHECK_ARG(norm_width >= 1 && norm_width <= BGTQ_MAX_SEGMENTS);
+    BGTQ_CHECK_ARG(quant_mode == BGTQ_QUANT_LUT256 || quant_mode == BGTQ_QUANT_EXACT);
+    EncodeArgs a{};
+    a.plans = plan; a.x = (const uint16_t*)k; a.x_sb = 0; a.x_sh = 0; a.x_ss = D;
+    a.B = 1; a.n_kv = 1; a.S = (int)N;
+    a.codes_out = (uint8_t*)codes; a.norms_f32_out = norms; a.norm_width = norm_width;
+    a.corrected = corrected; a.layout = BGTQ_K_BITPACKED; a.quant_mode = quant_mode;
+    return launch_encode<false>(a, (hipStream_t)stream);
+}
+
+int bgtq_compress_v_codes(const bgtq_head_plan* plan, const void* v, int64_t N,
+                          void* codes, void* norms_f16, void* stream) {
+    BGTQ_CHECK_ARG(plan && v && codes && norms_f16);
+    BGTQ_CHECK_ARG(N >= 0 && N < (int64_t)1 << 31);
+    EncodeArgs a{};
+    a.plans = plan; a.x = (const uint16_t*)v; a.x_sb = 0; a.x_sh = 0; a.x_ss = D;
+    a.B = 1; a.n_kv = 1; a.S = (int)N;
+    a.codes_out = (uint8_t*)codes; a.norms = (uint16_t*)norms_f16; a.norm_width = 1;
+    return launch_encode<true>(a, (hipStream_t)stream);
+}
+
+int bgtq_rotate_q(const bgtq_head_plan* plans,
+                  const void* q, int64_t q_sr, int64_t q_sh,
+                  void* q_rot, int64_t qr_sr, int64_t qr_sh,
+                  int n_rows, int n_kv, int gqa, void* stream) {
+    BGTQ_CHECK_ARG(plans && q && q_rot);
+    BGTQ_CHECK_ARG(n_rows >= 0 && n_kv >= 0 && gqa >= 1);
+    if (n_rows == 0 || n_kv == 0) return BGTQ_OK;
+    dim3 grid((unsigned)n_rows, (unsigned)(n_kv * gqa));
+    hipLaunchKernelGGL(rotate_q_kernel, grid, dim3(NT), 0, (hipStream_t)stream,
+                       plans, (const uint16_t*)q, q_sr, q_sh,
+                       (uint16_t*)q_rot, qr_sr, qr_sh, gqa);
+    return bgtq_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+"""Host mirror of ``bgtq_head_plan`` (include/bgtq.h) and its builder.
+
+One plan per (layer, KV head) gathers every static table the device kernels
+read: the K segment table, permutation, 256-bin code LUT, codebooks in fp32
+and fp16, the block-diagonal K rotation, and the V rotation/boundaries/LUT.
+Plans of the KV heads of one layer are concatenated and uploaded once.
+"""
+import numpy as np
+import torch
+
+HEAD_DIM = 128
+MAX_SEGMENTS = 8
+MAX_CENTROIDS = 256
+LUT_BINS = 256
+
+K_BITPACKED, K_MIXED = 0, 1
+V_BITPACKED, V_NIBBLE = 0, 1
+QUANT_LUT256, QUANT_EXACT = 0, 1
+
+_S, _D, _C = MAX_SEGMENTS, HEAD_DIM, MAX_CENTROIDS
+
+PLAN_DTYPE = np.dtype([
+    ('n_seg', '<i4'), ('n_zero_dims', '<i4'), ('k_row_bytes', '<i4'),
+    ('k_mixed_bytes', '<i4'), ('nopack_start', '<i4'), ('nopack_len', '<i4'),
+    ('v_bits', '<i4'), ('reserved0', '<i4'),
+    ('seg_bw', '<i4', (_S,)), ('seg_start', '<i4', (_S,)), ('seg_len', '<i4', (_S,)),
+    ('seg_pack_off', '<i4', (_S,)), ('seg_mixed_off', '<i4', (_S,)),
+    ('seg_identity', '<i4', (_S,)),
+    ('head_perm', '<i4', (_D,)), ('group_of', '<i4', (_D,)),
+    ('lut_offset', '<f4', (_D,)), ('lut_inv_scale', '<f4', (_D,)),
+    ('code_lut', 'u1', (_S, LUT_BINS)),
+    ('k_centroids', '<f4', (_S, _C)), ('k_boundaries', '<f4', (_S, _C)),
+    ('k_codebook_f16', '<u2', (_S, _C)),
+    ('k_rot_T', '<f4', (_D * _D,)),
+    ('v_centroids', '<f4', (16,)), ('v_boundaries', '<f4', (16,)),
+    ('v_lut_f16', '<u2', (16,)),
+    ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
+], align=True)
+
+
+def segment_bytes(bw: int, length: int) -> int:
+    """Bytes a K segment of ``length`` codes takes in the bit-packed record."""
+    if bw == 1:
+        return (length + 7) // 8
+    if bw == 2:
+        return (length + 3) // 4
+    if bw == 3:
+        return ((length + 7) // 8) * 3
+    if bw == 4:
+        return (length + 1) // 2
+    return length
+
+
+def build_head_plan(quantizer) -> np.ndarray:
+    """Fill one ``bgtq_head_plan`` from a calibrated ``BlockGTQQuantizer``
+    whose V quantizer has been initialised."""
+    q = quantizer
+    hd = q.head_dim
+    if hd != HEAD_DIM:
+        raise ValueError(f"kernels are built for head_dim {HEAD_DIM}, got {hd}")
+    pm = q._pack_meta
+    widths = [bw for bw in range(1, 9) if bw in pm]
+    if len(widths) > MAX_SEGMENTS:
+        raise ValueError("more than 8 distinct bit widths")
+    p = np.zeros((), dtype=PLAN_DTYPE)
+    p['n_seg'] = len(widths)
+    p['n_zero_dims'] = q._n_zero_dims
+    p['k_row_bytes'] = pm['total_packed_bytes']
+    p['nopack_start'] = pm['nopack_start']
+    p['nopack_len'] = pm['nopack_len']
+    nib_bytes = (pm['nopack_start'] - q._n_zero_dims) // 2
+    p['k_mixed_bytes'] = nib_bytes + pm['nopack_len']
+    p['v_bits'] = q._v_bits
+    p['k_boundaries'][...] = np.inf
+    p['v_boundaries'][...] = np.inf
+
+    cents = q._pos_centroids.detach().cpu().numpy()
+    bounds = q._pos_boundaries.detach().cpu().numpy()
+    code_lut = q._code_lut.detach().cpu().numpy()
+    pos_to_cb = q._pos_to_cb.detach().cpu().numpy()
+    group_of = (q._group_of_full.detach().cpu().numpy())
+    rot_T = q._block_rot_T.detach().cpu().numpy().astype(np.float32)
+    for g, bw in enumerate(widths):
+        s, ln = pm[bw]['start'], pm[bw]['length']
+        nc = 1 << bw
+        p['seg_bw'][g] = bw
+        p['seg_start'][g] = s
+        p['seg_len'][g] = ln
+        p['seg_pack_off'][g] = pm[bw]['pack_offset']
+        p['seg_mixed_off'][g] = ((s - q._n_zero_dims) // 2 if bw <= 4
+                                 else nib_bytes + (s - pm['nopack_start']))
+        blk = rot_T[s:s + ln, s:s + ln]
+        p['seg_identity'][g] = int(np.array_equal(blk, np.eye(ln, dtype=np.float32)))
+        if not (group_of[s:s + ln] == g).all():
+            raise ValueError("segments and norm groups disagree")
+        cb = int(pos_to_cb[s])
+        if not (pos_to_cb[s:s + ln] == cb).all():
+            raise ValueError("a segment uses more than one codebook")
+        p['code_lut'][g] = code_lut[cb]
+        p['k_centroids'][g, :nc] = cents[s, :nc]
+        p['k_boundaries'][g, :nc - 1] = bounds[s, :nc - 1]
+        p['k_codebook_f16'][g, :nc] = cents[s, :nc].astype(np.float16).view(np.uint16)
+    p['head_perm'] = q._head_perm.detach().cpu().numpy().astype(np.int32)
+    p['group_of'] = group_of.astype(np.int32)
+    p['lut_offset'] = q._lut_offsets.detach().cpu().numpy()
+    p['lut_inv_scale'] = q._lut_inv_scales.detach().cpu().numpy()
+    p['k_rot_T'] = rot_T.reshape(-1)
+
+    nv = 1 << q._v_bits
+    vc = q._v_centroids_f32.detach().cpu().numpy()
+    p['v_centroids'][:nv] = vc
+    p['v_boundaries'][:nv - 1] = q._v_boundaries.detach().cpu().numpy()
+    p['v_lut_f16'][:nv] = vc.astype(np.float16).view(np.uint16)
+    p['v_rot_T'] = q._v_rot_T.detach().cpu().numpy().astype(np.float32).reshape(-1)
+    p['v_rot'] = q._v_rot.detach().cpu().numpy().astype(np.float32).reshape(-1)
+    return p.reshape(1)
+
+
+def stack_plans(quantizers) -> np.ndarray:
+    """Plans of all KV heads of one layer as one (n_kv,) structured array."""
+    return np.concatenate([build_head_plan(q) for q in quantizers])
+
+
+def upload_plans(plans: np.ndarray, device) -> torch.Tensor:
+    """Copy a structured plan array to ``device`` as a flat uint8 tensor."""
+    raw = torch.from_numpy(np.ascontiguousarray(plans).view(np.uint8).copy())
+    return raw.to(device)

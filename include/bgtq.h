@@ -1,0 +1,243 @@
+/*
+ * bgtq.h - C ABI of the MI355X packed-KV decode path of Block-GTQ.
+ *
+ * One shared library (libbgtq.so, built from blockgtq_amd/csrc for gfx950)
+ * exports the entry points below.  Every pointer is a plain device pointer
+ * unless stated otherwise, every stride is in ELEMENTS of the pointed-to type,
+ * `stream` is a hipStream_t passed as void*, and every function returns 0 on
+ * success or a negative BGTQ_E* code / positive hipError_t.  Nothing in here
+ * allocates or frees device memory and nothing throws.
+ *
+ * The reference has no FFI: its device code is Triton launched from Python.
+ * Each entry point therefore cites the Python/Triton function whose launch it
+ * replaces (paths relative to the reference checkout).
+ */
+#ifndef BGTQ_H
+#define BGTQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BGTQ_HEAD_DIM      128   /* the only head width the kernels are built for */
+#define BGTQ_MAX_SEGMENTS  8     /* distinct K bit widths per head */
+#define BGTQ_MAX_CENTROIDS 256   /* 8-bit codebook */
+#define BGTQ_LUT_BINS      256
+#define BGTQ_MAX_GQA       16    /* query heads per KV head */
+#define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
+
+/* error codes (negative); positive return values are hipError_t */
+#define BGTQ_OK            0
+#define BGTQ_EINVAL       -1     /* bad argument (null pointer, shape, stride, flag) */
+#define BGTQ_EUNSUPPORTED -2     /* legal in the reference but not built here */
+#define BGTQ_ELIMIT       -3     /* size beyond a documented maximum */
+
+/* K record layouts (blockgtq/quantizer.py:34-102 and :1930-1951) */
+#define BGTQ_K_BITPACKED   0     /* [1b|2b|3b|4b segments bit-packed|5..8b raw], raw group norms */
+#define BGTQ_K_MIXED       1     /* [bw<=4 dims as nibbles | bw>=5 raw], corrected norms */
+/* V record layouts (blockgtq/v_packing.py:17-28, blockgtq/quantizer.py:2096-2099) */
+#define BGTQ_V_BITPACKED   0     /* v_bits per code, LSB first */
+#define BGTQ_V_NIBBLE      1     /* 4 bits per code whatever v_bits is */
+/* K scalar quantisation rule */
+#define BGTQ_QUANT_LUT256  0     /* 256-bin table, blockgtq/quantizer.py:841-850 */
+#define BGTQ_QUANT_EXACT   1     /* count of boundaries below y, blockgtq/block_gtq_pipeline.py:337-341 */
+
+/*
+ * Static per-(layer, KV head) plan.  Built once on the host from the
+ * calibrated quantizer (blockgtq/quantizer.py:1024-1148 and :1478-1497) and
+ * uploaded as an array of n_kv structs per layer.  All dim indices are in
+ * "packed order": coordinates sorted by ascending bit width, the two
+ * coordinates of a RoPE block adjacent (blockgtq/block_gtq_pipeline.py:161-177).
+ */
+typedef struct bgtq_head_plan {
+    /* K segment table: one segment == one bit width == one norm group */
+    int32_t  n_seg;                             /* 0..BGTQ_MAX_SEGMENTS */
+    int32_t  n_zero_dims;                       /* leading dims that got 0 bits */
+    int32_t  k_row_bytes;                       /* BGTQ_K_BITPACKED record length */
+    int32_t  k_mixed_bytes;                     /* BGTQ_K_MIXED record length */
+    int32_t  nopack_start;                      /* first dim with bw >= 5, HEAD_DIM if none */
+    int32_t  nopack_len;
+    int32_t  v_bits;                            /* 1..4 */
+    int32_t  reserved0;
+    int32_t  seg_bw[BGTQ_MAX_SEGMENTS];
+    int32_t  seg_start[BGTQ_MAX_SEGMENTS];      /* first dim of the segment */
+    int32_t  seg_len[BGTQ_MAX_SEGMENTS];        /* dims in the segment (even) */
+    int32_t  seg_pack_off[BGTQ_MAX_SEGMENTS];   /* byte offset, BGTQ_K_BITPACKED */
+    int32_t  seg_mixed_off[BGTQ_MAX_SEGMENTS];  /* byte offset, BGTQ_K_MIXED */
+    int32_t  seg_identity[BGTQ_MAX_SEGMENTS];   /* 1: rotation block is the identity */
+    /* K encode tables */
+    int32_t  head_perm[BGTQ_HEAD_DIM];          /* packed dim -> original coordinate */
+    int32_t  group_of[BGTQ_HEAD_DIM];           /* packed dim -> segment, -1 for 0-bit dims */
+    float    lut_offset[BGTQ_HEAD_DIM];
+    float    lut_inv_scale[BGTQ_HEAD_DIM];
+    uint8_t  code_lut[BGTQ_MAX_SEGMENTS][BGTQ_LUT_BINS];
+    float    k_centroids[BGTQ_MAX_SEGMENTS][BGTQ_MAX_CENTROIDS];
+    float    k_boundaries[BGTQ_MAX_SEGMENTS][BGTQ_MAX_CENTROIDS]; /* 2^bw-1 valid, +inf after */
+    uint16_t k_codebook_f16[BGTQ_MAX_SEGMENTS][BGTQ_MAX_CENTROIDS];
+    float    k_rot_T[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];  /* y = xhat @ k_rot_T, block diagonal */
+    /* V tables */
+    float    v_centroids[16];
+    float    v_boundaries[16];                  /* 2^v_bits-1 valid, +inf after */
+    uint16_t v_lut_f16[16];
+    float    v_rot_T[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];  /* encode: y = vhat @ v_rot_T */
+    float    v_rot[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];    /* decode: out = acc @ v_rot */
+} bgtq_head_plan;
+
+/* sizeof(bgtq_head_plan) as the library was compiled; the host mirror checks it. */
+size_t bgtq_plan_sizeof(void);
+
+/* Library/ABI version, bumped whenever a signature or the plan struct changes. */
+int bgtq_abi_version(void);
+
+/* Human-readable text for a return code of this library (static storage). */
+const char* bgtq_strerror(int code);
+
+/*
+ * K encode + pack, all KV heads of one layer in one launch, written straight
+ * into the cache slots.
+ * Replaces _compress_pack_kernel_v8_batched (blockgtq/quantizer.py:713-990)
+ * as driven by compress_k_packed_batched (:2105-2172) for BGTQ_K_BITPACKED and
+ * by compress_k_mixed_batched (:1844-1976, nibble repack + norm correction)
+ * for BGTQ_K_MIXED, plus the slice-assign cache writes of
+ * blockgtq/packed_kv_manager.py:138-180 / blockgtq/production_cache.py:174-201.
+ *
+ *   plans      n_kv structs (device)
+ *   k          fp16 [B][n_kv][S][128], strides k_sb/k_sh/k_ss in halves, dim contiguous
+ *   k_packed   u8   [B][n_kv][T][row],  strides in bytes; record written at token
+ *              t_pos[b] + s (t_pos device int32[B]) or t_pos_scalar + s when t_pos is NULL;
+ *              bytes beyond the head's own record up to k_row_width are zeroed
+ *   k_norms    fp16 [B][n_kv][T][norm_width], strides in halves; entries beyond the
+ *              head's own n_seg up to norm_width are zeroed
+ */
+int bgtq_encode_k(const bgtq_head_plan* plans,
+                  const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                  int B, int n_kv, int S,
+                  void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                  void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
+                  const int32_t* t_pos, int t_pos_scalar,
+                  int k_layout, int quant_mode, void* stream);
+
+/*
+ * V encode + pack, all KV heads in one launch, written into the cache slots.
+ * Replaces _compress_v_pack_kernel_batched (blockgtq/quantizer.py:518-706) as
+ * driven by compress_v_packed_batched (:1980-2029) for BGTQ_V_BITPACKED and by
+ * compress_v_nibble4_batched (:2033-2101) for BGTQ_V_NIBBLE.
+ *   v_norms    fp16 [B][n_kv][T], corrected norm ||v|| / ||centroids[codes]||
+ */
+int bgtq_encode_v(const bgtq_head_plan* plans,
+                  const void* v, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                  int B, int n_kv, int S,
+                  void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                  void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                  const int32_t* t_pos, int t_pos_scalar,
+                  int v_layout, void* stream);
+
+/*
+ * Unpacked K codes + raw group norms (no packing), one head.
+ * Replaces _compress_only_kernel (blockgtq/kernels/quant_kernels.py:471-565)
+ * behind BlockGTQQuantizer.compress (blockgtq/quantizer.py:1246-1296).
+ *   k      fp16 [N][128] contiguous
+ *   codes  u8   [N][128] in packed order
+ *   norms  fp32 [N][norm_width] raw group norms (corrected when `corrected` != 0)
+ */
+int bgtq_compress_k_codes(const bgtq_head_plan* plan, const void* k, int64_t N,
+                          void* codes, float* norms, int norm_width,
+                          int corrected, int quant_mode, void* stream);
+
+/* Unpacked V codes + fp16 corrected norms, one head
+ * (PolarQuantGPU.quantize + _corrected_v_norms, blockgtq/quantizer.py:1510-1541). */
+int bgtq_compress_v_codes(const bgtq_head_plan* plan, const void* v, int64_t N,
+                          void* codes, void* norms_f16, void* stream);
+
+/*
+ * Query permute + rotate into the packed K space, all query heads of a layer.
+ * Replaces BlockGTQQuantizer.rotate_q_for_packed_kernel
+ * (blockgtq/quantizer.py:1160-1187), called once per KV head per step by
+ * blockgtq/production_cache.py:240-245.
+ *   q      fp16 [n_rows][n_q][128], strides q_sr/q_sh in halves
+ *   q_rot  fp16 [n_rows][n_q][128], strides likewise; n_q = n_kv * gqa
+ */
+int bgtq_rotate_q(const bgtq_head_plan* plans,
+                  const void* q, int64_t q_sr, int64_t q_sh,
+                  void* q_rot, int64_t qr_sr, int64_t qr_sh,
+                  int n_rows, int n_kv, int gqa, void* stream);
+
+/* Bytes of fp32 scratch bgtq_decode_attn needs for (B, n_q, n_splits). */
+size_t bgtq_workspace_bytes(int B, int n_q, int n_splits);
+
+/* Partition count bgtq_decode_attn would pick for n_splits <= 0. */
+int bgtq_default_splits(int B, int n_kv, int max_T);
+
+/*
+ * Fused unpack + dequant + split-T decode attention over the packed cache,
+ * every (batch row, KV head, partition) in one launch.
+ * Replaces _packed_decode_kernel (blockgtq/kernels/fused_packed_attention.py:153-894)
+ * which the reference launches once per KV head from
+ * fused_blockgtq_decode_attention (:1541-1843).
+ *
+ *   q_rot      fp16 [B][n_q][128] already permuted+rotated (bgtq_rotate_q)
+ *   k_packed / k_norms / v_packed / v_norms as written by the encoders;
+ *              k_row_width / v_row_width = record bytes per token the cache holds
+ *              (the widest head's record), strides may be larger
+ *   seq_lens   device int32[B] tokens visible per batch row, or NULL -> T for all
+ *   n_splits   partitions per (b, kv head); partition c covers
+ *              [c*chunk, min((c+1)*chunk, T_b)), chunk = ceil(T_b / n_splits)
+ *   partial_out fp32 [B][n_q][n_splits][128]  (normalised, V still rotated)
+ *   partial_lse fp32 [B][n_q][n_splits]       (natural log; -inf for an empty partition)
+ */
+int bgtq_decode_attn(const bgtq_head_plan* plans,
+                     const void* q_rot, int64_t q_sb, int64_t q_sh,
+                     const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                     const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                     const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                     const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                     const int32_t* seq_lens, int T,
+                     int B, int n_kv, int gqa, int n_splits,
+                     float* partial_out, float* partial_lse,
+                     int k_layout, int v_layout, float scale, void* stream);
+
+/*
+ * Log-sum-exp merge of the partitions, optional extra partials (an fp16
+ * sink/recent-window attention computed elsewhere), V un-rotation applied once
+ * to the merged vector, fp16 store.
+ * Replaces _split_t_merge_kernel (blockgtq/kernels/fused_packed_attention.py:60-103),
+ * the per-partition `partial_out @ R` of :875-882 and the return_lse
+ * logsumexp of :1856-1860.  Partitions whose lse is -inf are skipped.
+ *
+ *   extra_out  fp32 [B][n_q][n_extra][128] or NULL (same rotated-V space)
+ *   extra_lse  fp32 [B][n_q][n_extra] or NULL
+ *   unrotate   != 0: multiply the merged vector by plans[h].v_rot
+ *   out        fp16 [B][n_q][128], strides o_sb/o_sh in halves
+ *   lse_out    fp32 [B][n_q] total log-sum-exp, or NULL
+ */
+int bgtq_lse_reduce(const bgtq_head_plan* plans,
+                    const float* partial_out, const float* partial_lse, int n_splits,
+                    const float* extra_out, const float* extra_lse, int n_extra,
+                    int B, int n_kv, int gqa, int unrotate,
+                    void* out, int64_t o_sb, int64_t o_sh,
+                    float* lse_out, void* stream);
+
+/*
+ * Dense fp16 attention partial for the with-buffer setting (sink tokens and a
+ * recent window kept in fp16 next to the packed cache).  K is stored already
+ * permuted+rotated into the packed space of its head and V rotated by v_rot_T,
+ * so the partial lives in the same space as bgtq_decode_attn's and feeds
+ * bgtq_lse_reduce as `extra`.  The reference has this three-region cache only
+ * in its unaccelerated path (blockgtq/unaccelerated.py:163-244).
+ *   kbuf, vbuf fp16 [B][n_kv][W][128]; lens device int32[B] valid rows (<= W) or NULL -> W
+ *   part_out   fp32 [B][n_q][128], part_lse fp32 [B][n_q]
+ */
+int bgtq_window_attn(const void* q_rot, int64_t q_sb, int64_t q_sh,
+                     const void* kbuf, const void* vbuf,
+                     int64_t w_sb, int64_t w_sh, int64_t w_st,
+                     const int32_t* lens, int W,
+                     int B, int n_kv, int gqa, float scale,
+                     float* part_out, float* part_lse, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BGTQ_H */
