@@ -1,0 +1,115 @@
+"""Torch-facing wrappers of the decode entry points of the C ABI.
+
+These take cache-shaped tensors (batch, KV head, token, ...) and launch one
+kernel for every (batch row, KV head, partition) plus one merge kernel; the
+per-KV-head Python loop of the reference (blockgtq/production_cache.py:234-262)
+has no counterpart here.
+"""
+import math
+from typing import Optional
+
+import torch
+
+from . import _capi, plan as _plan
+
+
+class Workspace:
+    """Reusable fp32 partial buffers for (B, n_q, n_splits) so a decode step
+    allocates nothing after the first call."""
+
+    def __init__(self):
+        self._buf = None
+
+    def get(self, B, n_q, n_splits, device):
+        need = B * n_q * n_splits * (_plan.HEAD_DIM + 1)
+        if self._buf is None or self._buf.numel() < need or self._buf.device != torch.device(device):
+            self._buf = torch.empty(need, dtype=torch.float32, device=device)
+        out = self._buf[:B * n_q * n_splits * _plan.HEAD_DIM]
+        lse = self._buf[B * n_q * n_splits * _plan.HEAD_DIM:need]
+        return out, lse
+
+
+_default_ws = Workspace()
+
+
+def default_splits(B: int, n_kv: int, T: int) -> int:
+    return _capi.lib().bgtq_default_splits(int(B), int(n_kv), int(T))
+
+
+@torch.no_grad()
+def rotate_q(plans: torch.Tensor, q: torch.Tensor, n_kv: int) -> torch.Tensor:
+    """q (B, n_q, D) fp16 -> permuted + rotated into each KV head's packed space."""
+    _capi.require_cuda(q, "q")
+    assert q.dim() == 3 and q.dtype == torch.float16 and q.stride(-1) == 1
+    B, n_q, _ = q.shape
+    out = torch.empty((B, n_q, _plan.HEAD_DIM), dtype=torch.float16, device=q.device)
+    _capi.check(_capi.lib().bgtq_rotate_q(
+        _capi.ptr(plans), _capi.ptr(q), q.stride(0), q.stride(1),
+        _capi.ptr(out), out.stride(0), out.stride(1),
+        B, n_kv, n_q // n_kv, _capi.stream_ptr(q.device)), "bgtq_rotate_q")
+    return out
+
+
+@torch.no_grad()
+def decode_attention(plans: torch.Tensor, q_rot: torch.Tensor,
+                     k_packed: torch.Tensor, k_norms: torch.Tensor,
+                     v_packed: torch.Tensor, v_norms: torch.Tensor,
+                     T: int, *, seq_lens: Optional[torch.Tensor] = None,
+                     n_splits: int = 0, k_layout: int = _plan.K_BITPACKED,
+                     v_layout: int = _plan.V_BITPACKED, scale: Optional[float] = None,
+                     k_row_width: Optional[int] = None, v_row_width: Optional[int] = None,
+                     unrotate: bool = True, return_lse: bool = False,
+                     extra_out: Optional[torch.Tensor] = None,
+                     extra_lse: Optional[torch.Tensor] = None,
+                     workspace: Optional[Workspace] = None):
+    """Decode attention of one layer over the packed cache.
+
+    q_rot (B, n_q, D) fp16 rotated queries; k_packed (B, n_kv, >=T, Kb) uint8;
+    k_norms (B, n_kv, >=T, G) fp16; v_packed (B, n_kv, >=T, Vb) uint8; v_norms
+    (B, n_kv, >=T) fp16.  ``T`` tokens are visible for every batch row unless
+    ``seq_lens`` (int32 device tensor, B) gives per-row counts (then ``T`` must
+    be their maximum).  Returns (B, n_q, D) fp16 [and the total lse (B, n_q)].
+    """
+    _capi.require_cuda(q_rot, "q_rot")
+    assert q_rot.dim() == 3 and q_rot.dtype == torch.float16 and q_rot.stride(-1) == 1
+    assert k_packed.dtype == torch.uint8 and k_packed.stride(-1) == 1
+    assert v_packed.dtype == torch.uint8 and v_packed.stride(-1) == 1
+    assert k_norms.dtype == torch.float16 and k_norms.stride(-1) == 1
+    assert v_norms.dtype == torch.float16
+    B, n_q, D = q_rot.shape
+    n_kv = k_packed.shape[1]
+    gqa = n_q // n_kv
+    assert k_packed.shape[2] >= T and v_packed.shape[2] >= T
+    if seq_lens is not None:
+        assert seq_lens.dtype == torch.int32 and seq_lens.is_cuda and seq_lens.numel() == B
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    k_row_width = k_packed.shape[-1] if k_row_width is None else k_row_width
+    v_row_width = v_packed.shape[-1] if v_row_width is None else v_row_width
+    L = _capi.lib()
+    if n_splits <= 0:
+        n_splits = L.bgtq_default_splits(B, n_kv, max(T, 1))
+    ws = workspace or _default_ws
+    part_out, part_lse = ws.get(B, n_q, n_splits, q_rot.device)
+    st = _capi.stream_ptr(q_rot.device)
+    _capi.check(L.bgtq_decode_attn(
+        _capi.ptr(plans), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1),
+        _capi.ptr(k_packed), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2), k_row_width,
+        _capi.ptr(k_norms), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2),
+        _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), v_row_width,
+        _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
+        _capi.ptr(seq_lens), int(T), B, n_kv, gqa, n_splits,
+        _capi.ptr(part_out), _capi.ptr(part_lse), k_layout, v_layout, scale, st),
+        "bgtq_decode_attn")
+    out = torch.empty((B, n_q, D), dtype=torch.float16, device=q_rot.device)
+    lse = torch.empty((B, n_q), dtype=torch.float32, device=q_rot.device) if return_lse else None
+    n_extra = 0
+    if extra_out is not None:
+        assert extra_out.dtype == torch.float32 and extra_lse.dtype == torch.float32
+        assert extra_out.is_contiguous() and extra_lse.is_contiguous()
+        n_extra = extra_lse.shape[-1] if extra_lse.dim() == 3 else 1
+    _capi.check(L.bgtq_lse_reduce(
+        _capi.ptr(plans), _capi.ptr(part_out), _capi.ptr(part_lse), n_splits,
+        _capi.ptr(extra_out), _capi.ptr(extra_lse), n_extra,
+        B, n_kv, gqa, int(unrotate), _capi.ptr(out), out.stride(0), out.stride(1),
+        _capi.ptr(lse), st), "bgtq_lse_reduce")
+    return (out, lse) if return_lse else out

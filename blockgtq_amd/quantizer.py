@@ -183,14 +183,15 @@ class BlockGTQQuantizer:
             segments.append((bw, s, ln, pm[bw]['pack_offset'], lut_off, si))
             lut_off += 1 << bw
         flat = torch.cat(parts) if parts else torch.zeros(0, dtype=torch.float16)
-        return {
+        from .kernels import register_kernel_args
+        return register_kernel_args({
             'codebook_flat': flat.to(dev),
             'lut_offset': lut_offset.to(dev),
             'norm_group': norm_group.to(dev),
             'segments_b': segments,
             'total_packed_bytes': pm['total_packed_bytes'],
             'quantizer': self,
-        }
+        })
 
     # -------------------------------------------------------------- plan
     def plan(self):
