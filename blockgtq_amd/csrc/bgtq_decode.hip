@@ -323,6 +323,56 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     if (lse_out && j == 0) lse_out[row] = m + __logf(den);
 }
 
+
+// ---- dense fp16 partial over the sink + recent-window tokens ------------------
+constexpr int WT = 256;
+__global__ __launch_bounds__(WT) void window_attn_kernel(
+    const uint16_t* q, int64_t q_sb, int64_t q_sh,
+    const uint16_t* kbuf, const uint16_t* vbuf, int64_t w_sb, int64_t w_sh, int64_t w_st,
+    const int32_t* lens, int W, int n_q, int gqa, float scale, float* part_out, float* part_lse) {
+    extern __shared__ float wlog[];            // [W] logits, then weights
+    __shared__ float q_s[D];
+    __shared__ float red[WT / 64];
+    const int tid = threadIdx.x;
+    const int hq = blockIdx.x, b = blockIdx.y, h = hq / gqa;
+    const int n = lens ? min(lens[b], W) : W;
+    const size_t row = (size_t)b * n_q + hq;
+    if (tid < D) q_s[tid] = bgtq_h2f(q[b * q_sb + hq * q_sh + tid]);
+    __syncthreads();
+    const uint16_t* kb = kbuf + b * w_sb + h * w_sh;
+    const uint16_t* vb = vbuf + b * w_sb + h * w_sh;
+    float m = -INFINITY;
+    for (int t = tid; t < n; t += WT) {
+        const uint16_t* kr = kb + (int64_t)t * w_st;
+        float acc = 0.f;
+        for (int d = 0; d < D; d++) acc += q_s[d] * bgtq_h2f(kr[d]);
+        acc *= scale;
+        wlog[t] = acc;
+        m = fmaxf(m, acc);
+    }
+    m = wave_max(m);
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float l = 0.f;
+    for (int t = tid; t < n; t += WT) {
+        float p = __expf(wlog[t] - m);
+        wlog[t] = p;
+        l += p;
+    }
+    l = wave_sum(l);
+    if ((tid & 63) == 0) red[tid >> 6] = l;
+    __syncthreads();
+    l = red[0] + red[1] + red[2] + red[3];
+    if (tid < D) {
+        float acc = 0.f;
+        for (int t = 0; t < n; t++) acc += wlog[t] * bgtq_h2f(vb[(int64_t)t * w_st + tid]);
+        part_out[row * D + tid] = n > 0 ? acc / l : 0.f;
+    }
+    if (tid == 0) part_lse[row] = n > 0 ? m + __logf(l) : -INFINITY;
+}
+
 }  // namespace
 
 extern "C" {
@@ -398,6 +448,24 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
                        plans, partial_out, partial_lse, n_splits,
                        n_extra ? extra_out : nullptr, n_extra ? extra_lse : nullptr, n_extra,
                        n_kv * gqa, gqa, unrotate, (uint16_t*)out, o_sb, o_sh, lse_out);
+    return bgtq_launch_status();
+}
+
+int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
+                     const void* kbuf, const void* vbuf,
+                     int64_t w_sb, int64_t w_sh, int64_t w_st,
+                     const int32_t* lens, int W,
+                     int B, int n_kv, int gqa, float scale,
+                     float* part_out, float* part_lse, void* stream) {
+    BGTQ_CHECK_ARG(q && kbuf && vbuf && part_out && part_lse);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && gqa >= 1 && W >= 0);
+    if (W > 8192) return BGTQ_ELIMIT;
+    if (B == 0 || n_kv == 0) return BGTQ_OK;
+    dim3 grid((unsigned)(n_kv * gqa), (unsigned)B);
+    hipLaunchKernelGGL(window_attn_kernel, grid, dim3(WT), (size_t)(W > 0 ? W : 1) * sizeof(float),
+                       (hipStream_t)stream, (const uint16_t*)q, q_sb, q_sh,
+                       (const uint16_t*)kbuf, (const uint16_t*)vbuf, w_sb, w_sh, w_st,
+                       lens, W, n_kv * gqa, gqa, scale, part_out, part_lse);
     return bgtq_launch_status();
 }
 

@@ -302,8 +302,9 @@ int bgtq_encode_k(const bgtq_head_plan* plans,
                   void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
                   const int32_t* t_pos, int t_pos_scalar,
                   int k_layout, int quant_mode, void* stream) {
-    BGTQ_CHECK_ARG(plans && k && k_packed && k_norms);
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
+    if (B == 0 || n_kv == 0 || S == 0) return BGTQ_OK;     // nothing to encode
+    BGTQ_CHECK_ARG(plans && k && k_packed && k_norms);
     BGTQ_CHECK_ARG(k_row_width >= 0 && k_row_width <= NT);
     BGTQ_CHECK_ARG(norm_width >= 0 && norm_width <= BGTQ_MAX_SEGMENTS);
     BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
@@ -328,8 +329,9 @@ int bgtq_encode_v(const bgtq_head_plan* plans,
                   void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
                   const int32_t* t_pos, int t_pos_scalar,
                   int v_layout, void* stream) {
-    BGTQ_CHECK_ARG(plans && v && v_packed && v_norms);
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
+    if (B == 0 || n_kv == 0 || S == 0) return BGTQ_OK;
+    BGTQ_CHECK_ARG(plans && v && v_packed && v_norms);
     BGTQ_CHECK_ARG(v_row_width >= 0 && v_row_width <= NT);
     BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
     BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);

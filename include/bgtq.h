@@ -207,7 +207,8 @@ int bgtq_decode_attn(const bgtq_head_plan* plans,
  * the per-partition `partial_out @ R` of :875-882 and the return_lse
  * logsumexp of :1856-1860.  Partitions whose lse is -inf are skipped.
  *
- *   extra_out  fp32 [B][n_q][n_extra][128] or NULL (same rotated-V space)
+ *   extra_out  fp32 [B][n_q][n_extra][128] or NULL, in the ORIGINAL value space:
+ *              added after the packed sum has been un-rotated (needs unrotate != 0)
  *   extra_lse  fp32 [B][n_q][n_extra] or NULL
  *   unrotate   != 0: multiply the merged vector by plans[h].v_rot
  *   out        fp16 [B][n_q][128], strides o_sb/o_sh in halves
@@ -221,16 +222,19 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
                     float* lse_out, void* stream);
 
 /*
- * Dense fp16 attention partial for the with-buffer setting (sink tokens and a
- * recent window kept in fp16 next to the packed cache).  K is stored already
- * permuted+rotated into the packed space of its head and V rotated by v_rot_T,
- * so the partial lives in the same space as bgtq_decode_attn's and feeds
- * bgtq_lse_reduce as `extra`.  The reference has this three-region cache only
- * in its unaccelerated path (blockgtq/unaccelerated.py:163-244).
- *   kbuf, vbuf fp16 [B][n_kv][W][128]; lens device int32[B] valid rows (<= W) or NULL -> W
- *   part_out   fp32 [B][n_q][128], part_lse fp32 [B][n_q]
+ * Dense fp16 attention partial for the with-buffer setting: sink tokens and a
+ * recent window are kept as plain fp16 K/V (post-RoPE, unrotated) next to the
+ * packed cache.  The partial lives in the ORIGINAL value space and feeds
+ * bgtq_lse_reduce as `extra`, which adds it after un-rotating the packed sum.
+ * Takes the ORIGINAL queries (not bgtq_rotate_q's output).  The reference has
+ * this three-region cache only in its unaccelerated path
+ * (blockgtq/unaccelerated.py:163-244).
+ *   q          fp16 [B][n_q][128], strides q_sb/q_sh in halves
+ *   kbuf, vbuf fp16 [B][n_kv][W][128], common strides w_sb/w_sh/w_st in halves
+ *   lens       device int32[B] valid rows (<= W) or NULL -> W; W <= 8192
+ *   part_out   fp32 [B][n_q][128], part_lse fp32 [B][n_q] (-inf when no row is valid)
  */
-int bgtq_window_attn(const void* q_rot, int64_t q_sb, int64_t q_sh,
+int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
                      const void* kbuf, const void* vbuf,
                      int64_t w_sb, int64_t w_sh, int64_t w_st,
                      const int32_t* lens, int W,

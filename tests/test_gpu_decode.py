@@ -1,0 +1,259 @@
+"""GPU parity: fused packed decode attention + partition merge against the CPU
+checker, within 2e-3 max-abs (fp32 accumulate, fp16 output), through the C ABI
+and through the cache classes."""
+import numpy as np
+import pytest
+import torch
+
+from blockgtq_amd import ops, plan as P
+from blockgtq_amd import workloads as wl
+from helpers import make_kv, make_quantizer
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 2e-3
+
+
+def _reference(orc, mgr_plans, quantizers, kp, kn, vp, vn, q_rot, lens, gqa, k_layout=0, v_layout=0, v_bits=3):
+    B, H = kp.shape[:2]
+    out = np.zeros((B, H * gqa, 128), np.float32)
+    lse = np.zeros((B, H * gqa), np.float32)
+    for b in range(B):
+        for h in range(H):
+            pl = mgr_plans[h:h + 1]
+            own = int(pl['k_mixed_bytes'][0] if k_layout else pl['k_row_bytes'][0])
+            ng = max(int(pl['n_seg'][0]), 1)
+            T = lens[b]
+            o, l = orc.decode_attn(pl, q_rot[b, h * gqa:(h + 1) * gqa], kp[b, h, :T, :max(own, 1)],
+                                   kn[b, h, :T, :ng], vp[b, h, :T], vn[b, h, :T],
+                                   k_layout=k_layout, v_layout=v_layout)
+            out[b, h * gqa:(h + 1) * gqa] = o
+            lse[b, h * gqa:(h + 1) * gqa] = l
+    return out, lse
+
+
+def _build(budget, mn, mx, vb, n_kv, gqa, B, T, seed, k_layout=0, v_layout=0, student=None):
+    from blockgtq_amd.quantizer import build_batched_encode_args, encode_k_into, encode_v_into
+    qs, ens = zip(*[make_quantizer(seed=seed + h, head=h, budget=budget, min_bits=mn, max_bits=mx,
+                                   v_bits=vb, device=DEV) for h in range(n_kv)])
+    args = build_batched_encode_args(list(qs), device=DEV)
+    own = args['max_mixed_bytes'] if k_layout else args['max_tpb']
+    kw = max(4, (own + 3) // 4 * 4)
+    ng = args['max_n_groups']
+    vw = 64 if v_layout else args['v_packed_bytes']
+    ks, vs, qq = [], [], []
+    for h in range(n_kv):
+        kb, vb_, qb = [], [], []
+        for b in range(B):
+            k, v, q = make_kv(ens[h], T, seed=seed * 31 + h * 7 + b, n_q=gqa, student_t_nu=student)
+            kb.append(k); vb_.append(v); qb.append(q)
+        ks.append(np.stack(kb)); vs.append(np.stack(vb_)); qq.append(np.stack(qb))
+    k = torch.tensor(np.stack(ks, 1)).to(DEV)             # (B, H, T, D)
+    v = torch.tensor(np.stack(vs, 1)).to(DEV)
+    q = torch.tensor(np.concatenate(qq, 1)).to(DEV)        # (B, H*gqa, D)
+    kp = torch.zeros(B, n_kv, T + 2, kw, dtype=torch.uint8, device=DEV)
+    kn = torch.zeros(B, n_kv, T + 2, ng, dtype=torch.float16, device=DEV)
+    vp = torch.zeros(B, n_kv, T + 2, vw, dtype=torch.uint8, device=DEV)
+    vn = torch.zeros(B, n_kv, T + 2, dtype=torch.float16, device=DEV)
+    encode_k_into(args['plans'], k, kp, kn, 0, kw, ng, k_layout)
+    encode_v_into(args['plans'], v, vp, vn, 0, vw, v_layout)
+    q_rot = ops.rotate_q(args['plans'], q, n_kv)
+    return args, list(qs), q_rot, kp, kn, vp, vn
+
+
+CASES = [  # budget mn mx vb n_kv gqa B T k_layout v_layout
+    (192, 1, 5, 3, 2, 4, 1, 1000, 0, 0),
+    (192, 1, 8, 3, 2, 8, 2, 777, 0, 0),
+    (192, 1, 8, 3, 2, 8, 2, 777, 1, 1),
+    (128, 0, 4, 2, 2, 4, 1, 1500, 0, 0),
+    (300, 2, 8, 4, 1, 16, 1, 300, 0, 0),
+    (300, 2, 8, 4, 1, 16, 1, 300, 1, 0),
+    (64, 1, 1, 1, 1, 1, 3, 64, 0, 1),
+    (192, 3, 3, 3, 3, 2, 1, 513, 0, 0),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_decode_matches_checker(oracle_lib, case):
+    budget, mn, mx, vb, n_kv, gqa, B, T, kl, vl = case
+    args, qs, q_rot, kp, kn, vp, vn = _build(budget, mn, mx, vb, n_kv, gqa, B, T, seed=budget + T, k_layout=kl, v_layout=vl)
+    ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
+                              vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), [T] * B, gqa, kl, vl, vb)
+    for ns in (1, 3, 16, 0):
+        out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, T, n_splits=ns,
+                                        k_layout=kl, v_layout=vl, return_lse=True)
+        torch.cuda.synchronize()
+        assert np.abs(out.float().cpu().numpy() - ref).max() < TOL
+        assert np.abs(lse.cpu().numpy() - ref_lse).max() < 1e-3
+
+
+def test_tiny_contexts_and_empty_partitions(oracle_lib):
+    args, qs, q_rot, kp, kn, vp, vn = _build(192, 1, 5, 3, 2, 4, 2, 70, seed=5)
+    kpn, knn, vpn, vnn, qn = (t.cpu().numpy() for t in (kp, kn, vp, vn, q_rot))
+    for T in (1, 2, 63, 64, 65, 70):
+        ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kpn, knn, vpn, vnn, qn, [T, T], 4)
+        for ns in (1, 8, 64, 512):                  # more partitions than tokens
+            out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, T, n_splits=ns, return_lse=True)
+            assert np.abs(out.float().cpu().numpy() - ref).max() < TOL, (T, ns)
+            assert np.abs(lse.cpu().numpy() - ref_lse).max() < 1e-3
+    out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 0, n_splits=4, return_lse=True)
+    assert (out == 0).all() and torch.isinf(lse).all()
+
+
+def test_ragged_batch(oracle_lib):
+    args, qs, q_rot, kp, kn, vp, vn = _build(192, 1, 6, 3, 2, 4, 4, 600, seed=9)
+    lens = [600, 1, 257, 64]
+    lens_dev = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
+                              vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), lens, 4)
+    for ns in (1, 5, 32):
+        out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 600, seq_lens=lens_dev,
+                                        n_splits=ns, return_lse=True)
+        assert np.abs(out.float().cpu().numpy() - ref).max() < TOL
+        assert np.abs(lse.cpu().numpy() - ref_lse).max() < 1e-3
+
+
+def test_heavy_tailed_long_context_split_stress(oracle_lib):
+    """K2V2 with 0-bit blocks, Student-t(4) coordinates, many partitions."""
+    args, qs, q_rot, kp, kn, vp, vn = _build(128, 0, 4, 2, 1, 4, 1, 20000, seed=77, student=4)
+    ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
+                              vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), [20000], 4, v_bits=2)
+    # Student-t values push outputs to |x| ~ 4-5 where fp16 itself is spaced 3.9e-3 apart,
+    # so the 2e-3 bound is applied relative to max(1, |reference|).
+    bound = TOL * np.maximum(1.0, np.abs(ref))
+    for ns in (1, 64, 500):
+        out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 20000, n_splits=ns, return_lse=True)
+        assert (np.abs(out.float().cpu().numpy() - ref) < bound).all()
+        assert np.abs(lse.cpu().numpy() - ref_lse).max() < 2e-3
+
+
+def test_manager_append_and_attend_matches_checker(oracle_lib):
+    """Config-1 geometry (32 query / 8 KV heads) at a reduced context through the
+    manager API: append one token, attend, compare, repeat."""
+    w = wl.Workload("t", 2, 32, 8, 2, 500, 5e5, min_bits=1, max_bits=5, seed=4321)
+    mgr, energies = wl.build_manager(w, DEV)
+    wl.fill_cache(mgr, w, energies, DEV)
+    for step in range(2):
+        for li in range(2):
+            T = mgr.seq_len
+            q = wl.draw_q(w, li + 10 * step, DEV, T)
+            k1, v1 = wl.draw_kv(w, energies[li], 1, 555 + li + 10 * step, DEV, pos0=T)
+            out = mgr.append_and_attend(li, q, k1, v1)
+            assert out.shape == (2, 32, 1, 128) and out.dtype == torch.float16
+            plans = mgr._batched_args[li]['plans_np']
+            q_rot = ops.rotate_q(mgr._batched_args[li]['plans'], q[:, :, 0].contiguous(), 8)
+            ref, _ = _reference(oracle_lib, plans, mgr.quantizers[li],
+                                mgr._k_packed[li].cpu().numpy(), mgr._k_norms[li].cpu().numpy(),
+                                mgr._v_packed[li].cpu().numpy(), mgr._v_norms[li].cpu().numpy(),
+                                q_rot.cpu().numpy(), [T + 1] * 2, 4)
+            assert np.abs(out[:, :, 0].float().cpu().numpy() - ref).max() < TOL
+        mgr.increment_seq_len()
+    assert mgr.seq_len == 502
+    assert mgr.cache_memory_bytes() < mgr.fp16_cache_bytes() / 3
+
+
+def test_production_cache_and_fused_entry(oracle_lib):
+    """Nibble layouts through BlockGTQProductionCache, and the reference-style
+    per-head fused entry on slices of its cache."""
+    from blockgtq_amd import BlockGTQProductionCache
+    from blockgtq_amd.calibration import build_quantizers
+    from blockgtq_amd.kernels import fused_blockgtq_decode_attention
+    gen = torch.Generator().manual_seed(5)
+    n_layers, nkv, nq, T = 1, 2, 8, 400
+    en = wl.syn.block_energies(nkv, 64, gen)
+    amp = torch.cat([en.sqrt(), en.sqrt()], -1).unsqueeze(1)
+    layer_data = {0: {'q': torch.randn(nkv, 1024, 128, generator=gen) * amp,
+                      'k': torch.randn(nkv, 256, 128, generator=gen) * amp}}
+    quantizers, ba, ka = build_quantizers(layer_data, n_layers, nkv, 128, device=DEV)
+    cache = BlockGTQProductionCache(quantizers, ba, ka, n_layers, nkv, nq, 128, T + 8, device=DEV)
+    k = (torch.randn(1, nkv, T, 128, generator=gen) * amp).half().to(DEV)
+    v = torch.randn(1, nkv, T, 128, generator=gen).half().to(DEV)
+    cache._encode_batched(0, k, v, 0)
+    cache.seq_len = T
+    q = torch.randn(1, nq, 1, 128, generator=gen).half().to(DEV)
+    k1 = (torch.randn(1, nkv, 1, 128, generator=gen) * amp).half().to(DEV)
+    v1 = torch.randn(1, nkv, 1, 128, generator=gen).half().to(DEV)
+    out = cache.encode_and_attend(0, q, k1, v1)
+    q_rot = ops.rotate_q(ba[0]['plans'], q[:, :, 0].contiguous(), nkv)
+    ref, ref_lse = _reference(oracle_lib, ba[0]['plans_np'], quantizers[0], cache.k_packed[0].cpu().numpy(),
+                              cache.k_norms[0].cpu().numpy(), cache.v_packed[0].cpu().numpy(),
+                              cache.v_norms[0].cpu().numpy(), q_rot.cpu().numpy(), [T + 1], 4, 1, 1)
+    assert np.abs(out[:, :, 0].float().cpu().numpy() - ref).max() < TOL
+    # the appended record equals the checker's bytes
+    pl = ba[0]['plans_np'][1:2]
+    codes, _, corr = oracle_lib.encode_k(pl, k1[0, 1].cpu().numpy())
+    own = int(pl['k_mixed_bytes'][0])
+    assert np.array_equal(cache.k_packed[0, 0, 1, T, :own].cpu().numpy(), oracle_lib.pack_k(pl, codes, 1)[0])
+    # per-head fused entry with the reference's argument list
+    Tn = T + 1
+    for hi in range(nkv):
+        q8, a = quantizers[0][hi], ka[0][hi]
+        q_h = q8.rotate_q_for_packed_kernel(q[:, hi * 4:(hi + 1) * 4])
+        o, lse = fused_blockgtq_decode_attention(
+            q_h, cache.k_packed[0, :, hi:hi + 1, :Tn], cache.k_norms[0, :, hi:hi + 1, :Tn],
+            a['codebook_flat'], a['lut_offset'], a['norm_group'], a['segments_b'],
+            cache.v_packed[0, :, hi:hi + 1, :Tn], cache.v_norms[0, :, hi:hi + 1, :Tn], q8.v_lut,
+            scale=cache.scale, t_splits=8, v_bits=3, v_rotation=q8._v_rot,
+            k_nibble=True, v_nibble=True, return_lse=True)
+        assert o.shape == (1, 4, 1, 128)
+        assert np.abs(o[0, :, 0].float().cpu().numpy() - ref[0, hi * 4:(hi + 1) * 4]).max() < TOL
+        assert np.abs(lse[0].cpu().numpy() - ref_lse[0, hi * 4:(hi + 1) * 4]).max() < 1e-3
+
+
+def test_full_size_properties_config1():
+    """Llama-3.1-8B head geometry at the full 4096-token context: invariance to
+    the partition count and to the order of the context (softmax over a set)."""
+    w = wl.WORKLOADS["llama8b_4k_k3v3"]
+    mgr, energies = wl.build_manager(w, DEV)
+    wl.fill_cache(mgr, w, energies, DEV)
+    T = mgr.seq_len
+    q = wl.draw_q(w, 0, DEV, T)[:, :, 0].contiguous()
+    plans = mgr._batched_args[0]['plans']
+    q_rot = ops.rotate_q(plans, q, w.n_kv)
+    args = (mgr._k_packed[0], mgr._k_norms[0], mgr._v_packed[0], mgr._v_norms[0])
+    base = ops.decode_attention(plans, q_rot, *args, T, n_splits=1, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+    for ns in (7, 64, 512):
+        o = ops.decode_attention(plans, q_rot, *args, T, n_splits=ns, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+        assert (o - base).abs().max() < 1e-3
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(1)).to(DEV)
+    shuffled = tuple(t[:, :, :T][:, :, perm].contiguous() for t in args)
+    o = ops.decode_attention(plans, q_rot, *shuffled, T, n_splits=16, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+    assert (o - base).abs().max() < 1e-3
+    # doubling the context by repeating it leaves the output unchanged
+    doubled = tuple(torch.cat([t[:, :, :T], t[:, :, :T]], dim=2).contiguous() for t in args)
+    o = ops.decode_attention(plans, q_rot, *doubled, 2 * T, n_splits=32, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+    assert (o - base).abs().max() < 1e-3
+
+
+def test_window_partial_merges_like_one_softmax(oracle_lib):
+    """Closed form: softmax over [window ++ packed] == lse-merge of the two partials."""
+    from blockgtq_amd import _capi
+    args, qs, q_rot, kp, kn, vp, vn = _build(192, 1, 5, 3, 2, 4, 2, 300, seed=13)
+    gen = torch.Generator().manual_seed(2)
+    W = 37
+    q = torch.randn(2, 8, 128, generator=gen).half().to(DEV)
+    q_rot = ops.rotate_q(args['plans'], q, 2)
+    kb = torch.randn(2, 2, W, 128, generator=gen).half().to(DEV)
+    vb = torch.randn(2, 2, W, 128, generator=gen).half().to(DEV)
+    lens = torch.tensor([W, 5], dtype=torch.int32, device=DEV)
+    po = torch.empty(2, 8, 128, device=DEV); pl = torch.empty(2, 8, device=DEV)
+    L = _capi.lib()
+    _capi.check(L.bgtq_window_attn(_capi.ptr(q), q.stride(0), q.stride(1), _capi.ptr(kb), _capi.ptr(vb),
+                                   kb.stride(0), kb.stride(1), kb.stride(2), _capi.ptr(lens), W, 2, 2, 4,
+                                   128 ** -0.5, _capi.ptr(po), _capi.ptr(pl), _capi.stream_ptr()), "window")
+    out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 300, n_splits=4, return_lse=True,
+                                    extra_out=po, extra_lse=pl)
+    ref_p, lse_p = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
+                              vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), [300, 300], 4)
+    for b in range(2):
+        n = int(lens[b])
+        for hq in range(8):
+            h = hq // 4
+            lw = (q[b, hq].double() @ kb[b, h, :n].double().T).cpu() / np.sqrt(128)
+            w_lse = torch.logsumexp(lw, 0)
+            w_out = torch.softmax(lw, 0) @ vb[b, h, :n].double().cpu()
+            a = torch.tensor([float(lse_p[b, hq]), float(w_lse)], dtype=torch.float64)
+            wgt = torch.softmax(a, 0)
+            want = wgt[0] * torch.tensor(ref_p[b, hq]).double() + wgt[1] * w_out
+            assert (out[b, hq].double().cpu() - want).abs().max() < TOL
+            assert abs(float(lse[b, hq]) - float(torch.logsumexp(a, 0))) < 1e-3

@@ -1,0 +1,256 @@
+"""Host-side plan builders against closed forms, invariants and brute force."""
+import itertools
+import math
+import re
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from blockgtq_amd import BlockGTQPipeline, BlockGTQQuantizer, greedy_bit_allocation
+from blockgtq_amd import codebooks, plan as P, v_packing
+from blockgtq_amd.quantizer import build_pack_meta
+from helpers import make_quantizer, stream_pack
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---------------------------------------------------------------- allocator
+def _objective(s, b):
+    return float((np.asarray(s, dtype=np.float64) * 4.0 ** (-np.asarray(b, dtype=np.float64))).sum())
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_allocator_is_the_exact_optimum_on_small_problems(seed):
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(2, 6))
+    lo, hi = int(rng.integers(0, 2)), int(rng.integers(3, 5))
+    budget = int(rng.integers(n * lo, n * hi + 1))
+    s = torch.tensor(rng.uniform(0.01, 50.0, n), dtype=torch.float32)
+    got = greedy_bit_allocation(s, budget, lo, hi).numpy()
+    assert got.sum() == budget and got.min() >= lo and got.max() <= hi
+    best = min(_objective(s.numpy(), b)
+               for b in itertools.product(range(lo, hi + 1), repeat=n) if sum(b) == budget)
+    assert _objective(s.numpy(), got) == pytest.approx(best, rel=1e-12)
+
+
+def test_allocator_invariants_and_ties():
+    s = torch.ones(8)
+    # equal scores: bits go to the lowest indices first
+    assert greedy_bit_allocation(s, 8 + 3, 1, 4).tolist() == [2, 2, 2, 1, 1, 1, 1, 1]
+    # monotone in the score
+    s = torch.tensor([0.1, 1.0, 10.0, 100.0])
+    a = greedy_bit_allocation(s, 12, 1, 8).tolist()
+    assert a == sorted(a) and sum(a) == 12
+    # budget below the floor: everything stays at min_bits
+    assert greedy_bit_allocation(s, 2, 1, 8).tolist() == [1, 1, 1, 1]
+    # budget above the ceiling: saturates at max_bits
+    assert greedy_bit_allocation(s, 99, 1, 3).tolist() == [3, 3, 3, 3]
+    # zero scores never receive bits beyond the floor
+    assert greedy_bit_allocation(torch.tensor([0.0, 1.0]), 6, 0, 8).tolist() == [0, 6]
+
+
+# ---------------------------------------------------------------- codebooks
+def test_centroid_closed_forms():
+    d = 36
+    c1 = codebooks.lloyd_max_centroids(1, d)
+    assert np.allclose(c1, [-math.sqrt(2 / (math.pi * d)), math.sqrt(2 / (math.pi * d))], rtol=0, atol=1e-15)
+    c2 = codebooks.lloyd_max_centroids(2, d)
+    assert np.allclose(c2 * math.sqrt(d), [-1.51, -0.453, 0.453, 1.51], atol=1e-12)
+    # textbook Lloyd-Max levels of the unit Gaussian, 8 and 16 levels
+    c3 = codebooks.lloyd_max_centroids(3, d) * math.sqrt(d)
+    assert np.allclose(c3[4:], [0.2451, 0.7560, 1.3439, 2.1520], atol=2e-4)
+    assert np.allclose(c3, -c3[::-1], atol=1e-9)
+    # 16 levels: 100 Lloyd iterations stop a little short of the textbook optimum
+    c4 = codebooks.lloyd_max_centroids(4, d) * math.sqrt(d)
+    assert np.allclose(c4[8:], [0.1284, 0.3881, 0.6568, 0.9424, 1.2562, 1.6181, 2.0690, 2.7326], atol=2e-2)
+    assert np.allclose(c4, -c4[::-1], atol=1e-9)
+
+
+def _cell_means_by_quadrature(edges, sig):
+    from scipy.stats import norm
+    from scipy import integrate
+    ext = np.concatenate([[-14 * sig], edges, [14 * sig]])
+    out = []
+    for lo, hi in zip(ext[:-1], ext[1:]):
+        num = integrate.quad(lambda x: x * norm.pdf(x, scale=sig), lo, hi, epsabs=0, epsrel=1e-12)[0]
+        den = integrate.quad(lambda x: norm.pdf(x, scale=sig), lo, hi, epsabs=0, epsrel=1e-12)[0]
+        out.append(num / den)
+    return np.array(out)
+
+
+def test_three_bit_centroids_are_a_lloyd_fixed_point():
+    d = 128
+    c = codebooks.lloyd_max_centroids(3, d)
+    again = _cell_means_by_quadrature((c[:-1] + c[1:]) / 2, 1 / math.sqrt(d))
+    assert np.allclose(c, again, rtol=1e-7, atol=1e-10)
+
+
+def test_lloyd_schedule_against_numerical_integration():
+    """100 Lloyd iterations from the equal-mass cells, cell means by quadrature
+    instead of the pdf/cdf closed form."""
+    from scipy.stats import norm
+    bw, d = 4, 20
+    sig = 1 / math.sqrt(d)
+    n = 1 << bw
+    c = _cell_means_by_quadrature(norm.ppf(np.linspace(0, 1, n + 1)[1:-1], scale=sig), sig)
+    for _ in range(100):
+        c = _cell_means_by_quadrature((c[:-1] + c[1:]) / 2, sig)
+    assert np.allclose(codebooks.lloyd_max_centroids(bw, d), np.sort(c), rtol=1e-7, atol=1e-10)
+
+
+@pytest.mark.parametrize("fix", [True, False])
+def test_rotation_is_proper_and_deterministic(fix):
+    r = codebooks.haar_rotation(48, 45, zero_sign_fix=fix)
+    assert np.allclose(r.T @ r, np.eye(48), atol=1e-12)
+    assert np.linalg.det(r) == pytest.approx(1.0, abs=1e-10)
+    assert np.array_equal(r, codebooks.haar_rotation(48, 45, zero_sign_fix=fix))
+    assert not np.allclose(r, codebooks.haar_rotation(48, 46, zero_sign_fix=fix))
+    # uniqueness of QR with positive diag(R): Q^T G must be upper triangular, diag > 0
+    g = np.random.default_rng(45).standard_normal((48, 48))
+    rr = r.T @ g
+    rr[:, 0] *= 1.0  # no-op, keeps the intent readable
+    lower = np.tril(rr, -1)
+    if np.linalg.det(np.linalg.qr(g)[0] * np.sign(np.diag(np.linalg.qr(g)[1]))) > 0:
+        assert np.allclose(lower, 0, atol=1e-10) and (np.diag(rr) > 0).all()
+
+
+def test_mc_lloyd_centroids_properties():
+    c = codebooks.mc_lloyd_centroids(3, 128)
+    assert c.shape == (8,) and (np.diff(c) > 0).all()
+    # fixed point on its own sample set
+    sig = 1 / np.sqrt(128)
+    x = np.random.default_rng(0).normal(0, sig, 100000)
+    cell = np.searchsorted((c[:-1] + c[1:]) / 2, x)
+    means = np.array([x[cell == i].mean() for i in range(8)])
+    assert np.allclose(c, means, atol=2e-8)
+    # and close to the analytic Lloyd-Max levels (sampling noise of 100k draws)
+    assert np.allclose(c, codebooks.lloyd_max_centroids(3, 128), atol=1.5e-3)
+
+
+def test_code_lut_is_nearest_centroid_of_bin_centres():
+    q, _ = make_quantizer(seed=3, max_bits=6)
+    lut = q._code_lut.numpy()
+    for g, bw in enumerate(q._group_bits):
+        s = q._pack_meta[bw]['start']
+        c = q._pos_centroids[s, :1 << bw].double().numpy()
+        off, inv = float(q._lut_offsets[s]), float(q._lut_inv_scales[s])
+        centres = off + (np.arange(256) + 0.5) / inv
+        nearest = np.abs(centres[:, None] - c[None, :]).argmin(1)
+        row = lut[int(q._pos_to_cb[s])]
+        assert (np.diff(row.astype(int)) >= 0).all()
+        assert row[0] == 0 and row[-1] == (1 << bw) - 1
+        # bins whose centre sits within fp32 noise of a boundary may go either way
+        b = (c[:-1] + c[1:]) / 2
+        near = np.abs(centres[:, None] - b[None, :]).min(1) < 1e-6
+        assert (row[~near] == nearest[~near]).all()
+        # table spans [c_min - sp/2, c_max + sp/2]
+        sp = (c[-1] - c[0]) / (len(c) - 1)
+        assert off == pytest.approx(c[0] - sp / 2, rel=1e-6)
+        assert 256 / inv == pytest.approx(c[-1] - c[0] + sp, rel=1e-6)
+
+
+# ---------------------------------------------------------------- pipeline
+def test_pipeline_layout_invariants():
+    q, _ = make_quantizer(seed=5, min_bits=0, max_bits=6, budget=160)
+    bits = q.bit_allocation
+    hp = q._head_perm
+    per_dim = torch.cat([bits, bits])[hp]
+    assert sorted(hp.tolist()) == list(range(128))
+    assert (per_dim[1:] >= per_dim[:-1]).all()
+    assert ((hp[1::2] - hp[0::2]) == 64).all()            # a block's two dims stay adjacent
+    rot = q._block_rot_T.T
+    assert torch.allclose(rot @ rot.T, torch.diag((per_dim > 0).float()), atol=1e-5)
+    for g, bw in enumerate(q._group_bits):
+        m = q._pack_meta[bw]
+        s, e = m['start'], m['start'] + m['length']
+        blk = rot[s:e, s:e]
+        assert rot[s:e, :s].abs().sum() == 0 and rot[s:e, e:].abs().sum() == 0
+        if bw < q.rotation_threshold:
+            assert torch.equal(blk, torch.eye(e - s))
+        else:
+            assert not torch.equal(blk, torch.eye(e - s))
+        assert (q._group_of_full[s:e] == g).all()
+    assert (q._group_of_full[:q._n_zero_dims] == -1).all()
+
+
+def test_pack_meta_sizes_match_the_documented_example():
+    # 1b x 10 blocks, 2b x 12, 3b x 18, 4b x 16, 5b x 8 -> bytes 3+6+15+16+16 = 56
+    alloc = torch.tensor([1] * 10 + [2] * 12 + [3] * 18 + [4] * 16 + [5] * 8)
+    pipe = BlockGTQPipeline(128, device='cpu')
+    pipe.set_allocation(alloc)
+    pm = build_pack_meta(alloc, pipe._head_perm)
+    assert [pm[b]['length'] for b in (1, 2, 3, 4, 5)] == [20, 24, 36, 32, 16]
+    assert [pm[b]['packed_bytes'] for b in (1, 2, 3, 4, 5)] == [3, 6, 15, 16, 16]
+    assert [pm[b]['pack_offset'] for b in (1, 2, 3, 4, 5)] == [0, 3, 9, 24, 40]
+    assert pm['total_packed_bytes'] == 56
+    assert (pm['nopack_start'], pm['nopack_len'], pm['nopack_off']) == (112, 16, 40)
+    # widths <= 4 only: the raw-byte run starts past the end of the vector
+    pm = build_pack_meta(torch.full((64,), 3), BlockGTQPipeline(128, device='cpu')._head_perm
+                         if False else torch.arange(128).view(2, 64).T.reshape(-1))
+    assert pm['nopack_start'] == 128 and pm['nopack_len'] == 0 and pm['total_packed_bytes'] == 48
+
+
+def test_plan_struct_mirrors_the_quantizer():
+    q, _ = make_quantizer(seed=9, max_bits=7, budget=200)
+    p = q.plan()[0]
+    n = int(p['n_seg'])
+    assert n == q._n_groups
+    assert int(p['k_row_bytes']) == q._total_packed_bytes
+    assert int(p['k_mixed_bytes']) == q._pack_meta['nopack_start'] // 2 + q._pack_meta['nopack_len']
+    assert sum(int(x) for x in p['seg_len'][:n]) == 128
+    for g in range(n):
+        bw = int(p['seg_bw'][g])
+        nc = 1 << bw
+        assert np.isinf(p['k_boundaries'][g][nc - 1:]).all()
+        c = p['k_centroids'][g][:nc]
+        assert np.allclose(p['k_boundaries'][g][:nc - 1], (c[:-1] + c[1:]) / 2, atol=1e-7)
+        assert np.array_equal(p['k_codebook_f16'][g][:nc].view(np.float16), c.astype(np.float16))
+    assert np.allclose(p['v_rot'].reshape(128, 128), p['v_rot_T'].reshape(128, 128).T)
+
+
+# ---------------------------------------------------------------- V packing
+@pytest.mark.parametrize("bits", [1, 2, 3, 4])
+def test_v_packing_matches_a_plain_bit_stream(bits):
+    rng = np.random.default_rng(bits)
+    codes = rng.integers(0, 1 << bits, size=(17, 128)).astype(np.uint8)
+    packed = v_packing.pack_v_codes(torch.tensor(codes), bits).numpy()
+    assert packed.shape[1] == v_packing.packed_v_bytes(128, bits) == {1: 16, 2: 32, 3: 48, 4: 64}[bits]
+    assert np.array_equal(packed, stream_pack(codes, bits))
+    back = v_packing.unpack_v_codes(torch.tensor(packed), bits, 128).numpy()
+    assert np.array_equal(back, codes)
+    if bits == 3:       # the 8-codes-in-3-bytes formulas
+        c = codes[:, :8].astype(int)
+        assert np.array_equal(packed[:, 0], (c[:, 0] | c[:, 1] << 3 | c[:, 2] << 6) & 0xFF)
+        assert np.array_equal(packed[:, 1], (c[:, 2] >> 2 | c[:, 3] << 1 | c[:, 4] << 4 | c[:, 5] << 7) & 0xFF)
+        assert np.array_equal(packed[:, 2], (c[:, 5] >> 1 | c[:, 6] << 2 | c[:, 7] << 5) & 0xFF)
+
+
+# ---------------------------------------------------------------- library surface
+def test_library_loads_and_exports_every_declared_symbol():
+    from blockgtq_amd import _capi
+    lib = _capi.lib()
+    text = open(os.path.join(ROOT, "include", "bgtq.h")).read()
+    declared = set(re.findall(r"\b(bgtq_[a-z_0-9]+)\s*\(", text))
+    declared -= {"bgtq_head_plan"}
+    assert declared, "no declarations parsed"
+    missing = [name for name in sorted(declared) if not hasattr(lib, name)]
+    assert not missing, f"library lacks {missing}"
+    assert lib.bgtq_plan_sizeof() == P.PLAN_DTYPE.itemsize
+    assert lib.bgtq_abi_version() >= 1
+    assert lib.bgtq_workspace_bytes(2, 16, 8) == 2 * 16 * 8 * 129 * 4
+    assert lib.bgtq_strerror(-1).decode() == "invalid argument"
+    # argument validation happens on the host before any launch
+    assert lib.bgtq_encode_k(None, None, 0, 0, 0, 1, 1, 1, None, 0, 0, 0, 8,
+                             None, 0, 0, 0, 1, None, 0, 0, 0, None) == -1
+    # an empty call is legal and launches nothing
+    assert lib.bgtq_encode_k(None, None, 0, 0, 0, 1, 1, 0, None, 0, 0, 0, 8,
+                             None, 0, 0, 0, 1, None, 0, 0, 0, None) == 0
+
+
+def test_device_paths_refuse_cpu_tensors():
+    from blockgtq_amd import _capi
+    q, _ = make_quantizer(seed=1)
+    with pytest.raises(_capi.BgtqError):
+        q.compress(torch.zeros(4, 128, dtype=torch.float16))
