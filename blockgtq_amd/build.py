@@ -21,7 +21,9 @@ COMMON = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
 # behind the author's back.
 SOURCES = {
     "bgtq_encode.hip": ["-ffp-contract=off"],
-    "bgtq_decode.hip": [],
+    "bgtq_decode.hip": ["-fno-strict-aliasing"],
+    # LDS tiles are written as 128-bit / 16-bit words and read back as 32-bit words
+    "bgtq_decode_mfma.hip": ["-fno-strict-aliasing"],
 }
 
 

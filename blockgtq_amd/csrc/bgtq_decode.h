@@ -1,0 +1,24 @@
+// Argument block shared by the decode attention kernels (internal).
+#pragma once
+#include "bgtq_common.h"
+
+struct DecodeArgs {
+    const bgtq_head_plan* plans;
+    const uint16_t* q;  int64_t q_sb, q_sh;
+    const uint8_t* kp;  int64_t kp_sb, kp_sh, kp_st;
+    const uint16_t* kn; int64_t kn_sb, kn_sh, kn_st;
+    const uint8_t* vp;  int64_t vp_sb, vp_sh, vp_st;
+    const uint16_t* vn; int64_t vn_sb, vn_sh, vn_st;
+    const int32_t* seq_lens; int T;
+    int B, n_kv, gqa, n_splits;
+    float* part_out; float* part_lse;
+    int k_layout, v_layout;
+    float scale;
+    int k_row_width;       // widest K record over the heads (LDS sizing)
+    int v_row_width;
+};
+
+// Fast path: MFMA kernel for bit-packed K and V records (bgtq_decode_mfma.hip).
+// Returns BGTQ_EUNSUPPORTED when the arguments do not meet its layout
+// requirements, in which case the caller takes the layout-agnostic kernel.
+int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream);

@@ -11,6 +11,7 @@
 // work-group, and thread (d, half) accumulates output dim d for one half of
 // the query heads over the tile's tokens.
 #include "bgtq_common.h"
+#include "bgtq_decode.h"
 
 namespace {
 
@@ -18,21 +19,6 @@ constexpr int D = BGTQ_D;
 constexpr int GT = 256;          // threads == tokens per tile of the generic kernel
 constexpr int ROW_PAD = 4;       // slack bytes so a 2-byte window never leaves the tile
 
-struct DecodeArgs {
-    const bgtq_head_plan* plans;
-    const uint16_t* q;  int64_t q_sb, q_sh;
-    const uint8_t* kp;  int64_t kp_sb, kp_sh, kp_st;
-    const uint16_t* kn; int64_t kn_sb, kn_sh, kn_st;
-    const uint8_t* vp;  int64_t vp_sb, vp_sh, vp_st;
-    const uint16_t* vn; int64_t vn_sb, vn_sh, vn_st;
-    const int32_t* seq_lens; int T;
-    int B, n_kv, gqa, n_splits;
-    float* part_out; float* part_lse;
-    int k_layout, v_layout;
-    float scale;
-    int k_row_width;       // widest K record over the heads (LDS sizing)
-    int v_row_width;
-};
 
 __device__ inline float wave_max(float v) {
 #pragma unroll
@@ -375,7 +361,15 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
 
 }  // namespace
 
+static int g_decode_path = 0;
+
 extern "C" {
+
+int bgtq_set_decode_path(int path) {
+    if (path < 0 || path > 2) return BGTQ_EINVAL;
+    g_decode_path = path;
+    return BGTQ_OK;
+}
 
 size_t bgtq_workspace_bytes(int B, int n_q, int n_splits) {
     if (B <= 0 || n_q <= 0 || n_splits <= 0) return 0;
@@ -428,6 +422,11 @@ int bgtq_decode_attn(const bgtq_head_plan* plans,
     BGTQ_CHECK_ARG(v_row_width >= 1 && v_row_width <= BGTQ_D / 2);
     a.k_row_width = k_row_width; a.v_row_width = v_row_width;
     hipStream_t st = (hipStream_t)stream;
+    if (g_decode_path != 1) {
+        int rc = bgtq_launch_decode_mfma(a, st);
+        if (rc != BGTQ_EUNSUPPORTED) return rc;
+        if (g_decode_path == 2) return rc;        // forced fast path: report why it refused
+    }
     if (gqa <= 4) return launch_generic<4>(a, st);
     if (gqa <= 8) return launch_generic<8>(a, st);
     return launch_generic<16>(a, st);

@@ -165,6 +165,14 @@ int bgtq_rotate_q(const bgtq_head_plan* plans,
                   void* q_rot, int64_t qr_sr, int64_t qr_sh,
                   int n_rows, int n_kv, int gqa, void* stream);
 
+/*
+ * Kernel selection of bgtq_decode_attn (process-wide; meant for tests and
+ * profiling): 0 = automatic (MFMA kernel when the layout allows it, otherwise
+ * the layout-agnostic kernel), 1 = always the layout-agnostic kernel,
+ * 2 = MFMA kernel only (BGTQ_EUNSUPPORTED if it cannot take the call).
+ */
+int bgtq_set_decode_path(int path);
+
 /* Bytes of fp32 scratch bgtq_decode_attn needs for (B, n_q, n_splits). */
 size_t bgtq_workspace_bytes(int B, int n_q, int n_splits);
 
@@ -183,8 +191,8 @@ int bgtq_default_splits(int B, int n_kv, int max_T);
  *              k_row_width / v_row_width = record bytes per token the cache holds
  *              (the widest head's record), strides may be larger
  *   seq_lens   device int32[B] tokens visible per batch row, or NULL -> T for all
- *   n_splits   partitions per (b, kv head); partition c covers
- *              [c*chunk, min((c+1)*chunk, T_b)), chunk = ceil(T_b / n_splits)
+ *   n_splits   partitions per (b, kv head); the partitions tile [0, T_b) in
+ *              order, how the boundaries are rounded is up to the kernel
  *   partial_out fp32 [B][n_q][n_splits][128]  (normalised, V still rotated)
  *   partial_lse fp32 [B][n_q][n_splits]       (natural log; -inf for an empty partition)
  */
