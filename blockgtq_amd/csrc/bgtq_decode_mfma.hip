@@ -1,27 +1,28 @@
 // MFMA decode attention over bit-packed K and V records (gfx950).
 //
 // One work-group of 4 waves owns one partition of one (batch row, KV head);
-// every wave walks its own 32-token tiles with a private online softmax and the
+// every wave walks its own 64-token tiles with a private online softmax and the
 // four results are merged through LDS at the end.
 //
 // Dequantisation is table driven.  A "unit" is 8 consecutive codes of one
 // token (bw bytes of the record).  For every bit width <= 4 the work-group
 // builds a pair table in LDS: entry (c0 | c1 << bw) holds the two fp16
-// centroids of a code pair, replicated once per LDS bank so that 64 lanes with
-// 64 different indices never collide (lane l reads the copy in bank l % 32).
-// A unit therefore costs one raw read, four {bit-field extract, shift-add,
-// table read} triples and gives the eight fp16 operands of one MFMA k-group.
+// centroids of a code pair, replicated across LDS banks so that lanes with
+// different indices do not collide (32 copies, 8 for the 256-entry 4-bit table).
+// A unit costs one raw read, four {bit-field extract, shift-add, table read}
+// triples and yields the eight fp16 operands of one MFMA k-group.
 //
-// QK^T:  v_mfma_f32_16x16x32_f16 with A = dequantised K (row = token, lane group
-//        g supplies unit 4m+g of MFMA step m, steps never mix segments so the
-//        field widths are wave-uniform scalars), B = rotated queries (kept in
-//        registers for the whole partition, zero on padding dims), D[token][head].
+// QK^T:  v_mfma_f32_16x16x32_f16, A = dequantised K (row = token, lane group g
+//        supplies unit 4m+g of step m; a step never mixes segments, so field
+//        width and table are the same for the whole wave), B = rotated queries
+//        laid out per step in LDS (zero on padding dims), D[token][head].  Each
+//        segment accumulates on its own and is scaled by the fp32 group norm of
+//        its token row when the segment ends.
 // PV:    the D layout of two 16-token blocks is exactly the A layout of a
 //        K=32 step (row = head, lane group g holds 8 tokens), so P never leaves
 //        its lane; B = dequantised V where lane (j, g) decodes unit j of its 8
-//        tokens and hands dim 8j+e to MFMA e.
-// K group norms are applied in fp32 to each segment's partial score, the V norm
-// scales P before it is rounded to fp16.
+//        tokens and hands dim 8j+e to MFMA e.  The V norm is folded into P in
+//        fp32 before P is rounded to fp16.
 #include "bgtq_decode.h"
 
 namespace {
@@ -29,49 +30,71 @@ namespace {
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef int int4v __attribute__((ext_vector_type(4)));
 
 constexpr int D = BGTQ_D;
 constexpr int MW = 4;              // waves per work-group
 constexpr int NT = MW * 64;
-constexpr int MT = 32;             // tokens per wave tile
-constexpr int MAX_STEPS = 12;      // sum over segments of ceil(ceil(len/8)/4) <= 11
-constexpr int REPL = 128;          // bytes per pair-table entry (32 banks x 4 B)
+constexpr int MT = 64;             // tokens per wave tile = 4 MFMA row blocks
+constexpr int NBLK = MT / 16;
+constexpr int MAX_STEPS = BGTQ_MAX_STEPS;
+constexpr int KR = 6;              // 128-bit prefetch registers per lane for a K tile (row <= 95 B)
+constexpr int VR = 5;              // same for a V tile (row <= 64 B)
 
-// LDS byte offsets of the K pair tables by bit width (each width occurs at most once)
-__host__ __device__ constexpr int klut_off(int bw) {
-    return bw == 1 ? 0 : bw == 2 ? 4 * REPL : bw == 3 ? (4 + 16) * REPL : (4 + 16 + 64) * REPL;
-}
-constexpr int KLUT_BYTES = (4 + 16 + 64 + 256) * REPL;          // 43520
-constexpr int KRAW_OFF = KLUT_BYTES;                             // 4 tables x 256 fp16
-constexpr int KRAW_BYTES = 4 * 256 * 2;
-constexpr int VLUT_OFF = KRAW_OFF + KRAW_BYTES;
-__host__ __device__ constexpr int vlut_bytes(int vbw) { return (1 << (2 * vbw)) * REPL; }
-
-struct StepTable {            // wave-uniform description of the MFMA steps of QK^T
-    int n_steps;
-    int bw[MAX_STEPS];        // code width (5..8 = raw bytes)
-    int seg[MAX_STEPS];       // segment index (norm column)
-    int unit0[MAX_STEPS];     // first unit of the step inside its segment
-    int n_units[MAX_STEPS];   // units of the whole segment
-};
+// ---- LDS layout (bytes) -----------------------------------------------------------
+constexpr int KLUT1 = 0;                       // 4 entries   x 128 B
+constexpr int KLUT2 = KLUT1 + 4 * 128;         // 16 entries  x 128 B
+constexpr int KLUT3 = KLUT2 + 16 * 128;        // 64 entries  x 128 B
+constexpr int KLUT4 = KLUT3 + 64 * 128;        // 256 entries x 32 B
+constexpr int KRAW = KLUT4 + 256 * 32;         // 4 tables x 256 fp16 (bw 5..8)
+constexpr int VLUT = KRAW + 4 * 512;
+__host__ __device__ constexpr int vlut_bytes(int vbw) { return vbw == 4 ? 256 * 32 : (1 << (2 * vbw)) * 128; }
+__host__ __device__ constexpr int steps_off(int vbw) { return VLUT + vlut_bytes(vbw); }   // MAX_STEPS x 32 B
+__host__ __device__ constexpr int qop_off(int vbw) { return steps_off(vbw) + MAX_STEPS * 32; }  // MAX_STEPS x 1 KB
+__host__ __device__ constexpr int wave_off(int vbw) { return qop_off(vbw) + MAX_STEPS * 1024; }
 
 __device__ inline uint32_t lds_u32(const uint8_t* base, uint32_t off) {
     return *(const uint32_t*)(base + off);
 }
-__device__ inline float wave_xor_max(float v, int m) { return fmaxf(v, __shfl_xor(v, m, 64)); }
 
-// copy nbytes (multiple of 4) from 4-byte aligned global memory into LDS keeping
-// the 16-byte phase of the source, so full 128-bit loads stay aligned
-__device__ inline uint32_t stage_bytes(const uint8_t* src, int nbytes, uint8_t* dst, int lane) {
-    uint32_t phase = (uint32_t)((uintptr_t)src & 15);
-    const uint8_t* al = src - phase;
-    int total = (int)phase + nbytes;
-    int full = total & ~15;
-    for (int off = lane * 16; off < full; off += 64 * 16)
-        *(uint4*)(dst + off) = *(const uint4*)(al + off);
-    int tail = (total - full) >> 2;           // 0..3 dwords
-    if (lane < tail) *(uint32_t*)(dst + full + lane * 4) = *(const uint32_t*)(al + full + lane * 4);
-    return phase;
+// A tile of packed records is one contiguous byte range.  It is fetched with
+// aligned 128-bit loads (the 16-byte phase of the source is kept in LDS), first
+// into registers while the previous tile is being processed, then into LDS.
+template <int NR>
+struct TileRegs {
+    uint4 r[NR];
+    uint32_t phase;
+    int total;      // phase + valid bytes
+};
+
+template <int NR>
+__device__ inline void tile_issue(TileRegs<NR>& t, const uint8_t* src, int nbytes, int lane) {
+    t.phase = (uint32_t)((uintptr_t)src & 15);
+    t.total = (int)t.phase + nbytes;
+    const uint8_t* al = src - t.phase;
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+        const int off = lane * 16 + i * 1024;
+        uint4 v = {0, 0, 0, 0};
+        if (off + 16 <= t.total) {
+            v = *(const uint4*)(al + off);
+        } else if (off < t.total) {            // last, partial chunk: never read past the tile
+            const uint32_t* w = (const uint32_t*)(al + off);
+            v.x = w[0];
+            if (off + 8 <= t.total) v.y = w[1];
+            if (off + 12 <= t.total) v.z = w[2];
+        }
+        t.r[i] = v;
+    }
+}
+
+template <int NR>
+__device__ inline void tile_commit(const TileRegs<NR>& t, uint8_t* dst, int lane) {
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+        const int off = lane * 16 + i * 1024;
+        if (off < t.total) *(uint4*)(dst + off) = t.r[i];
+    }
 }
 
 template <int VBW>
@@ -90,97 +113,112 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
 
     // ---- LDS carve-up --------------------------------------------------------
     const int krow = a.k_row_width, vrow = a.v_row_width;
-    const int kt_bytes = (MT * krow + 16 + 8 + 15) & ~15;
-    const int vt_bytes = (MT * vrow + 16 + 8 + 15) & ~15;
+    const int kt_bytes = (MT * krow + 16 + 12 + 15) & ~15;
+    const int vt_bytes = (MT * vrow + 16 + 12 + 15) & ~15;
     constexpr int kn_bytes = BGTQ_MAX_SEGMENTS * MT * 4;  // fp32 norms, [segment][token]
-    const int wave_bytes = kt_bytes + vt_bytes + kn_bytes + 64;
-    uint8_t* klut = smem;
-    uint8_t* vlut = smem + VLUT_OFF;
-    uint8_t* wbuf = smem + VLUT_OFF + vlut_bytes(VBW) + wave * wave_bytes;
-    uint8_t* kt_s = wbuf;
+    const int wave_bytes = kt_bytes + vt_bytes + kn_bytes + MT * 2;
+    uint8_t* vlut = smem + VLUT;
+    int4v* steps_s = (int4v*)(smem + steps_off(VBW));
+    uint8_t* qop_s = smem + qop_off(VBW);
+    uint8_t* wbuf0 = smem + wave_off(VBW);
+    uint8_t* kt_s = wbuf0 + wave * wave_bytes;
     uint8_t* vt_s = kt_s + kt_bytes;
     float* kn_s = (float*)(vt_s + vt_bytes);
-    uint8_t* vn_s = (uint8_t*)kn_s + kn_bytes;            // 32 fp16
+    uint16_t* vn_s = (uint16_t*)((uint8_t*)kn_s + kn_bytes);
 
-    // ---- tables -----------------------------------------------------------------
-    for (int s = 0; s < P.n_seg; s++) {
-        const int bw = P.seg_bw[s];
+    // ---- init 1: plan header, step schedule, codebooks and queries into LDS scratch --
+    // (scratch lives in the tile buffers, which are idle until the main loop)
+    int* hdr_s = (int*)wbuf0;                             // first 56 ints of the plan
+    uint16_t* cb_s = (uint16_t*)(wbuf0 + 256);            // [8][16] K codebooks + [16] V
+    int* stp_s = (int*)(wbuf0 + 576);                     // n_steps, 3 pad, step[12][8]
+    uint16_t* q_s = (uint16_t*)(wbuf0 + 1024);            // [16][128] rotated queries
+    if (tid < 56) hdr_s[tid] = ((const int*)&P)[tid];
+    if (tid >= 64 && tid < 64 + 4 + MAX_STEPS * 8) stp_s[tid - 64] = (&P.n_steps)[tid - 64];
+    for (int i = tid; i < BGTQ_MAX_SEGMENTS * 16; i += NT) cb_s[i] = P.k_codebook_f16[i >> 4][i & 15];
+    if (tid < 16) cb_s[BGTQ_MAX_SEGMENTS * 16 + tid] = P.v_lut_f16[tid];
+    for (int i = tid; i < 16 * D / 2; i += NT) {
+        int hq = i / (D / 2), d2 = i - hq * (D / 2);
+        uint32_t v = 0;
+        if (hq < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + hq) * a.q_sh + d2 * 2);
+        ((uint32_t*)q_s)[i] = v;
+    }
+    __syncthreads();
+    const int n_seg = hdr_s[0];
+    const int* seg_bw = hdr_s + 8;
+    const int* seg_start = hdr_s + 16;
+    const int* seg_len = hdr_s + 24;
+    const int n_steps = min(stp_s[0], MAX_STEPS);
+
+    // ---- init 2: pair tables, step table -------------------------------------------
+    for (int s = 0; s < n_seg; s++) {
+        const int bw = seg_bw[s];
         if (bw <= 4) {
             const int n = 1 << (2 * bw);
-            uint8_t* tb = klut + klut_off(bw);
-            for (int i = tid; i < n * 32; i += NT) {
-                int e = i >> 5, bank = i & 31;
-                uint32_t v = (uint32_t)P.k_codebook_f16[s][e & ((1 << bw) - 1)] |
-                             ((uint32_t)P.k_codebook_f16[s][e >> bw] << 16);
-                *(uint32_t*)(tb + e * REPL + bank * 4) = v;
+            const int rep = bw == 4 ? 8 : 32;
+            uint8_t* tb = smem + (bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : KLUT4);
+            for (int i = tid; i < n * rep; i += NT) {
+                int e = i / rep;
+                uint32_t v = (uint32_t)cb_s[s * 16 + (e & ((1 << bw) - 1))] |
+                             ((uint32_t)cb_s[s * 16 + (e >> bw)] << 16);
+                *(uint32_t*)(tb + i * 4) = v;
             }
         } else {
-            uint16_t* tb = (uint16_t*)(smem + KRAW_OFF) + (bw - 5) * 256;
             // every byte value needs a finite entry: the last unit of a segment also
-            // decodes bytes that belong to its neighbour (their products meet a zero query)
+            // decodes bytes of its neighbour (their products meet a zero query)
+            uint16_t* tb = (uint16_t*)(smem + KRAW) + (bw - 5) * 256;
             for (int i = tid; i < 256; i += NT) tb[i] = i < (1 << bw) ? P.k_codebook_f16[s][i] : (uint16_t)0;
         }
     }
-    for (int i = tid; i < (1 << (2 * VBW)) * 32; i += NT) {
-        int e = i >> 5, bank = i & 31;
-        uint32_t v = (uint32_t)P.v_lut_f16[e & ((1 << VBW) - 1)] | ((uint32_t)P.v_lut_f16[e >> VBW] << 16);
-        *(uint32_t*)(vlut + e * REPL + bank * 4) = v;
-    }
-    if (lane < 16) ((uint32_t*)vn_s)[lane] = 0;
-
-    // ---- step table (identical in every lane, lives in scalar registers) -------
-    StepTable st;
-    st.n_steps = 0;
-#pragma unroll
-    for (int m = 0; m < MAX_STEPS; m++) { st.bw[m] = 1; st.seg[m] = 0; st.unit0[m] = 0; st.n_units[m] = 0; }
     {
-        int m = 0;
-        for (int s = 0; s < P.n_seg; s++) {
-            int nu = (P.seg_len[s] + 7) >> 3;
-            for (int u0 = 0; u0 < nu; u0 += 4) {
-#pragma unroll
-                for (int k = 0; k < MAX_STEPS; k++)
-                    if (k == m) { st.bw[k] = P.seg_bw[s]; st.seg[k] = s; st.unit0[k] = u0; st.n_units[k] = nu; }
-                m++;
-            }
+        constexpr int n = 1 << (2 * VBW);
+        constexpr int rep = VBW == 4 ? 8 : 32;
+        for (int i = tid; i < n * rep; i += NT) {
+            int e = i / rep;
+            uint32_t v = (uint32_t)cb_s[BGTQ_MAX_SEGMENTS * 16 + (e & ((1 << VBW) - 1))] |
+                         ((uint32_t)cb_s[BGTQ_MAX_SEGMENTS * 16 + (e >> VBW)] << 16);
+            *(uint32_t*)(vlut + i * 4) = v;
         }
-        st.n_steps = m;
+    }
+    // step m: {unit0 byte offset, bytes per unit, bits per pair (0 = raw bytes), table offset}
+    //         {table shift, table lane mask, norm row | last-of-segment << 8, real units in the step}
+    if (tid < n_steps) {
+        const int* sp = stp_s + 4 + tid * 8;
+        const int bw = sp[3];
+        int4v p0, p1;
+        p0.x = sp[0];
+        p0.y = sp[1];
+        p0.z = sp[2];
+        p0.w = bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : bw == 4 ? KLUT4
+                                                            : KRAW + (bw - 5) * 512;
+        p1.x = bw == 4 ? 5 : 7;
+        p1.y = bw == 4 ? 7 * 4 : 31 * 4;
+        p1.z = sp[4] | (sp[5] ? 256 : 0);
+        p1.w = sp[6];
+        steps_s[2 * tid] = p0;
+        steps_s[2 * tid + 1] = p1;
     }
 
-    // ---- rotated queries as B operands, one per step (zero on padding dims) ----
-    half8 qB[MAX_STEPS];
-#pragma unroll
-    for (int m = 0; m < MAX_STEPS; m++) {
-        half8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (m < st.n_steps && li < gqa) {
-            int s = st.seg[m];
-            int u = st.unit0[m] + lg;
-            const uint16_t* qp = a.q + b * a.q_sb + (h * gqa + li) * a.q_sh + P.seg_start[s] + u * 8;
-            int left = P.seg_len[s] - u * 8;
-#pragma unroll
-            for (int i = 0; i < 8; i++)
-                if (i < left) v[i] = __builtin_bit_cast(_Float16, qp[i]);
-        }
-        qB[m] = v;
+    // ---- init 3: query B operands per step, [step][lane][8 halves] ------------------
+    for (int i = tid; i < n_steps * 64 * 4; i += NT) {
+        int m = i >> 8, l = (i >> 2) & 63, p = i & 3;          // p: pair of halves
+        int d = 8 * (l >> 4) + 2 * p;                          // dim inside the step
+        const int* sp = stp_s + 4 + m * 8;
+        int left = seg_start[sp[4]] + seg_len[sp[4]] - sp[7];   // dims of the segment from this step on
+        const uint16_t* row = q_s + (l & 15) * D + sp[7] + d;
+        uint32_t lo = d < left ? row[0] : 0, hi = d + 1 < left ? row[1] : 0;
+        ((uint32_t*)qop_s)[i] = lo | (hi << 16);
     }
-    // per-lane byte offset of this lane's unit inside a K record, per step
-    int koff[MAX_STEPS];
-#pragma unroll
-    for (int m = 0; m < MAX_STEPS; m++) {
-        int s = st.seg[m];
-        int u = min(st.unit0[m] + lg, max(st.n_units[m] - 1, 0));     // clamp: padding units re-read a real one
-        int ub = st.bw[m] <= 4 ? st.bw[m] : 8;
-        koff[m] = P.seg_pack_off[s] + u * ub;
-    }
-    __syncthreads();
+    __syncthreads();                                        // scratch is dead from here
+    if (lane < MT / 2) ((uint32_t*)vn_s)[lane] = 0;
 
     const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
     const uint16_t* kn_base = a.kn + b * a.kn_sb + h * a.kn_sh;
     const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
     const uint16_t* vn_base = a.vn + b * a.vn_sb + h * a.vn_sh;
-    const int n_seg = P.n_seg;
     const float c2 = a.scale * 1.44269504088896340736f;      // logits go through exp2
-    const uint32_t bank4 = (uint32_t)(lane & 31) * 4;
+    const uint32_t lane4 = (uint32_t)lane * 4;
+    const uint32_t vbank = VBW == 4 ? (lane4 & 28u) : (lane4 & 124u);
+    constexpr int vshift = VBW == 4 ? 5 : 7;
 
     float m_ref = -INFINITY;        // running max of head li, in exp2 units
     float l_part = 0.f;             // this lane's share of the softmax denominator
@@ -188,93 +226,113 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
 #pragma unroll
     for (int e = 0; e < 8; e++) acc[e] = (float4v){0, 0, 0, 0};
 
-    for (int tile = t0 + wave * MT; tile < t1; tile += MW * MT) {
+    TileRegs<KR> kreg;
+    TileRegs<VR> vreg;
+    uint16_t nreg[BGTQ_MAX_SEGMENTS];
+    uint16_t vnreg = 0;
+    auto issue = [&](int tile) {
         const int nt = min(MT, t1 - tile);
-        // ---- stage the tile (wave private) -------------------------------------
-        uint32_t kph = stage_bytes(kp_base + (int64_t)tile * a.kp_st, nt * krow, kt_s, lane);
-        uint32_t vph = stage_bytes(vp_base + (int64_t)tile * a.vp_st, nt * vrow, vt_s, lane);
-        // group norms: fp16 -> fp32, transposed to [segment][token] so that a lane
-        // later fetches the four tokens of its MFMA rows with one 128-bit read
-        if (lane < MT) {
-            const uint16_t* nr = kn_base + (int64_t)(tile + lane) * a.kn_st;
-            for (int s = 0; s < n_seg; s++)
-                kn_s[s * MT + lane] = lane < nt ? bgtq_h2f(nr[s]) : 0.f;
-        }
-        if (lane < MT) ((uint16_t*)vn_s)[lane] = lane < nt ? vn_base[tile + lane] : (uint16_t)0;
+        tile_issue(kreg, kp_base + (int64_t)tile * a.kp_st, nt * krow, lane);
+        tile_issue(vreg, vp_base + (int64_t)tile * a.vp_st, nt * vrow, lane);
+        const uint16_t* nr = kn_base + (int64_t)(tile + lane) * a.kn_st;    // lane = token
+#pragma unroll
+        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) nreg[s] = (s < n_seg && lane < nt) ? nr[s] : (uint16_t)0;
+        vnreg = lane < nt ? vn_base[tile + lane] : (uint16_t)0;
+    };
+    int tile = t0 + wave * MT;
+    if (tile < t1) issue(tile);
+
+    for (; tile < t1; tile += MW * MT) {
+        const int nt = min(MT, t1 - tile);
+        // ---- registers -> LDS (wave private), then start fetching the next tile ------
+        const uint32_t kph = kreg.phase, vph = vreg.phase;
+        tile_commit(kreg, kt_s, lane);
+        tile_commit(vreg, vt_s, lane);
+#pragma unroll
+        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++)          // fp16 -> fp32, [segment][token]
+            if (s < n_seg) kn_s[s * MT + lane] = bgtq_h2f(nreg[s]);
+        vn_s[lane] = vnreg;
+        if (tile + MW * MT < t1) issue(tile + MW * MT);
         // a wave's LDS operations execute in issue order; the clobber keeps the
         // compiler from moving the tile reads above the staging writes
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
 
         // ---- scores ---------------------------------------------------------------
-        // Per segment: MFMA over its unscaled fp16 centroids, then the fp32 group norm
-        // of each token row scales the segment's partial sum.
-        float4v S[2];
+        float4v S[NBLK], dseg[NBLK];
+        uint32_t rowb[NBLK];
 #pragma unroll
-        for (int blk = 0; blk < 2; blk++) {
-            float4v s4 = {0, 0, 0, 0}, dseg = {0, 0, 0, 0};
-            const uint32_t rowb = kph + (uint32_t)(blk * 16 + li) * krow;
+        for (int k = 0; k < NBLK; k++) {
+            S[k] = (float4v){0, 0, 0, 0};
+            dseg[k] = (float4v){0, 0, 0, 0};
+            rowb[k] = kph + (uint32_t)(k * 16 + li) * krow;
+        }
+        for (int m = 0; m < n_steps; m++) {
+            const int4v p0 = steps_s[2 * m], p1 = steps_s[2 * m + 1];
+            const half8 Q = *(const half8*)(qop_s + m * 1024 + lane * 16);
+            const uint32_t off = (uint32_t)p0.x + (uint32_t)min(lg, p1.w - 1) * (uint32_t)p0.y;
+            const int pw = __builtin_amdgcn_readfirstlane(p0.z);
+            if (pw != 0) {
+                const uint32_t lb = (uint32_t)p0.w + (lane4 & (uint32_t)p1.y);
+                const uint32_t sh = (uint32_t)p1.x;
 #pragma unroll
-            for (int m = 0; m < MAX_STEPS; m++) {
-                if (m < st.n_steps) {
-                    const int bw = st.bw[m];
-                    uint32_t o = rowb + (uint32_t)koff[m];
+                for (int k = 0; k < NBLK; k++) {
+                    uint32_t o = rowb[k] + off;
                     uint32_t lo = lds_u32(kt_s, o & ~3u), hi = lds_u32(kt_s, (o & ~3u) + 4);
-                    uint32_t w[4];
-                    if (bw <= 4) {
-                        uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
-                        const uint32_t tboff = bw == 1 ? klut_off(1) : bw == 2 ? klut_off(2)
-                                             : bw == 3 ? klut_off(3) : klut_off(4);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            uint32_t idx = __builtin_amdgcn_ubfe(raw, e * 2 * bw, 2 * bw);
-                            w[e] = lds_u32(klut, tboff + (idx << 7) + bank4);
-                        }
-                    } else {
-                        // raw bytes: 8 single-code look-ups
-                        uint32_t hi2 = lds_u32(kt_s, (o & ~3u) + 8);
-                        uint32_t r0 = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
-                        uint32_t r1 = __builtin_amdgcn_alignbyte(hi2, hi, o & 3u);
-                        const uint16_t* tb = (const uint16_t*)(smem + KRAW_OFF) + (bw - 5) * 256;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            uint32_t r = e < 2 ? r0 : r1;
-                            uint32_t ca = (r >> ((e & 1) * 16)) & 0xFF, cb = (r >> ((e & 1) * 16 + 8)) & 0xFF;
-                            w[e] = (uint32_t)tb[ca] | ((uint32_t)tb[cb] << 16);
-                        }
-                    }
+                    uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
                     half8 A;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        half2v pr = __builtin_bit_cast(half2v, w[e]);
+                        uint32_t idx = __builtin_amdgcn_ubfe(raw, e * pw, pw);
+                        half2v pr = __builtin_bit_cast(half2v, lds_u32(smem, (idx << sh) + lb));
                         A[2 * e] = pr[0];
                         A[2 * e + 1] = pr[1];
                     }
-                    const bool first = (m == 0) || (st.seg[m] != st.seg[m > 0 ? m - 1 : 0]);
-                    const bool last = (m + 1 >= st.n_steps) || (st.seg[m] != st.seg[m + 1 < MAX_STEPS ? m + 1 : m]);
-                    if (first) dseg = (float4v){0, 0, 0, 0};
-                    dseg = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, qB[m], dseg, 0, 0, 0);
-                    if (last) {
-                        const float4v n4 = *(const float4v*)(kn_s + st.seg[m] * MT + blk * 16 + lg * 4);
-                        s4 += dseg * n4;
+                    dseg[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Q, dseg[k], 0, 0, 0);
+                }
+            } else {
+                const uint16_t* tb = (const uint16_t*)(smem + p0.w);
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) {
+                    uint32_t o = rowb[k] + off;
+                    uint32_t lo = lds_u32(kt_s, o & ~3u), hi = lds_u32(kt_s, (o & ~3u) + 4);
+                    uint32_t hi2 = lds_u32(kt_s, (o & ~3u) + 8);
+                    uint32_t r0 = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
+                    uint32_t r1 = __builtin_amdgcn_alignbyte(hi2, hi, o & 3u);
+                    half8 A;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        uint32_t r = e < 4 ? r0 : r1;
+                        A[e] = __builtin_bit_cast(_Float16, tb[(r >> ((e & 3) * 8)) & 0xFF]);
                     }
+                    dseg[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Q, dseg[k], 0, 0, 0);
                 }
             }
-            S[blk] = s4;
+            const int sz = __builtin_amdgcn_readfirstlane(p1.z);
+            if (sz & 256) {       // segment complete: scale by the token rows' group norms
+                const float* nrm = kn_s + (sz & 255) * MT + lg * 4;
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) {
+                    const float4v n4 = *(const float4v*)(nrm + k * 16);
+                    S[k] += dseg[k] * n4;
+                    dseg[k] = (float4v){0, 0, 0, 0};
+                }
+            }
         }
 
-        // ---- online softmax: lane (head li, group lg) holds tokens 4lg+r, 16+4lg+r --
-        float sv[8];
+        // ---- online softmax: lane (head li, group lg) holds tokens 16k + 4lg + r ------
+        float sv[4 * NBLK];
         float mx = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 8; r++) {
+        for (int r = 0; r < 4 * NBLK; r++) {
             int tk = (r >> 2) * 16 + lg * 4 + (r & 3);
             float x = S[r >> 2][r & 3] * c2;
             x = tk < nt ? x : -INFINITY;
             sv[r] = x;
             mx = fmaxf(mx, x);
         }
-        mx = wave_xor_max(wave_xor_max(mx, 16), 32);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_ref, mx);
         if (__builtin_amdgcn_ballot_w64(m_new > m_ref)) {          // wave-uniform: rescale only when needed
             const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -289,56 +347,58 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
             l_part *= alpha;
             m_ref = m_new;
         }
-        // P * v_norm is formed in fp32 and rounded to fp16 once
-        half8 Pm;
-        {
-            const uint2 vlo = *(const uint2*)(vn_s + (lg * 4) * 2);          // tokens 4lg .. 4lg+3
-            const uint2 vhi = *(const uint2*)(vn_s + (16 + lg * 4) * 2);     // tokens 16+4lg ..
-            const uint32_t vnn[4] = {vlo.x, vlo.y, vhi.x, vhi.y};
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                half2v vn2 = __builtin_bit_cast(half2v, vnn[e]);
-                float p0 = __builtin_amdgcn_exp2f(sv[2 * e] - m_ref);
-                float p1 = __builtin_amdgcn_exp2f(sv[2 * e + 1] - m_ref);
-                l_part += p0 + p1;
-                Pm[2 * e] = (_Float16)(p0 * (float)vn2[0]);
-                Pm[2 * e + 1] = (_Float16)(p1 * (float)vn2[1]);
-            }
-        }
 
-        // ---- values: lane (j = li, group lg) decodes unit j of its 8 tokens -----------
-        uint32_t W[8][4];
 #pragma unroll
-        for (int r = 0; r < 8; r++) {
-            const int tk = (r >> 2) * 16 + lg * 4 + (r & 3);
-            uint32_t o = vph + (uint32_t)tk * vrow + (uint32_t)li * VBW;
-            uint32_t lo = lds_u32(vt_s, o & ~3u), hi = lds_u32(vt_s, (o & ~3u) + 4);
-            uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
+        for (int half = 0; half < NBLK / 2; half++) {
+            // P * v_norm is formed in fp32 and rounded to fp16 once
+            half8 Pm;
+            {
+                const uint2 vlo = *(const uint2*)(vn_s + half * 32 + lg * 4);        // tokens 4lg .. 4lg+3
+                const uint2 vhi = *(const uint2*)(vn_s + half * 32 + 16 + lg * 4);   // tokens 16+4lg ..
+                const uint32_t vnn[4] = {vlo.x, vlo.y, vhi.x, vhi.y};
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                uint32_t idx = __builtin_amdgcn_ubfe(raw, e * 2 * VBW, 2 * VBW);
-                W[r][e] = lds_u32(vlut, (idx << 7) + bank4);
+                for (int e = 0; e < 4; e++) {
+                    half2v vn2 = __builtin_bit_cast(half2v, vnn[e]);
+                    float p0 = __builtin_amdgcn_exp2f(sv[half * 8 + 2 * e] - m_ref);
+                    float p1 = __builtin_amdgcn_exp2f(sv[half * 8 + 2 * e + 1] - m_ref);
+                    l_part += p0 + p1;
+                    Pm[2 * e] = (_Float16)(p0 * (float)vn2[0]);
+                    Pm[2 * e + 1] = (_Float16)(p1 * (float)vn2[1]);
+                }
             }
-        }
+            // values: lane (j = li, group lg) decodes unit j of its 8 tokens
+            uint32_t W[8][4];
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            half8 Bv;
-            const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;   // high or low halves
+            for (int r = 0; r < 8; r++) {
+                const int tk = half * 32 + (r >> 2) * 16 + lg * 4 + (r & 3);
+                uint32_t o = vph + (uint32_t)tk * vrow + (uint32_t)li * VBW;
+                uint32_t lo = lds_u32(vt_s, o & ~3u), hi = lds_u32(vt_s, (o & ~3u) + 4);
+                uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
 #pragma unroll
-            for (int p = 0; p < 4; p++) {
-                uint32_t x = __builtin_amdgcn_perm(W[2 * p + 1][e >> 1], W[2 * p][e >> 1], sel);
-                half2v hv = __builtin_bit_cast(half2v, x);
-                Bv[2 * p] = hv[0];
-                Bv[2 * p + 1] = hv[1];
+                for (int e = 0; e < 4; e++) {
+                    uint32_t idx = __builtin_amdgcn_ubfe(raw, e * 2 * VBW, 2 * VBW);
+                    W[r][e] = lds_u32(vlut, (idx << vshift) + vbank);
+                }
             }
-            acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Pm, Bv, acc[e], 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                half8 Bv;
+                const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;   // high or low halves
+#pragma unroll
+                for (int p = 0; p < 4; p++) {
+                    uint32_t x = __builtin_amdgcn_perm(W[2 * p + 1][e >> 1], W[2 * p][e >> 1], sel);
+                    half2v hv = __builtin_bit_cast(half2v, x);
+                    Bv[2 * p] = hv[0];
+                    Bv[2 * p + 1] = hv[1];
+                }
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Pm, Bv, acc[e], 0, 0, 0);
+            }
         }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();     // tile buffers are rewritten next iteration
     }
 
     // ---- merge the four waves ------------------------------------------------------
-    // denominators: sum the lane groups of each head
     float l_tot = l_part;
     l_tot += __shfl_xor(l_tot, 16, 64);
     l_tot += __shfl_xor(l_tot, 32, 64);
@@ -362,7 +422,7 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
 #pragma unroll
         for (int w = 0; w < MW; w++) {
             float mw = mg_m[w * 16 + hq];
-            float f = (mw == -INFINITY) ? 0.f : exp2f(mw - m);
+            float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
             den += f * mg_l[w * 16 + hq];
             num += f * mg_o[(w * 16 + hq) * D + d];
         }
@@ -373,13 +433,11 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
 }
 
 size_t mfma_smem_bytes(int vbw, int krow, int vrow) {
-    size_t kt = (size_t)((MT * krow + 16 + 8 + 15) & ~15);
-    size_t vt = (size_t)((MT * vrow + 16 + 8 + 15) & ~15);
-    size_t kn = (size_t)BGTQ_MAX_SEGMENTS * MT * 4;
-    size_t tables = (size_t)VLUT_OFF + vlut_bytes(vbw);
-    size_t waves = (kt + vt + kn + 64) * MW;
+    size_t kt = (size_t)((MT * krow + 16 + 12 + 15) & ~15);
+    size_t vt = (size_t)((MT * vrow + 16 + 12 + 15) & ~15);
+    size_t wave = kt + vt + (size_t)BGTQ_MAX_SEGMENTS * MT * 4 + MT * 2;
+    size_t need = (size_t)wave_off(vbw) + wave * MW;
     size_t merge = (size_t)(MW * 16 * 2 + MW * 16 * D) * 4;
-    size_t need = tables + waves;
     return need > merge ? need : merge;
 }
 
@@ -404,6 +462,8 @@ int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     if ((a.vp_st & 3) || (a.vp_sb & 3) || (a.vp_sh & 3) || ((uintptr_t)a.vp & 3)) return BGTQ_EUNSUPPORTED;
     if (a.kp_st != a.k_row_width || a.vp_st != a.v_row_width) return BGTQ_EUNSUPPORTED;   // records contiguous
     if (a.vn_st != 1) return BGTQ_EUNSUPPORTED;
+    if (MT * a.k_row_width + 12 > KR * 1024 || MT * a.v_row_width + 12 > VR * 1024) return BGTQ_EUNSUPPORTED;
+    if ((a.q_sb & 1) || (a.q_sh & 1) || ((uintptr_t)a.q & 3)) return BGTQ_EUNSUPPORTED;
     // a bit-packed V record of 128 dims is 16 bytes per bit of code width
     switch (a.v_row_width) {
     case 16: return launch<1>(a, stream);

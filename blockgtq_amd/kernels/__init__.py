@@ -61,6 +61,7 @@ def _plan_from_args(codebook_flat, segments, v_lut, v_rotation, v_bits, device):
     p['v_lut_f16'][:lut.size] = lut
     if v_rotation is not None:
         p['v_rot'] = v_rotation.detach().cpu().float().numpy().reshape(-1)
+    _plan.fill_decode_steps(p)
     return _plan.upload_plans(p.reshape(1), device)
 
 

@@ -12,6 +12,7 @@ HEAD_DIM = 128
 MAX_SEGMENTS = 8
 MAX_CENTROIDS = 256
 LUT_BINS = 256
+MAX_STEPS = 12
 
 K_BITPACKED, K_MIXED = 0, 1
 V_BITPACKED, V_NIBBLE = 0, 1
@@ -35,6 +36,7 @@ PLAN_DTYPE = np.dtype([
     ('v_centroids', '<f4', (16,)), ('v_boundaries', '<f4', (16,)),
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
+    ('n_steps', '<i4'), ('reserved1', '<i4', (3,)), ('step', '<i4', (MAX_STEPS, 8)),
 ], align=True)
 
 
@@ -49,6 +51,24 @@ def segment_bytes(bw: int, length: int) -> int:
     if bw == 4:
         return (length + 1) // 2
     return length
+
+
+def fill_decode_steps(p) -> None:
+    """Derive the MFMA step schedule of the bit-packed K record from the
+    segment table already stored in plan ``p`` (a 0-d structured array)."""
+    m = 0
+    for s in range(int(p['n_seg'])):
+        bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
+        n_units = (ln + 7) // 8
+        unit_bytes = bw if bw <= 4 else 8
+        for u0 in range(0, n_units, 4):
+            if m >= MAX_STEPS:
+                raise ValueError("segment table needs more MFMA steps than the plan holds")
+            p['step'][m] = (int(p['seg_pack_off'][s]) + u0 * unit_bytes, unit_bytes,
+                            2 * bw if bw <= 4 else 0, bw, s, int(u0 + 4 >= n_units),
+                            min(4, n_units - u0), int(p['seg_start'][s]) + u0 * 8)
+            m += 1
+    p['n_steps'] = m
 
 
 def build_head_plan(quantizer) -> np.ndarray:
@@ -113,6 +133,7 @@ def build_head_plan(quantizer) -> np.ndarray:
     p['v_lut_f16'][:nv] = vc.astype(np.float16).view(np.uint16)
     p['v_rot_T'] = q._v_rot_T.detach().cpu().numpy().astype(np.float32).reshape(-1)
     p['v_rot'] = q._v_rot.detach().cpu().numpy().astype(np.float32).reshape(-1)
+    fill_decode_steps(p)
     return p.reshape(1)
 
 

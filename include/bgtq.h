@@ -28,6 +28,7 @@ extern "C" {
 #define BGTQ_LUT_BINS      256
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
+#define BGTQ_MAX_STEPS     12    /* MFMA steps of one K record, see bgtq_head_plan.step */
 
 /* error codes (negative); positive return values are hipError_t */
 #define BGTQ_OK            0
@@ -84,6 +85,17 @@ typedef struct bgtq_head_plan {
     uint16_t v_lut_f16[16];
     float    v_rot_T[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];  /* encode: y = vhat @ v_rot_T */
     float    v_rot[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];    /* decode: out = acc @ v_rot */
+    /*
+     * Decode schedule of the bit-packed K record.  A "unit" is 8 consecutive
+     * dims of one segment; a step covers up to 4 units of ONE segment (one
+     * 16x16x32 MFMA).  step[m] = { byte offset of the step's first unit in the
+     * record, bytes per unit (bw, or 8 for raw-byte segments), bits per code
+     * pair (2*bw, 0 for raw bytes), bw, segment index, 1 if last step of its
+     * segment, real units in the step (1..4), first dim of the step }.
+     */
+    int32_t  n_steps;
+    int32_t  reserved1[3];
+    int32_t  step[BGTQ_MAX_STEPS][8];
 } bgtq_head_plan;
 
 /* sizeof(bgtq_head_plan) as the library was compiled; the host mirror checks it. */
