@@ -377,11 +377,12 @@ size_t bgtq_workspace_bytes(int B, int n_q, int n_splits) {
 }
 
 int bgtq_default_splits(int B, int n_kv, int max_T) {
-    // Enough partitions to put several work-groups on each of the 256 CUs, but
-    // never fewer than 256 tokens per partition.
+    // One work-group per partition and the fast kernel keeps a whole CU busy with
+    // one work-group, so aim for one partition per CU (256 of them), but never
+    // fewer than 128 tokens per partition.
     if (B <= 0 || n_kv <= 0 || max_T <= 0) return 1;
-    int by_tokens = (max_T + 255) / 256;
-    int want = (1024 + B * n_kv - 1) / (B * n_kv);
+    int by_tokens = (max_T + 127) / 128;
+    int want = (256 + B * n_kv - 1) / (B * n_kv);
     int s = want < by_tokens ? want : by_tokens;
     if (s < 1) s = 1;
     if (s > BGTQ_MAX_SPLITS) s = BGTQ_MAX_SPLITS;

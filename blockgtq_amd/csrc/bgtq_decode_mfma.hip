@@ -1,8 +1,15 @@
 // MFMA decode attention over bit-packed K and V records (gfx950).
 //
-// One work-group of 4 waves owns one partition of one (batch row, KV head);
-// every wave walks its own 64-token tiles with a private online softmax and the
-// four results are merged through LDS at the end.
+// One work-group of up to 8 waves owns one partition of one (batch row, KV
+// head); every wave walks its own 64-token tiles with a private online softmax
+// and the results are merged through LDS at the end.
+//
+// Data movement.  A tile of packed records is one contiguous byte range of the
+// cache.  It goes from HBM straight into LDS with global_load_lds_dwordx4
+// (aligned 16-byte pieces, the 16-byte phase of the source is kept), into one of
+// two buffers per wave, one tile ahead of the tile being processed.  The raw
+// fp16 norms of the tile travel the same way.  Nothing on the streaming path
+// passes through vector registers.
 //
 // Dequantisation is table driven.  A "unit" is 8 consecutive codes of one
 // token (bw bytes of the record).  For every bit width <= 4 the work-group
@@ -15,31 +22,37 @@
 // QK^T:  v_mfma_f32_16x16x32_f16, A = dequantised K (row = token, lane group g
 //        supplies unit 4m+g of step m; a step never mixes segments, so field
 //        width and table are the same for the whole wave), B = rotated queries
-//        laid out per step in LDS (zero on padding dims), D[token][head].  Each
-//        segment accumulates on its own and is scaled by the fp32 group norm of
-//        its token row when the segment ends.
+//        stored per unit in LDS (zero on padding dims), D[token][head].  Each
+//        segment accumulates on its own and is scaled by the fp16 group norm of
+//        its token row, in fp32, when the segment ends.
 // PV:    the D layout of two 16-token blocks is exactly the A layout of a
 //        K=32 step (row = head, lane group g holds 8 tokens), so P never leaves
 //        its lane; B = dequantised V where lane (j, g) decodes unit j of its 8
 //        tokens and hands dim 8j+e to MFMA e.  The V norm is folded into P in
 //        fp32 before P is rounded to fp16.
+// Softmax: exponentials are taken relative to a per-head reference that is kept
+//        above every score seen so far.  It is only moved (to the new maximum
+//        plus a headroom of 4 in log2 units) when a score of the tile exceeds it;
+//        otherwise the tile needs no cross-lane traffic at all.
 #include "bgtq_decode.h"
 
 namespace {
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
-typedef int int4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
 constexpr int D = BGTQ_D;
-constexpr int MW = 4;              // waves per work-group
-constexpr int NT = MW * 64;
 constexpr int MT = 64;             // tokens per wave tile = 4 MFMA row blocks
 constexpr int NBLK = MT / 16;
 constexpr int MAX_STEPS = BGTQ_MAX_STEPS;
-constexpr int KR = 6;              // 128-bit prefetch registers per lane for a K tile (row <= 95 B)
-constexpr int VR = 5;              // same for a V tile (row <= 64 B)
+constexpr int MAX_WAVES = 8;
+constexpr int MAX_KN = 8;          // norm columns per token row the staging area can hold
+constexpr int LDS_LIMIT = 160 * 1024;
+constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
 constexpr int KLUT1 = 0;                       // 4 entries   x 128 B
@@ -48,59 +61,170 @@ constexpr int KLUT3 = KLUT2 + 16 * 128;        // 64 entries  x 128 B
 constexpr int KLUT4 = KLUT3 + 64 * 128;        // 256 entries x 32 B
 constexpr int KRAW = KLUT4 + 256 * 32;         // 4 tables x 256 fp16 (bw 5..8)
 constexpr int VLUT = KRAW + 4 * 512;
+constexpr int QROW = 400;                      // one head: zero unit + up to 24 units x 16 B
 __host__ __device__ constexpr int vlut_bytes(int vbw) { return vbw == 4 ? 256 * 32 : (1 << (2 * vbw)) * 128; }
-__host__ __device__ constexpr int steps_off(int vbw) { return VLUT + vlut_bytes(vbw); }   // MAX_STEPS x 32 B
-__host__ __device__ constexpr int qop_off(int vbw) { return steps_off(vbw) + MAX_STEPS * 32; }  // MAX_STEPS x 1 KB
-__host__ __device__ constexpr int wave_off(int vbw) { return qop_off(vbw) + MAX_STEPS * 1024; }
+__host__ __device__ constexpr int steptab_off(int vbw) { return VLUT + vlut_bytes(vbw); }   // [step][lane group] x 32 B
+__host__ __device__ constexpr int qpad_off(int vbw) { return steptab_off(vbw) + MAX_STEPS * 4 * 32; }
+__host__ __device__ constexpr int waves_off(int vbw) { return qpad_off(vbw) + 16 * QROW; }
+constexpr int WAVE_NORM_BYTES = BGTQ_MAX_SEGMENTS * MT * 2 + MT * 4;   // fp16 K norms [seg][token], fp32 V norms
+constexpr int INIT_SCRATCH = 768 + 4096 + 16 * D * 2;
+
+struct TileLayout {
+    int kt, vt, knr, vnr, kbuf;    // bytes of the K, V, K-norm, V-norm areas; K + both norm areas
+};
+__host__ __device__ inline TileLayout tile_layout(int krow, int vrow, int kn_st) {
+    TileLayout t;
+    t.kt = (MT * krow + 32 + 15) & ~15;
+    t.vt = (MT * vrow + 32 + 15) & ~15;
+    t.knr = (MT * kn_st * 2 + 16 + 15) & ~15;
+    t.vnr = MT * 2 + 16;
+    t.kbuf = t.kt + t.knr + t.vnr;
+    return t;
+}
 
 __device__ inline uint32_t lds_u32(const uint8_t* base, uint32_t off) {
     return *(const uint32_t*)(base + off);
 }
 
-// A tile of packed records is one contiguous byte range.  It is fetched with
-// aligned 128-bit loads (the 16-byte phase of the source is kept in LDS), first
-// into registers while the previous tile is being processed, then into LDS.
-template <int NR>
-struct TileRegs {
-    uint4 r[NR];
-    uint32_t phase;
-    int total;      // phase + valid bytes
-};
+// 16 bytes per lane from sbase + voff + IMM into LDS at lds_addr + lane * 16 + IMM.
+template <int IMM>
+__device__ __forceinline__ void dma16(uint32_t voff, const uint8_t* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3\n"
+                 :: "v"(voff), "s"(sbase), "s"(lds_addr), "n"(IMM) : "memory", "m0");
+}
 
-template <int NR>
-__device__ inline void tile_issue(TileRegs<NR>& t, const uint8_t* src, int nbytes, int lane) {
-    t.phase = (uint32_t)((uintptr_t)src & 15);
-    t.total = (int)t.phase + nbytes;
-    const uint8_t* al = src - t.phase;
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
+    uint64_t v = (uint64_t)(uintptr_t)p;
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Copies the aligned 16-byte pieces of [src_al, src_al + total) to LDS.  Pieces
+// are aligned, so a piece that holds at least one wanted byte never crosses into
+// a page the range itself does not touch.  Exactly dma_count(total) load
+// instructions are issued (lane 0 takes part in every one of them).
+__device__ __forceinline__ int dma_count(int total) { return (total + 1023) >> 10; }
+
+template <int NCH>
+__device__ __forceinline__ void dma_region(const uint8_t* src_al, uint32_t lds_addr, int total, uint32_t voff) {
+    src_al = uniform_ptr(src_al);
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
 #pragma unroll
-    for (int i = 0; i < NR; i++) {
-        const int off = lane * 16 + i * 1024;
-        uint4 v = {0, 0, 0, 0};
-        if (off + 16 <= t.total) {
-            v = *(const uint4*)(al + off);
-        } else if (off < t.total) {            // last, partial chunk: never read past the tile
-            const uint32_t* w = (const uint32_t*)(al + off);
-            v.x = w[0];
-            if (off + 8 <= t.total) v.y = w[1];
-            if (off + 12 <= t.total) v.z = w[2];
+    for (int c = 0; c < NCH; c++) {
+        if (c * 1024 < total) {
+            if ((int)voff + c * 1024 < total) {
+                const uint8_t* sb = src_al + (c >> 2) * 4096;
+                const uint32_t la = lds_addr + (c >> 2) * 4096;
+                switch (c & 3) {
+                case 0: dma16<0>(voff, sb, la); break;
+                case 1: dma16<1024>(voff, sb, la); break;
+                case 2: dma16<2048>(voff, sb, la); break;
+                default: dma16<3072>(voff, sb, la); break;
+                }
+            }
         }
-        t.r[i] = v;
     }
 }
 
-template <int NR>
-__device__ inline void tile_commit(const TileRegs<NR>& t, uint8_t* dst, int lane) {
-#pragma unroll
-    for (int i = 0; i < NR; i++) {
-        const int off = lane * 16 + i * 1024;
-        if (off < t.total) *(uint4*)(dst + off) = t.r[i];
+// Waits until at most n of the loads issued so far are still in flight.
+__device__ __forceinline__ void wait_loads(int n) {
+    switch (n) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+    case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
     }
 }
+
+// U consecutive packed steps, straight line.  Per (step, lane group) the table
+// holds {aligned row offset, byte shift, pair table, bank mask} and
+// {bits per pair, log2 entry stride, norm row offset, query unit offset}.
+// Every step starts from a zero accumulator and is scaled by the fp16 group norm
+// of its token rows in fp32, so segments never mix before the norm is applied.
+template <int U>
+__device__ __forceinline__ void k_packed_steps(float4v (&S)[NBLK], const uint8_t* smem, const uint4* st,
+                                               const uint8_t* qrow, uint32_t kbase, uint32_t kstride,
+                                               uint32_t lane4, const uint8_t* nrm) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint4 e0 = st[u * 8], e1 = st[u * 8 + 1];
+        const half8 Q = *(const half8*)(qrow + e1.w);
+        const uint32_t oa = kbase + e0.x;
+        const uint32_t lb = (lane4 & e0.w) | e0.z;
+        const uint32_t pw = e1.x, pw2 = pw * 2, pw3 = pw * 3, tsh = e1.y;
+#pragma unroll
+        for (int k = 0; k < NBLK; k++) {
+            const uint32_t ad = oa + k * kstride;
+            const uint32_t lo = lds_u32(smem, ad), hi = lds_u32(smem, ad + 4);
+            const uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, e0.y);
+            const uint32_t i0 = __builtin_amdgcn_ubfe(raw, 0, pw), i1 = __builtin_amdgcn_ubfe(raw, pw, pw);
+            const uint32_t i2 = __builtin_amdgcn_ubfe(raw, pw2, pw), i3 = __builtin_amdgcn_ubfe(raw, pw3, pw);
+            const uint4 w = {lds_u32(smem, (i0 << tsh) + lb), lds_u32(smem, (i1 << tsh) + lb),
+                             lds_u32(smem, (i2 << tsh) + lb), lds_u32(smem, (i3 << tsh) + lb)};
+            const float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, w), Q,
+                                                                     (float4v){0, 0, 0, 0}, 0, 0, 0);
+            const half4v n4 = *(const half4v*)(nrm + e1.z + k * 32);
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[r], d[r], S[k][r]);
+        }
+    }
+}
+
+// One step of raw byte codes (bw 5..8): one table read per code.
+__device__ __forceinline__ void k_raw_step(float4v (&S)[NBLK], const uint8_t* smem, const uint4* st,
+                                           const uint8_t* qrow, uint32_t kbase, uint32_t kstride,
+                                           const uint8_t* nrm) {
+    const uint4 e0 = st[0], e1 = st[1];
+    const half8 Q = *(const half8*)(qrow + e1.w);
+    const uint32_t oa = kbase + e0.x;
+#pragma unroll
+    for (int k = 0; k < NBLK; k++) {
+        const uint32_t ad = oa + k * kstride;
+        const uint32_t lo = lds_u32(smem, ad), hi = lds_u32(smem, ad + 4), hi2 = lds_u32(smem, ad + 8);
+        const uint32_t r0 = __builtin_amdgcn_alignbyte(hi, lo, e0.y);
+        const uint32_t r1 = __builtin_amdgcn_alignbyte(hi2, hi, e0.y);
+        half8 A;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t r = e < 4 ? r0 : r1;
+            const uint32_t byte = (r >> ((e & 3) * 8)) & 0xFF;
+            A[e] = __builtin_bit_cast(_Float16, *(const uint16_t*)(smem + e0.z + byte * 2));
+        }
+        const float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Q, (float4v){0, 0, 0, 0}, 0, 0, 0);
+        const half4v n4 = *(const half4v*)(nrm + e1.z + k * 32);
+#pragma unroll
+        for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[r], d[r], S[k][r]);
+    }
+}
+
+#ifdef BGTQ_TRACE
+__device__ unsigned long long* g_trace;
+#define TRACE(slot)                                                                              \
+    do {                                                                                         \
+        if (lane == 0 && (slot) < 64)                                                            \
+            g_trace[(((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + wave) * 64 + (slot)] = \
+                __builtin_readcyclecounter();                                                    \
+    } while (0)
+#else
+#define TRACE(slot) do {} while (0)
+#endif
 
 template <int VBW>
-__global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nw = blockDim.x >> 6, nthr = blockDim.x;
     const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const bgtq_head_plan& P = a.plans[h];
     const int gqa = a.gqa;
@@ -110,231 +234,232 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
     int chunk = (T + a.n_splits - 1) / a.n_splits;
     chunk = (chunk + MT - 1) / MT * MT;
     const int t0 = min(c * chunk, T), t1 = min(t0 + chunk, T);
+    TRACE(0);
 
     // ---- LDS carve-up --------------------------------------------------------
-    const int krow = a.k_row_width, vrow = a.v_row_width;
-    const int kt_bytes = (MT * krow + 16 + 12 + 15) & ~15;
-    const int vt_bytes = (MT * vrow + 16 + 12 + 15) & ~15;
-    constexpr int kn_bytes = BGTQ_MAX_SEGMENTS * MT * 4;  // fp32 norms, [segment][token]
-    const int wave_bytes = kt_bytes + vt_bytes + kn_bytes + MT * 2;
+    const int krow = a.k_row_width;
+    constexpr int vrow = 16 * VBW;
+    const int kn_st = (int)a.kn_st;
+    const TileLayout tl = tile_layout(krow, vrow, kn_st);
     uint8_t* vlut = smem + VLUT;
-    int4v* steps_s = (int4v*)(smem + steps_off(VBW));
-    uint8_t* qop_s = smem + qop_off(VBW);
-    uint8_t* wbuf0 = smem + wave_off(VBW);
-    uint8_t* kt_s = wbuf0 + wave * wave_bytes;
-    uint8_t* vt_s = kt_s + kt_bytes;
-    float* kn_s = (float*)(vt_s + vt_bytes);
-    uint16_t* vn_s = (uint16_t*)((uint8_t*)kn_s + kn_bytes);
+    uint4* steptab = (uint4*)(smem + steptab_off(VBW));
+    uint8_t* qpad = smem + qpad_off(VBW);
+    const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+    const uint32_t kbufs_off = waves_off(VBW);                                   // [2][nw] K + norm buffers
+    const uint32_t vbuf_off = kbufs_off + 2 * nw * tl.kbuf + wave * tl.vt;        // [nw] V buffers
+    const uint32_t norm_off = kbufs_off + nw * (2 * tl.kbuf + tl.vt) + wave * WAVE_NORM_BYTES;
+    uint8_t* kn_h = smem + norm_off;                                 // fp16 [segment][token]
+    float* vn_f = (float*)(kn_h + BGTQ_MAX_SEGMENTS * MT * 2);       // fp32 [token]
+    uint8_t* scratch = smem + kbufs_off + nw * tl.kbuf;              // everything past the first K buffers is idle during init
+
+    // ---- streaming sources: 16-byte aligned bases and phases (constant per tile) ----
+    const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
+    const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
+    const uint8_t* kn_base = (const uint8_t*)(a.kn + b * a.kn_sb + h * a.kn_sh);
+    const uint8_t* vn_base = (const uint8_t*)(a.vn + b * a.vn_sb + h * a.vn_sh);
+    const uint32_t kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
+    const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
+    const uint32_t voff = (uint32_t)lane * 16;
+    // K records and both norm arrays of a tile go to K buffer `which`; returns the loads issued
+    auto issue_k = [&](int tile, int which) -> int {
+        const int nt = min(MT, t1 - tile);
+        const uint32_t buf = smem_lds + kbufs_off + (which * nw + wave) * tl.kbuf;
+        const int bk = (int)kph + nt * krow, bn = (int)knph + nt * kn_st * 2, bv = (int)vnph + nt * 2;
+        dma_region<9>(kp_base - kph + (int64_t)tile * krow, buf, bk, voff);
+        dma_region<2>(kn_base - knph + (int64_t)tile * kn_st * 2, buf + tl.kt, bn, voff);
+        dma_region<1>(vn_base - vnph + (int64_t)tile * 2, buf + tl.kt + tl.knr, bv, voff);
+        return dma_count(bk) + dma_count(bn) + dma_count(bv);
+    };
+    auto issue_v = [&](int tile) -> int {
+        const int nt = min(MT, t1 - tile);
+        const int bv = (int)vph + nt * vrow;
+        dma_region<5>(vp_base - vph + (int64_t)tile * vrow, smem_lds + vbuf_off, bv, voff);
+        return dma_count(bv);
+    };
+    const int step_tiles = nw * MT;
+    int tile = t0 + wave * MT;
+    int v_loads = 0;                 // loads of the V tile issued after the current K tile
+    if (tile < t1) issue_k(tile, 0);
+    TRACE(1);
 
     // ---- init 1: plan header, step schedule, codebooks and queries into LDS scratch --
-    // (scratch lives in the tile buffers, which are idle until the main loop)
-    int* hdr_s = (int*)wbuf0;                             // first 56 ints of the plan
-    uint16_t* cb_s = (uint16_t*)(wbuf0 + 256);            // [8][16] K codebooks + [16] V
-    int* stp_s = (int*)(wbuf0 + 576);                     // n_steps, 3 pad, step[12][8]
-    uint16_t* q_s = (uint16_t*)(wbuf0 + 1024);            // [16][128] rotated queries
-    if (tid < 56) hdr_s[tid] = ((const int*)&P)[tid];
-    if (tid >= 64 && tid < 64 + 4 + MAX_STEPS * 8) stp_s[tid - 64] = (&P.n_steps)[tid - 64];
-    for (int i = tid; i < BGTQ_MAX_SEGMENTS * 16; i += NT) cb_s[i] = P.k_codebook_f16[i >> 4][i & 15];
-    if (tid < 16) cb_s[BGTQ_MAX_SEGMENTS * 16 + tid] = P.v_lut_f16[tid];
-    for (int i = tid; i < 16 * D / 2; i += NT) {
+    int* hdr_s = (int*)scratch;                           // first 56 ints of the plan
+    int* stp_s = (int*)(scratch + 256);                   // n_steps, 3 pad, step[12][8]
+    uint16_t* vcb_s = (uint16_t*)(scratch + 704);         // [16] V centroids
+    uint16_t* cb_s = (uint16_t*)(scratch + 768);          // [8][256] K codebooks
+    uint16_t* q_s = (uint16_t*)(scratch + 768 + 4096);    // [16][128] rotated queries
+    for (int i = tid; i < 56; i += nthr) hdr_s[i] = ((const int*)&P)[i];
+    for (int i = tid; i < 4 + MAX_STEPS * 8; i += nthr) stp_s[i] = (&P.n_steps)[i];
+    for (int i = tid; i < 8; i += nthr) ((uint32_t*)vcb_s)[i] = ((const uint32_t*)P.v_lut_f16)[i];
+    for (int i = tid; i < BGTQ_MAX_SEGMENTS * 128; i += nthr)
+        ((uint32_t*)cb_s)[i] = ((const uint32_t*)&P.k_codebook_f16[0][0])[i];
+    for (int i = tid; i < 16 * D / 2; i += nthr) {
         int hq = i / (D / 2), d2 = i - hq * (D / 2);
         uint32_t v = 0;
         if (hq < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + hq) * a.q_sh + d2 * 2);
         ((uint32_t*)q_s)[i] = v;
     }
     __syncthreads();
-    const int n_seg = hdr_s[0];
+    TRACE(2);
+    const int n_seg = min(hdr_s[0], BGTQ_MAX_SEGMENTS);
     const int* seg_bw = hdr_s + 8;
     const int* seg_start = hdr_s + 16;
     const int* seg_len = hdr_s + 24;
     const int n_steps = min(stp_s[0], MAX_STEPS);
+    int n_packed = 0;                                      // raw-byte steps (bw >= 5) come last
+    for (int m = 0; m < n_steps; m++) n_packed += stp_s[4 + m * 8 + 2] != 0;
 
-    // ---- init 2: pair tables, step table -------------------------------------------
+    // ---- init 2: pair tables ---------------------------------------------------------
     for (int s = 0; s < n_seg; s++) {
         const int bw = seg_bw[s];
         if (bw <= 4) {
             const int n = 1 << (2 * bw);
-            const int rep = bw == 4 ? 8 : 32;
+            const int rsh = bw == 4 ? 3 : 5;               // log2 of the replication factor
             uint8_t* tb = smem + (bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : KLUT4);
-            for (int i = tid; i < n * rep; i += NT) {
-                int e = i / rep;
-                uint32_t v = (uint32_t)cb_s[s * 16 + (e & ((1 << bw) - 1))] |
-                             ((uint32_t)cb_s[s * 16 + (e >> bw)] << 16);
+            for (int i = tid; i < (n << rsh); i += nthr) {
+                int e = i >> rsh;
+                uint32_t v = (uint32_t)cb_s[s * 256 + (e & ((1 << bw) - 1))] |
+                             ((uint32_t)cb_s[s * 256 + (e >> bw)] << 16);
                 *(uint32_t*)(tb + i * 4) = v;
             }
         } else {
             // every byte value needs a finite entry: the last unit of a segment also
             // decodes bytes of its neighbour (their products meet a zero query)
             uint16_t* tb = (uint16_t*)(smem + KRAW) + (bw - 5) * 256;
-            for (int i = tid; i < 256; i += NT) tb[i] = i < (1 << bw) ? P.k_codebook_f16[s][i] : (uint16_t)0;
+            for (int i = tid; i < 256; i += nthr) tb[i] = i < (1 << bw) ? cb_s[s * 256 + i] : (uint16_t)0;
         }
     }
     {
         constexpr int n = 1 << (2 * VBW);
-        constexpr int rep = VBW == 4 ? 8 : 32;
-        for (int i = tid; i < n * rep; i += NT) {
-            int e = i / rep;
-            uint32_t v = (uint32_t)cb_s[BGTQ_MAX_SEGMENTS * 16 + (e & ((1 << VBW) - 1))] |
-                         ((uint32_t)cb_s[BGTQ_MAX_SEGMENTS * 16 + (e >> VBW)] << 16);
+        constexpr int rsh = VBW == 4 ? 3 : 5;
+        for (int i = tid; i < (n << rsh); i += nthr) {
+            int e = i >> rsh;
+            uint32_t v = (uint32_t)vcb_s[e & ((1 << VBW) - 1)] | ((uint32_t)vcb_s[e >> VBW] << 16);
             *(uint32_t*)(vlut + i * 4) = v;
         }
     }
-    // step m: {unit0 byte offset, bytes per unit, bits per pair (0 = raw bytes), table offset}
-    //         {table shift, table lane mask, norm row | last-of-segment << 8, real units in the step}
-    if (tid < n_steps) {
-        const int* sp = stp_s + 4 + tid * 8;
-        const int bw = sp[3];
-        int4v p0, p1;
-        p0.x = sp[0];
-        p0.y = sp[1];
-        p0.z = sp[2];
-        p0.w = bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : bw == 4 ? KLUT4
-                                                            : KRAW + (bw - 5) * 512;
-        p1.x = bw == 4 ? 5 : 7;
-        p1.y = bw == 4 ? 7 * 4 : 31 * 4;
-        p1.z = sp[4] | (sp[5] ? 256 : 0);
-        p1.w = sp[6];
-        steps_s[2 * tid] = p0;
-        steps_s[2 * tid + 1] = p1;
-    }
-
-    // ---- init 3: query B operands per step, [step][lane][8 halves] ------------------
-    for (int i = tid; i < n_steps * 64 * 4; i += NT) {
-        int m = i >> 8, l = (i >> 2) & 63, p = i & 3;          // p: pair of halves
-        int d = 8 * (l >> 4) + 2 * p;                          // dim inside the step
+    // ---- init 3: per (step, lane group) parameters and the padded query units -------------
+    // plan step m: {byte offset of unit 0, bytes per unit, bits per pair (0 = raw bytes), bw,
+    //               segment, last-of-segment, real units, first dim}
+    for (int i = tid; i < n_steps * 4; i += nthr) {
+        const int m = i >> 2, g = i & 3;
         const int* sp = stp_s + 4 + m * 8;
-        int left = seg_start[sp[4]] + seg_len[sp[4]] - sp[7];   // dims of the segment from this step on
-        const uint16_t* row = q_s + (l & 15) * D + sp[7] + d;
-        uint32_t lo = d < left ? row[0] : 0, hi = d + 1 < left ? row[1] : 0;
-        ((uint32_t*)qop_s)[i] = lo | (hi << 16);
+        const int bw = sp[3], nu = sp[6];
+        int ub = 0;
+        for (int j = 0; j < m; j++) ub += stp_s[4 + j * 8 + 6];
+        const uint32_t o = kph + (uint32_t)sp[0] + (uint32_t)min(g, nu - 1) * (uint32_t)sp[1];
+        uint4 e0, e1;
+        e0.x = o & ~3u;                                              // aligned byte offset in the row
+        e0.y = o & 3u;                                               // byte shift of the unit
+        e0.z = bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : bw == 4 ? KLUT4
+                                                            : KRAW + (bw - 5) * 512;
+        e0.w = bw == 4 ? 7 * 4 : bw <= 3 ? 31 * 4 : 0;               // bank replica mask
+        e1.x = (uint32_t)sp[2];
+        e1.y = bw == 4 ? 5 : 7;                                      // log2 of the table entry stride
+        e1.z = (uint32_t)sp[4] * (MT * 2);                           // norm row of the segment
+        e1.w = g < nu ? (uint32_t)(1 + ub + g) * 16 : 0;             // byte offset of the query unit
+        steptab[i * 2] = e0;
+        steptab[i * 2 + 1] = e1;
+    }
+    if (tid < 64) ((uint32_t*)qpad)[(tid >> 2) * (QROW / 4) + (tid & 3)] = 0;      // unit 0 is all zero (one wave is enough)
+    for (int i = tid; i < n_steps * 256; i += nthr) {
+        const int p = i & 3, hd = (i >> 2) & 15, g = (i >> 6) & 3, m = i >> 8;
+        const int* sp = stp_s + 4 + m * 8;
+        if (g < sp[6]) {
+            int ub = 0;
+            for (int j = 0; j < m; j++) ub += stp_s[4 + j * 8 + 6];
+            const int uid = 1 + ub + g;
+            const int dd = sp[7] + 8 * g + 2 * p;
+            const int end = seg_start[sp[4]] + seg_len[sp[4]];
+            const uint16_t* row = q_s + hd * D;
+            uint32_t lo = dd < end ? row[dd] : 0, hi = dd + 1 < end ? row[dd + 1] : 0;
+            if (uid < QROW / 16) ((uint32_t*)qpad)[hd * (QROW / 4) + uid * 4 + p] = lo | (hi << 16);
+        }
     }
     __syncthreads();                                        // scratch is dead from here
-    if (lane < MT / 2) ((uint32_t*)vn_s)[lane] = 0;
+    if (tile < t1) v_loads = issue_v(tile);
+    TRACE(4);
+#ifdef BGTQ_TRACE
+    int trace_j = 0;
+#endif
 
-    const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
-    const uint16_t* kn_base = a.kn + b * a.kn_sb + h * a.kn_sh;
-    const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
-    const uint16_t* vn_base = a.vn + b * a.vn_sb + h * a.vn_sh;
     const float c2 = a.scale * 1.44269504088896340736f;      // logits go through exp2
     const uint32_t lane4 = (uint32_t)lane * 4;
     const uint32_t vbank = VBW == 4 ? (lane4 & 28u) : (lane4 & 124u);
     constexpr int vshift = VBW == 4 ? 5 : 7;
+    const uint32_t rowoff = (uint32_t)li * krow;
+    const uint32_t kstride = 16u * krow;
+    const uint32_t vc = vph + (uint32_t)li * VBW;
+    const uint32_t vbase = vbuf_off + (vc & ~3u) + (uint32_t)lg * 4 * vrow, v_sh = vc & 3u;
+    const uint4* stl = steptab + lg * 2;
+    const uint8_t* qrow = qpad + li * QROW;
+    const uint8_t* nrm = kn_h + lg * 8;
 
-    float m_ref = -INFINITY;        // running max of head li, in exp2 units
+    float m_ref = -INFINITY;        // reference of head li, in exp2 units; never below a score seen
     float l_part = 0.f;             // this lane's share of the softmax denominator
     float4v acc[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) acc[e] = (float4v){0, 0, 0, 0};
 
-    TileRegs<KR> kreg;
-    TileRegs<VR> vreg;
-    uint16_t nreg[BGTQ_MAX_SEGMENTS];
-    uint16_t vnreg = 0;
-    auto issue = [&](int tile) {
+    int which = 0;
+    for (; tile < t1; tile += step_tiles, which ^= 1) {
         const int nt = min(MT, t1 - tile);
-        tile_issue(kreg, kp_base + (int64_t)tile * a.kp_st, nt * krow, lane);
-        tile_issue(vreg, vp_base + (int64_t)tile * a.vp_st, nt * vrow, lane);
-        const uint16_t* nr = kn_base + (int64_t)(tile + lane) * a.kn_st;    // lane = token
+        const bool more = tile + step_tiles < t1;
+        const uint32_t kbuf = kbufs_off + (which * nw + wave) * tl.kbuf;
+        TRACE(8 + trace_j * 8 + 0);
+        wait_loads(v_loads);                                 // K records and norms of this tile are in LDS
+        __builtin_amdgcn_wave_barrier();
+        TRACE(8 + trace_j * 8 + 1);
+        // ---- norms of the tile: lane = token; read raw, start the next K tile, then store
+        //      them as fp16 [segment][token] and fp32 V norms -------------------------------------
+        uint16_t nraw[BGTQ_MAX_SEGMENTS];
+        {
+            const uint8_t* kraw = smem + kbuf + tl.kt + knph + (uint32_t)lane * kn_st * 2;
 #pragma unroll
-        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) nreg[s] = (s < n_seg && lane < nt) ? nr[s] : (uint16_t)0;
-        vnreg = lane < nt ? vn_base[tile + lane] : (uint16_t)0;
-    };
-    int tile = t0 + wave * MT;
-    if (tile < t1) issue(tile);
-
-    for (; tile < t1; tile += MW * MT) {
-        const int nt = min(MT, t1 - tile);
-        // ---- registers -> LDS (wave private), then start fetching the next tile ------
-        const uint32_t kph = kreg.phase, vph = vreg.phase;
-        tile_commit(kreg, kt_s, lane);
-        tile_commit(vreg, vt_s, lane);
+            for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++)
+                if (s < n_seg) nraw[s] = *(const uint16_t*)(kraw + s * 2);
+        }
+        const uint16_t vraw = *(const uint16_t*)(smem + kbuf + tl.kt + tl.knr + vnph + lane * 2);
+        int k_loads = 0;
+        if (more) k_loads = issue_k(tile + step_tiles, which ^ 1);
 #pragma unroll
-        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++)          // fp16 -> fp32, [segment][token]
-            if (s < n_seg) kn_s[s * MT + lane] = bgtq_h2f(nreg[s]);
-        vn_s[lane] = vnreg;
-        if (tile + MW * MT < t1) issue(tile + MW * MT);
-        // a wave's LDS operations execute in issue order; the clobber keeps the
-        // compiler from moving the tile reads above the staging writes
+        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++)
+            if (s < n_seg) *(uint16_t*)(kn_h + (s * MT + lane) * 2) = nraw[s];
+        vn_f[lane] = lane < nt ? bgtq_h2f(vraw) : 0.f;
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
+        TRACE(8 + trace_j * 8 + 2);
 
         // ---- scores ---------------------------------------------------------------
-        float4v S[NBLK], dseg[NBLK];
-        uint32_t rowb[NBLK];
+        float4v S[NBLK];
 #pragma unroll
-        for (int k = 0; k < NBLK; k++) {
-            S[k] = (float4v){0, 0, 0, 0};
-            dseg[k] = (float4v){0, 0, 0, 0};
-            rowb[k] = kph + (uint32_t)(k * 16 + li) * krow;
+        for (int k = 0; k < NBLK; k++) S[k] = (float4v){0, 0, 0, 0};
+        {
+            const uint32_t kbase = kbuf + rowoff;
+            int m = 0;
+            for (; m + 4 <= n_packed; m += 4) k_packed_steps<4>(S, smem, stl + m * 8, qrow, kbase, kstride, lane4, nrm);
+            if (m + 2 <= n_packed) { k_packed_steps<2>(S, smem, stl + m * 8, qrow, kbase, kstride, lane4, nrm); m += 2; }
+            if (m < n_packed) { k_packed_steps<1>(S, smem, stl + m * 8, qrow, kbase, kstride, lane4, nrm); m += 1; }
+            for (; m < n_steps; m++) k_raw_step(S, smem, stl + m * 8, qrow, kbase, kstride, nrm);
         }
-        for (int m = 0; m < n_steps; m++) {
-            const int4v p0 = steps_s[2 * m], p1 = steps_s[2 * m + 1];
-            const half8 Q = *(const half8*)(qop_s + m * 1024 + lane * 16);
-            const uint32_t off = (uint32_t)p0.x + (uint32_t)min(lg, p1.w - 1) * (uint32_t)p0.y;
-            const int pw = __builtin_amdgcn_readfirstlane(p0.z);
-            if (pw != 0) {
-                const uint32_t lb = (uint32_t)p0.w + (lane4 & (uint32_t)p1.y);
-                const uint32_t sh = (uint32_t)p1.x;
-#pragma unroll
-                for (int k = 0; k < NBLK; k++) {
-                    uint32_t o = rowb[k] + off;
-                    uint32_t lo = lds_u32(kt_s, o & ~3u), hi = lds_u32(kt_s, (o & ~3u) + 4);
-                    uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
-                    half8 A;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        uint32_t idx = __builtin_amdgcn_ubfe(raw, e * pw, pw);
-                        half2v pr = __builtin_bit_cast(half2v, lds_u32(smem, (idx << sh) + lb));
-                        A[2 * e] = pr[0];
-                        A[2 * e + 1] = pr[1];
-                    }
-                    dseg[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Q, dseg[k], 0, 0, 0);
-                }
-            } else {
-                const uint16_t* tb = (const uint16_t*)(smem + p0.w);
-#pragma unroll
-                for (int k = 0; k < NBLK; k++) {
-                    uint32_t o = rowb[k] + off;
-                    uint32_t lo = lds_u32(kt_s, o & ~3u), hi = lds_u32(kt_s, (o & ~3u) + 4);
-                    uint32_t hi2 = lds_u32(kt_s, (o & ~3u) + 8);
-                    uint32_t r0 = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
-                    uint32_t r1 = __builtin_amdgcn_alignbyte(hi2, hi, o & 3u);
-                    half8 A;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        uint32_t r = e < 4 ? r0 : r1;
-                        A[e] = __builtin_bit_cast(_Float16, tb[(r >> ((e & 3) * 8)) & 0xFF]);
-                    }
-                    dseg[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Q, dseg[k], 0, 0, 0);
-                }
-            }
-            const int sz = __builtin_amdgcn_readfirstlane(p1.z);
-            if (sz & 256) {       // segment complete: scale by the token rows' group norms
-                const float* nrm = kn_s + (sz & 255) * MT + lg * 4;
-#pragma unroll
-                for (int k = 0; k < NBLK; k++) {
-                    const float4v n4 = *(const float4v*)(nrm + k * 16);
-                    S[k] += dseg[k] * n4;
-                    dseg[k] = (float4v){0, 0, 0, 0};
-                }
-            }
-        }
+        TRACE(8 + trace_j * 8 + 3);
 
         // ---- online softmax: lane (head li, group lg) holds tokens 16k + 4lg + r ------
-        float sv[4 * NBLK];
-        float mx = -INFINITY;
+        if (nt < MT) {
 #pragma unroll
-        for (int r = 0; r < 4 * NBLK; r++) {
-            int tk = (r >> 2) * 16 + lg * 4 + (r & 3);
-            float x = S[r >> 2][r & 3] * c2;
-            x = tk < nt ? x : -INFINITY;
-            sv[r] = x;
-            mx = fmaxf(mx, x);
+            for (int r = 0; r < 4 * NBLK; r++) {
+                const int tk = (r >> 2) * 16 + lg * 4 + (r & 3);
+                if (tk >= nt) S[r >> 2][r & 3] = -INFINITY;
+            }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_ref, mx);
-        if (__builtin_amdgcn_ballot_w64(m_new > m_ref)) {          // wave-uniform: rescale only when needed
+        float mx = S[0][0];
+#pragma unroll
+        for (int r = 1; r < 4 * NBLK; r++) mx = fmaxf(mx, S[r >> 2][r & 3]);
+        mx *= c2;
+        if (__builtin_amdgcn_ballot_w64(mx > m_ref)) {    // wave-uniform, rare after the first tiles
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_ref, mx + REFRESH);
             const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
             // acc rows are heads 4lg+r, not this lane's head: fetch their factors
             float al[4];
@@ -347,36 +472,41 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
             l_part *= alpha;
             m_ref = m_new;
         }
+        TRACE(8 + trace_j * 8 + 4);
+        wait_loads(k_loads);                                 // the V records of this tile are in LDS
+        __builtin_amdgcn_wave_barrier();
 
 #pragma unroll
         for (int half = 0; half < NBLK / 2; half++) {
             // P * v_norm is formed in fp32 and rounded to fp16 once
             half8 Pm;
             {
-                const uint2 vlo = *(const uint2*)(vn_s + half * 32 + lg * 4);        // tokens 4lg .. 4lg+3
-                const uint2 vhi = *(const uint2*)(vn_s + half * 32 + 16 + lg * 4);   // tokens 16+4lg ..
-                const uint32_t vnn[4] = {vlo.x, vlo.y, vhi.x, vhi.y};
+                const float4v vlo = *(const float4v*)(vn_f + half * 32 + lg * 4);        // tokens 4lg .. 4lg+3
+                const float4v vhi = *(const float4v*)(vn_f + half * 32 + 16 + lg * 4);   // tokens 16+4lg ..
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    half2v vn2 = __builtin_bit_cast(half2v, vnn[e]);
-                    float p0 = __builtin_amdgcn_exp2f(sv[half * 8 + 2 * e] - m_ref);
-                    float p1 = __builtin_amdgcn_exp2f(sv[half * 8 + 2 * e + 1] - m_ref);
+                    const int k = half * 2 + (e >> 1), r = (e & 1) * 2;
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(S[k][r], c2, -m_ref));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(S[k][r + 1], c2, -m_ref));
                     l_part += p0 + p1;
-                    Pm[2 * e] = (_Float16)(p0 * (float)vn2[0]);
-                    Pm[2 * e + 1] = (_Float16)(p1 * (float)vn2[1]);
+                    const float4v vn4 = (e >> 1) ? vhi : vlo;
+                    const float2v pv = {p0 * vn4[r], p1 * vn4[r + 1]};
+                    const half2v ph = __builtin_convertvector(pv, half2v);
+                    Pm[2 * e] = ph[0];
+                    Pm[2 * e + 1] = ph[1];
                 }
             }
             // values: lane (j = li, group lg) decodes unit j of its 8 tokens
             uint32_t W[8][4];
 #pragma unroll
             for (int r = 0; r < 8; r++) {
-                const int tk = half * 32 + (r >> 2) * 16 + lg * 4 + (r & 3);
-                uint32_t o = vph + (uint32_t)tk * vrow + (uint32_t)li * VBW;
-                uint32_t lo = lds_u32(vt_s, o & ~3u), hi = lds_u32(vt_s, (o & ~3u) + 4);
-                uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, o & 3u);
+                const int tk = half * 32 + (r >> 2) * 16 + (r & 3);      // + 4lg, folded into vbase
+                const uint32_t ad = vbase + (uint32_t)tk * vrow;
+                const uint32_t lo = lds_u32(smem, ad), hi = lds_u32(smem, ad + 4);
+                const uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, v_sh);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    uint32_t idx = __builtin_amdgcn_ubfe(raw, e * 2 * VBW, 2 * VBW);
+                    const uint32_t idx = __builtin_amdgcn_ubfe(raw, e * 2 * VBW, 2 * VBW);
                     W[r][e] = lds_u32(vlut, (idx << vshift) + vbank);
                 }
             }
@@ -395,17 +525,24 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
             }
         }
         asm volatile("" ::: "memory");
-        __builtin_amdgcn_wave_barrier();     // tile buffers are rewritten next iteration
+        __builtin_amdgcn_wave_barrier();     // V buffer and norm areas are rewritten from here on
+        v_loads = more ? issue_v(tile + step_tiles) : 0;
+        TRACE(8 + trace_j * 8 + 5);
+#ifdef BGTQ_TRACE
+        trace_j++;
+#endif
     }
+    TRACE(60);
 
-    // ---- merge the four waves ------------------------------------------------------
+    // ---- merge the waves -------------------------------------------------------------
     float l_tot = l_part;
     l_tot += __shfl_xor(l_tot, 16, 64);
     l_tot += __shfl_xor(l_tot, 32, 64);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                         // tables and tile buffers are dead from here
-    float* mg_m = (float*)smem;              // [MW][16]
-    float* mg_l = mg_m + MW * 16;            // [MW][16]
-    float* mg_o = mg_l + MW * 16;            // [MW][16][D]
+    float* mg_m = (float*)smem;              // [nw][16]
+    float* mg_l = mg_m + nw * 16;            // [nw][16]
+    float* mg_o = mg_l + nw * 16;            // [nw][16][D]
     if (lane < 16) { mg_m[wave * 16 + lane] = m_ref; mg_l[wave * 16 + lane] = l_tot; }
 #pragma unroll
     for (int e = 0; e < 8; e++)
@@ -413,14 +550,13 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
         for (int r = 0; r < 4; r++)
             mg_o[(wave * 16 + lg * 4 + r) * D + li * 8 + e] = acc[e][r];
     __syncthreads();
-    for (int i = tid; i < gqa * D; i += NT) {
+    TRACE(61);
+    for (int i = tid; i < gqa * D; i += nthr) {
         int hq = i / D, d = i - hq * D;
         float m = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < MW; w++) m = fmaxf(m, mg_m[w * 16 + hq]);
+        for (int w = 0; w < nw; w++) m = fmaxf(m, mg_m[w * 16 + hq]);
         float den = 0.f, num = 0.f;
-#pragma unroll
-        for (int w = 0; w < MW; w++) {
+        for (int w = 0; w < nw; w++) {
             float mw = mg_m[w * 16 + hq];
             float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
             den += f * mg_l[w * 16 + hq];
@@ -430,39 +566,57 @@ __global__ __launch_bounds__(NT) void decode_mfma_kernel(DecodeArgs a) {
         a.part_out[row * D + d] = (t1 > t0) ? num / den : 0.f;
         if (d == 0) a.part_lse[row] = (t1 > t0) ? (m + log2f(den)) * 0.69314718055994530942f : -INFINITY;
     }
+    TRACE(62);
 }
 
-size_t mfma_smem_bytes(int vbw, int krow, int vrow) {
-    size_t kt = (size_t)((MT * krow + 16 + 12 + 15) & ~15);
-    size_t vt = (size_t)((MT * vrow + 16 + 12 + 15) & ~15);
-    size_t wave = kt + vt + (size_t)BGTQ_MAX_SEGMENTS * MT * 4 + MT * 2;
-    size_t need = (size_t)wave_off(vbw) + wave * MW;
-    size_t merge = (size_t)(MW * 16 * 2 + MW * 16 * D) * 4;
-    return need > merge ? need : merge;
+// LDS bytes of a work-group of nw waves
+size_t mfma_smem_bytes(int vbw, int krow, int vrow, int kn_st, int nw) {
+    const TileLayout tl = tile_layout(krow, vrow, kn_st);
+    size_t need = (size_t)waves_off(vbw) + (size_t)nw * (2 * tl.kbuf + tl.vt + WAVE_NORM_BYTES);
+    size_t scratch = (size_t)waves_off(vbw) + (size_t)nw * tl.kbuf + INIT_SCRATCH;
+    size_t merge = (size_t)nw * (32 + 16 * D) * 4;
+    size_t s = need > scratch ? need : scratch;
+    return s > merge ? s : merge;
 }
 
 template <int VBW>
 int launch(const DecodeArgs& a, hipStream_t st) {
-    size_t smem = mfma_smem_bytes(VBW, a.k_row_width, a.v_row_width);
+    // no more waves than the longest partition has tiles
+    const int part = (a.T + a.n_splits - 1) / a.n_splits;
+    int nw = (part + MT - 1) / MT;
+    nw = nw < 1 ? 1 : nw > MAX_WAVES ? MAX_WAVES : nw;
+    while (nw > 1 && mfma_smem_bytes(VBW, a.k_row_width, a.v_row_width, (int)a.kn_st, nw) > (size_t)LDS_LIMIT) nw--;
+    const size_t smem = mfma_smem_bytes(VBW, a.k_row_width, a.v_row_width, (int)a.kn_st, nw);
+    if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
     auto kern = decode_mfma_kernel<VBW>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return (int)e;
+    static size_t attr_set = 0;              // largest size the attribute was raised to
+    if (smem > attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_LIMIT);
+        if (e != hipSuccess) return (int)e;
+        attr_set = LDS_LIMIT;
+    }
     dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)a.B);
-    hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(nw * 64), smem, st, a);
     return bgtq_launch_status();
 }
 
 }  // namespace
 
+#ifdef BGTQ_TRACE
+extern "C" int bgtq_debug_set_trace(void* buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &buf, sizeof(buf));
+}
+#endif
+
 int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     // layout requirements of the fast path; anything else takes the generic kernel
     if (a.k_layout != BGTQ_K_BITPACKED || a.v_layout != BGTQ_V_BITPACKED) return BGTQ_EUNSUPPORTED;
-    if (a.gqa > 16) return BGTQ_EUNSUPPORTED;
+    if (a.gqa > 16 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
     if ((a.kp_st & 3) || (a.kp_sb & 3) || (a.kp_sh & 3) || ((uintptr_t)a.kp & 3)) return BGTQ_EUNSUPPORTED;
     if ((a.vp_st & 3) || (a.vp_sb & 3) || (a.vp_sh & 3) || ((uintptr_t)a.vp & 3)) return BGTQ_EUNSUPPORTED;
     if (a.kp_st != a.k_row_width || a.vp_st != a.v_row_width) return BGTQ_EUNSUPPORTED;   // records contiguous
-    if (a.vn_st != 1) return BGTQ_EUNSUPPORTED;
-    if (MT * a.k_row_width + 12 > KR * 1024 || MT * a.v_row_width + 12 > VR * 1024) return BGTQ_EUNSUPPORTED;
+    if (a.k_row_width < 4 || a.k_row_width > 128) return BGTQ_EUNSUPPORTED;
+    if (a.vn_st != 1 || a.kn_st < 1 || a.kn_st > MAX_KN) return BGTQ_EUNSUPPORTED;
     if ((a.q_sb & 1) || (a.q_sh & 1) || ((uintptr_t)a.q & 3)) return BGTQ_EUNSUPPORTED;
     // a bit-packed V record of 128 dims is 16 bytes per bit of code width
     switch (a.v_row_width) {
