@@ -262,47 +262,83 @@ int launch_generic(const DecodeArgs& a, hipStream_t st) {
 }
 
 // ---- partition merge + V un-rotation ------------------------------------------
+// One work-group per (batch row, query head).  Thread j first takes part in
+// finding the global maximum and the weight of every partition (partitions are
+// spread over the threads, weights parked in LDS), then owns output dim j.
 __global__ __launch_bounds__(D) void lse_reduce_kernel(
     const bgtq_head_plan* plans, const float* part_out, const float* part_lse, int n_splits,
     const float* extra_out, const float* extra_lse, int n_extra,
     int n_q, int gqa, int unrotate, uint16_t* out, int64_t o_sb, int64_t o_sh, float* lse_out) {
     __shared__ float vec[D];
+    __shared__ float wgt[BGTQ_MAX_SPLITS];
+    __shared__ float red[4];
     const int j = threadIdx.x;
     const int hq = blockIdx.x, b = blockIdx.y;
     const size_t row = (size_t)b * n_q + hq;
     const float* pl = part_lse + row * n_splits;
     const float* el = extra_lse ? extra_lse + row * n_extra : nullptr;
+    const float* R = plans[hq / gqa].v_rot;
+    // the first rows of the un-rotation do not depend on anything computed here
+    constexpr int PF = 16;
+    float rpre[PF];
+#pragma unroll
+    for (int k = 0; k < PF; k++) rpre[k] = unrotate ? R[k * D + j] : 0.f;
 
     float m = -INFINITY;
-    for (int c = 0; c < n_splits; c++) m = fmaxf(m, pl[c]);
-    for (int c = 0; c < n_extra; c++) m = fmaxf(m, el[c]);
+    for (int c = j; c < n_splits; c += D) { float l = pl[c]; wgt[c] = l; m = fmaxf(m, l); }
+    for (int c = j; c < n_extra; c += D) m = fmaxf(m, el[c]);
+    m = wave_max(m);
+    if ((j & 63) == 0) red[j >> 6] = m;
+    __syncthreads();
+    m = fmaxf(red[0], red[1]);
     if (m == -INFINITY) {                      // nothing visible at all
         out[b * o_sb + hq * o_sh + j] = 0;
         if (lse_out && j == 0) lse_out[row] = -INFINITY;
         return;
     }
+    // weights: exp(lse - m), 0 for empty partitions (their vectors are undefined)
+    for (int c = j; c < n_splits; c += D) { float l = wgt[c]; wgt[c] = (l == -INFINITY) ? 0.f : __expf(l - m); }
+    __syncthreads();
     float den = 0.f, accp = 0.f, acce = 0.f;
-    for (int c = 0; c < n_splits; c++) {
-        float l = pl[c];
-        if (l == -INFINITY) continue;          // empty partition: its vector is undefined
-        float w = __expf(l - m);
-        den += w;
-        accp += w * part_out[(row * n_splits + c) * D + j];
+    const float* po = part_out + row * n_splits * D + j;
+    int c = 0;
+    for (; c + 8 <= n_splits; c += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = po[(size_t)(c + i) * D];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float w = wgt[c + i];
+            den += w;
+            if (w != 0.f) accp += w * v[i];
+        }
     }
-    for (int c = 0; c < n_extra; c++) {
-        float l = el[c];
+    for (; c < n_splits; c++) {
+        const float w = wgt[c];
+        den += w;
+        if (w != 0.f) accp += w * po[(size_t)c * D];
+    }
+    for (int e = 0; e < n_extra; e++) {
+        float l = el[e];
         if (l == -INFINITY) continue;
         float w = __expf(l - m);
         den += w;
-        acce += w * extra_out[(row * n_extra + c) * D + j];
+        acce += w * extra_out[(row * n_extra + e) * D + j];
     }
     float res = accp;
     if (unrotate) {
         vec[j] = accp;
         __syncthreads();
-        const float* R = plans[hq / gqa].v_rot;
         float r = 0.f;
-        for (int k = 0; k < D; k++) r += vec[k] * R[k * D + j];
+#pragma unroll
+        for (int k = 0; k < PF; k++) r += vec[k] * rpre[k];
+        for (int k0 = PF; k0 < D; k0 += 16) {
+            float rr[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) rr[i] = R[(k0 + i) * D + j];
+#pragma unroll
+            for (int i = 0; i < 16; i++) r += vec[k0 + i] * rr[i];
+        }
         res = r;
     }
     out[b * o_sb + hq * o_sh + j] = bgtq_f2h((res + acce) / den);
