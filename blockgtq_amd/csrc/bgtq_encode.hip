@@ -98,6 +98,7 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
             int s = IS_V ? 0 : P.seg_start[gg];
             int e = IS_V ? D : s + P.seg_len[gg];
             float ss = 0.f;
+#pragma unroll 8
             for (int k = s; k < e; k++) ss = __builtin_fmaf(xs[r][k], xs[r][k], ss);
             n = __builtin_sqrtf(ss + 1e-30f);
         }
@@ -121,6 +122,8 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
     __syncthreads();
 
     // ---- 4. rotate ------------------------------------------------------------
+    // Same chain as written in the contract above; the matrix column is fetched in
+    // batches of RB independent loads so the chain never waits on one load at a time.
     float y[ROWS];
     if (ident || g < 0) {
 #pragma unroll
@@ -128,14 +131,23 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
     } else {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) y[r] = 0.f;
-        for (int k = gs; k < ge; k++) {
-            float rt = RT[k * D + j];
+        constexpr int RB = 16;
+        for (int k0 = gs; k0 < ge; k0 += RB) {
+            float rt[RB];
 #pragma unroll
-            for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][k], rt, y[r]);
+            for (int i = 0; i < RB; i++) rt[i] = RT[min(k0 + i, ge - 1) * D + j];
+#pragma unroll
+            for (int i = 0; i < RB; i++) {
+                if (k0 + i < ge) {
+#pragma unroll
+                    for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][k0 + i], rt[i], y[r]);
+                }
+            }
         }
     }
 
     // ---- 5. scalar quantise ---------------------------------------------------
+    const bool need_cent = IS_V || a.layout == BGTQ_K_MIXED || a.corrected;
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
         int code = 0;
@@ -153,6 +165,14 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
             }
         }
         cds[r][j] = (uint8_t)code;
+        // centroid of the chosen code for the norm correction below; it is parked in xs
+        // after the barrier (other threads may still be reading xs in their rotation)
+        if (need_cent) y[r] = IS_V ? P.v_centroids[code] : (g >= 0 ? P.k_centroids[g][code] : 0.f);
+    }
+    __syncthreads();
+    if (need_cent) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) xs[r][j] = y[r];
     }
     __syncthreads();
 
@@ -164,8 +184,9 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
             float n = nrm[r][gg];
             if (IS_V) {
                 float cs = 0.f;
+#pragma unroll 8
                 for (int k = 0; k < D; k++) {
-                    float c = P.v_centroids[cds[r][k]];
+                    float c = xs[r][k];
                     cs = __builtin_fmaf(c, c, cs);
                 }
                 float cn = __builtin_sqrtf(cs + 1e-20f);
@@ -174,7 +195,7 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
                 int s = P.seg_start[gg], e = s + P.seg_len[gg];
                 float cs = 0.f;
                 for (int k = s; k < e; k++) {
-                    float c = P.k_centroids[gg][cds[r][k]];
+                    float c = xs[r][k];
                     cs = __builtin_fmaf(c, c, cs);
                 }
                 out = n / fmaxf(__builtin_sqrtf(cs), 1e-10f);
@@ -284,8 +305,16 @@ __global__ __launch_bounds__(NT) void rotate_q_kernel(
         if (P.seg_identity[g]) {
             acc = xs[j];
         } else {
-            int s = P.seg_start[g], e = s + P.seg_len[g];
-            for (int k = s; k < e; k++) acc = __builtin_fmaf(xs[k], P.k_rot_T[k * D + j], acc);
+            const int s = P.seg_start[g], e = s + P.seg_len[g];
+            constexpr int RB = 16;
+            for (int k0 = s; k0 < e; k0 += RB) {
+                float rt[RB];
+#pragma unroll
+                for (int i = 0; i < RB; i++) rt[i] = P.k_rot_T[min(k0 + i, e - 1) * D + j];
+#pragma unroll
+                for (int i = 0; i < RB; i++)
+                    if (k0 + i < e) acc = __builtin_fmaf(xs[k0 + i], rt[i], acc);
+            }
         }
     }
     q_rot[row * qr_sr + hq * qr_sh + j] = bgtq_f2h(acc);
