@@ -22,7 +22,15 @@
  *   decode          blockgtq/kernels/fused_packed_attention.py:257-294,770-894,
  *                   unpack rules :1010-1372, merge :60-103
  *
- * Parity pins (tests/test_oracle_*.py): packers against an independent
+ * Parity unpinned: the reference ships no tests or golden vectors for this
+ * path, and four things no independent check fixes: the Monte-Carlo Lloyd V
+ * centroids for 3 bits and more (blockgtq/v_quantize_gpu.py:19-117), the tie
+ * order of torch.argsort on equal bit widths (blockgtq/block_gtq_pipeline.py:163),
+ * scipy's Lloyd-Max centroids to the last ulp, and the TF32 / fp16-tile
+ * rounding of the reference's own kernels on NVIDIA hardware.  All four are
+ * inputs (tables) to the functions below, not part of their arithmetic.
+ *
+ * Parity pins (tests/test_oracle.py, tests/test_host_plan.py): packers against an independent
  * LSB-first bitstream writer and against the reference's per-dim unpack rule
  * (blockgtq/v_packing.py:118-120); V codes against numpy.searchsorted; K codes
  * of an identity-rotation single-group head against plain scalar quantisation;
