@@ -54,17 +54,16 @@ __device__ inline unsigned stream_byte(const uint8_t* codes, int len, int bw, in
 }
 
 template <int ROWS, bool IS_V>
-__global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
+__device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, const int h) {
     __shared__ float xs[ROWS][D];
     __shared__ float nrm[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ float nrm_out[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ uint8_t cds[ROWS][D];
 
     const int j = threadIdx.x;
-    const int h = blockIdx.y;
     const bgtq_head_plan& P = a.plans[h];
     const int64_t N = (int64_t)a.B * a.S;
-    const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+    const int64_t row0 = (int64_t)bx * ROWS;
 
     // ---- per-thread static data -------------------------------------------
     const int n_seg = IS_V ? 1 : P.n_seg;
@@ -271,6 +270,11 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
     }
 }
 
+template <int ROWS, bool IS_V>
+__global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
+    encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y);
+}
+
 template <bool IS_V>
 int launch_encode(const EncodeArgs& a, hipStream_t st) {
     int64_t N = (int64_t)a.B * a.S;
@@ -289,15 +293,18 @@ int launch_encode(const EncodeArgs& a, hipStream_t st) {
 }
 
 // ---- query permute + rotate ---------------------------------------------------
-__global__ __launch_bounds__(NT) void rotate_q_kernel(
-    const bgtq_head_plan* plans, const uint16_t* q, int64_t q_sr, int64_t q_sh,
-    uint16_t* q_rot, int64_t qr_sr, int64_t qr_sh, int gqa) {
+struct RotQArgs {
+    const bgtq_head_plan* plans;
+    const uint16_t* q;  int64_t q_sr, q_sh;
+    uint16_t* q_rot;    int64_t qr_sr, qr_sh;
+    int n_rows, n_q, gqa;
+};
+
+__device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t row, const int hq) {
     __shared__ float xs[D];
     const int j = threadIdx.x;
-    const int hq = blockIdx.y;
-    const int64_t row = blockIdx.x;
-    const bgtq_head_plan& P = plans[hq / gqa];
-    xs[j] = bgtq_h2f(q[row * q_sr + hq * q_sh + P.head_perm[j]]);
+    const bgtq_head_plan& P = a.plans[hq / a.gqa];
+    xs[j] = bgtq_h2f(a.q[row * a.q_sr + hq * a.q_sh + P.head_perm[j]]);
     __syncthreads();
     const int g = P.group_of[j];
     float acc = 0.f;
@@ -317,7 +324,71 @@ __global__ __launch_bounds__(NT) void rotate_q_kernel(
             }
         }
     }
-    q_rot[row * qr_sr + hq * qr_sh + j] = bgtq_f2h(acc);
+    a.q_rot[row * a.qr_sr + hq * a.qr_sh + j] = bgtq_f2h(acc);
+}
+
+__global__ __launch_bounds__(NT) void rotate_q_kernel(RotQArgs a) {
+    rotate_q_row(a, blockIdx.x, blockIdx.y);
+}
+
+// ---- decode-step preparation: append-encode K and V and rotate the queries, one launch ----
+// Work-groups [0, nk) encode K row pairs, [nk, nk + nv) V row pairs, the rest one query row each.
+__global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs av, RotQArgs aq,
+                                                     int k_tiles, int v_tiles) {
+    int bid = blockIdx.x;
+    const int nk = k_tiles * ak.n_kv, nv = v_tiles * av.n_kv;
+    if (bid < nk) {
+        encode_rows<2, false>(ak, bid % k_tiles, bid / k_tiles);
+    } else if (bid < nk + nv) {
+        bid -= nk;
+        encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles);
+    } else {
+        bid -= nk + nv;
+        rotate_q_row(aq, bid / aq.n_q, bid % aq.n_q);
+    }
+}
+
+// argument checks + EncodeArgs assembly shared by the separate and the fused entry points
+int fill_k_args(EncodeArgs& a, const bgtq_head_plan* plans,
+                const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss, int B, int n_kv, int S,
+                void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
+                const int32_t* t_pos, int t_pos_scalar, int k_layout, int quant_mode) {
+    BGTQ_CHECK_ARG(plans && k && k_packed && k_norms);
+    BGTQ_CHECK_ARG(k_row_width >= 0 && k_row_width <= NT);
+    BGTQ_CHECK_ARG(norm_width >= 0 && norm_width <= BGTQ_MAX_SEGMENTS);
+    BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
+    BGTQ_CHECK_ARG(quant_mode == BGTQ_QUANT_LUT256 || quant_mode == BGTQ_QUANT_EXACT);
+    BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
+    a.plans = plans; a.x = (const uint16_t*)k; a.x_sb = k_sb; a.x_sh = k_sh; a.x_ss = k_ss;
+    a.B = B; a.n_kv = n_kv; a.S = S;
+    a.packed = (uint8_t*)k_packed; a.p_sb = kp_sb; a.p_sh = kp_sh; a.p_st = kp_st;
+    a.row_width = k_row_width;
+    a.norms = (uint16_t*)k_norms; a.n_sb = kn_sb; a.n_sh = kn_sh; a.n_st = kn_st;
+    a.norm_width = norm_width;
+    a.t_pos = t_pos; a.t_pos_scalar = t_pos_scalar;
+    a.layout = k_layout; a.quant_mode = quant_mode;
+    return BGTQ_OK;
+}
+
+int fill_v_args(EncodeArgs& a, const bgtq_head_plan* plans,
+                const void* v, int64_t v_sb, int64_t v_sh, int64_t v_ss, int B, int n_kv, int S,
+                void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                const int32_t* t_pos, int t_pos_scalar, int v_layout) {
+    BGTQ_CHECK_ARG(plans && v && v_packed && v_norms);
+    BGTQ_CHECK_ARG(v_row_width >= 0 && v_row_width <= NT);
+    BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
+    BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
+    a.plans = plans; a.x = (const uint16_t*)v; a.x_sb = v_sb; a.x_sh = v_sh; a.x_ss = v_ss;
+    a.B = B; a.n_kv = n_kv; a.S = S;
+    a.packed = (uint8_t*)v_packed; a.p_sb = vp_sb; a.p_sh = vp_sh; a.p_st = vp_st;
+    a.row_width = v_row_width;
+    a.norms = (uint16_t*)v_norms; a.n_sb = vn_sb; a.n_sh = vn_sh; a.n_st = vn_st;
+    a.norm_width = 1;
+    a.t_pos = t_pos; a.t_pos_scalar = t_pos_scalar;
+    a.layout = v_layout;
+    return BGTQ_OK;
 }
 
 }  // namespace
@@ -333,21 +404,10 @@ int bgtq_encode_k(const bgtq_head_plan* plans,
                   int k_layout, int quant_mode, void* stream) {
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
     if (B == 0 || n_kv == 0 || S == 0) return BGTQ_OK;     // nothing to encode
-    BGTQ_CHECK_ARG(plans && k && k_packed && k_norms);
-    BGTQ_CHECK_ARG(k_row_width >= 0 && k_row_width <= NT);
-    BGTQ_CHECK_ARG(norm_width >= 0 && norm_width <= BGTQ_MAX_SEGMENTS);
-    BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
-    BGTQ_CHECK_ARG(quant_mode == BGTQ_QUANT_LUT256 || quant_mode == BGTQ_QUANT_EXACT);
-    BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
     EncodeArgs a{};
-    a.plans = plans; a.x = (const uint16_t*)k; a.x_sb = k_sb; a.x_sh = k_sh; a.x_ss = k_ss;
-    a.B = B; a.n_kv = n_kv; a.S = S;
-    a.packed = (uint8_t*)k_packed; a.p_sb = kp_sb; a.p_sh = kp_sh; a.p_st = kp_st;
-    a.row_width = k_row_width;
-    a.norms = (uint16_t*)k_norms; a.n_sb = kn_sb; a.n_sh = kn_sh; a.n_st = kn_st;
-    a.norm_width = norm_width;
-    a.t_pos = t_pos; a.t_pos_scalar = t_pos_scalar;
-    a.layout = k_layout; a.quant_mode = quant_mode;
+    int rc = fill_k_args(a, plans, k, k_sb, k_sh, k_ss, B, n_kv, S, k_packed, kp_sb, kp_sh, kp_st, k_row_width,
+                         k_norms, kn_sb, kn_sh, kn_st, norm_width, t_pos, t_pos_scalar, k_layout, quant_mode);
+    if (rc != BGTQ_OK) return rc;
     return launch_encode<false>(a, (hipStream_t)stream);
 }
 
@@ -360,19 +420,10 @@ int bgtq_encode_v(const bgtq_head_plan* plans,
                   int v_layout, void* stream) {
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
     if (B == 0 || n_kv == 0 || S == 0) return BGTQ_OK;
-    BGTQ_CHECK_ARG(plans && v && v_packed && v_norms);
-    BGTQ_CHECK_ARG(v_row_width >= 0 && v_row_width <= NT);
-    BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
-    BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
     EncodeArgs a{};
-    a.plans = plans; a.x = (const uint16_t*)v; a.x_sb = v_sb; a.x_sh = v_sh; a.x_ss = v_ss;
-    a.B = B; a.n_kv = n_kv; a.S = S;
-    a.packed = (uint8_t*)v_packed; a.p_sb = vp_sb; a.p_sh = vp_sh; a.p_st = vp_st;
-    a.row_width = v_row_width;
-    a.norms = (uint16_t*)v_norms; a.n_sb = vn_sb; a.n_sh = vn_sh; a.n_st = vn_st;
-    a.norm_width = 1;
-    a.t_pos = t_pos; a.t_pos_scalar = t_pos_scalar;
-    a.layout = v_layout;
+    int rc = fill_v_args(a, plans, v, v_sb, v_sh, v_ss, B, n_kv, S, v_packed, vp_sb, vp_sh, vp_st, v_row_width,
+                         v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, v_layout);
+    if (rc != BGTQ_OK) return rc;
     return launch_encode<true>(a, (hipStream_t)stream);
 }
 
@@ -409,10 +460,46 @@ int bgtq_rotate_q(const bgtq_head_plan* plans,
     BGTQ_CHECK_ARG(plans && q && q_rot);
     BGTQ_CHECK_ARG(n_rows >= 0 && n_kv >= 0 && gqa >= 1);
     if (n_rows == 0 || n_kv == 0) return BGTQ_OK;
+    RotQArgs a{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, n_rows, n_kv * gqa, gqa};
     dim3 grid((unsigned)n_rows, (unsigned)(n_kv * gqa));
-    hipLaunchKernelGGL(rotate_q_kernel, grid, dim3(NT), 0, (hipStream_t)stream,
-                       plans, (const uint16_t*)q, q_sr, q_sh,
-                       (uint16_t*)q_rot, qr_sr, qr_sh, gqa);
+    hipLaunchKernelGGL(rotate_q_kernel, grid, dim3(NT), 0, (hipStream_t)stream, a);
+    return bgtq_launch_status();
+}
+
+int bgtq_decode_prepare(const bgtq_head_plan* plans,
+                        const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                        const void* v, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                        int B, int n_kv, int S,
+                        void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                        void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
+                        void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                        void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                        const int32_t* t_pos, int t_pos_scalar,
+                        int k_layout, int v_layout, int quant_mode,
+                        const void* q, int64_t q_sr, int64_t q_sh,
+                        void* q_rot, int64_t qr_sr, int64_t qr_sh, int gqa, void* stream) {
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0 && gqa >= 1);
+    if (B == 0 || n_kv == 0) return BGTQ_OK;
+    EncodeArgs ak{}, av{};
+    int rc = fill_k_args(ak, plans, k, k_sb, k_sh, k_ss, B, n_kv, S, k_packed, kp_sb, kp_sh, kp_st, k_row_width,
+                         k_norms, kn_sb, kn_sh, kn_st, norm_width, t_pos, t_pos_scalar, k_layout, quant_mode);
+    if (rc != BGTQ_OK) return rc;
+    rc = fill_v_args(av, plans, v, v_sb, v_sh, v_ss, B, n_kv, S, v_packed, vp_sb, vp_sh, vp_st, v_row_width,
+                     v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, v_layout);
+    if (rc != BGTQ_OK) return rc;
+    BGTQ_CHECK_ARG(q && q_rot);
+    const int64_t N = (int64_t)B * S;
+    if (N > 64) {          // prefill-sized append: the three stages are big enough on their own
+        rc = launch_encode<false>(ak, (hipStream_t)stream);
+        if (rc != BGTQ_OK) return rc;
+        rc = launch_encode<true>(av, (hipStream_t)stream);
+        if (rc != BGTQ_OK) return rc;
+        return bgtq_rotate_q(plans, q, q_sr, q_sh, q_rot, qr_sr, qr_sh, B, n_kv, gqa, stream);
+    }
+    RotQArgs aq{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, B, n_kv * gqa, gqa};
+    const int tiles = (int)((N + 1) / 2);
+    const unsigned blocks = (unsigned)(2 * tiles * n_kv + B * n_kv * gqa);
+    hipLaunchKernelGGL(prepare_kernel, dim3(blocks), dim3(NT), 0, (hipStream_t)stream, ak, av, aq, tiles, tiles);
     return bgtq_launch_status();
 }
 

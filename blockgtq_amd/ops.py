@@ -113,3 +113,39 @@ def decode_attention(plans: torch.Tensor, q_rot: torch.Tensor,
         B, n_kv, gqa, int(unrotate), _capi.ptr(out), out.stride(0), out.stride(1),
         _capi.ptr(lse), st), "bgtq_lse_reduce")
     return (out, lse) if return_lse else out
+
+
+def decode_prepare(plans: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q: torch.Tensor,
+                   k_packed: torch.Tensor, k_norms: torch.Tensor, v_packed: torch.Tensor,
+                   v_norms: torch.Tensor, t_pos, k_row_width: int, norm_width: int,
+                   v_row_width: int, n_kv: int, k_layout: int, v_layout: int,
+                   quant_mode: int = _plan.QUANT_LUT256) -> torch.Tensor:
+    """One launch for everything a decode step does before attention: encode
+    ``k`` / ``v`` (B, n_kv, S, D) fp16 into the cache views at ``t_pos`` (int or
+    int32 device tensor (B,)) and rotate ``q`` (B, n_q, D) fp16.  Returns the
+    rotated queries; same results as ``encode_k_into`` + ``encode_v_into`` + ``rotate_q``."""
+    _capi.require_cuda(k, "k")
+    for t in (k, v, q):
+        assert t.dtype == torch.float16 and t.stride(-1) == 1
+    assert k_packed.dtype == torch.uint8 and v_packed.dtype == torch.uint8
+    assert k_norms.dtype == torch.float16 and v_norms.dtype == torch.float16
+    B, H, S, _ = k.shape
+    n_q = q.shape[1]
+    q_rot = torch.empty((B, n_q, q.shape[2]), dtype=torch.float16, device=q.device)
+    if isinstance(t_pos, torch.Tensor):
+        assert t_pos.dtype == torch.int32 and t_pos.is_cuda
+        tp, ts = _capi.ptr(t_pos), 0
+    else:
+        tp, ts = None, int(t_pos)
+    L = _capi.lib()
+    _capi.check(L.bgtq_decode_prepare(
+        _capi.ptr(plans), _capi.ptr(k), k.stride(0), k.stride(1), k.stride(2),
+        _capi.ptr(v), v.stride(0), v.stride(1), v.stride(2), B, H, S,
+        _capi.ptr(k_packed), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2), k_row_width,
+        _capi.ptr(k_norms), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2), norm_width,
+        _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), v_row_width,
+        _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
+        tp, ts, k_layout, v_layout, quant_mode,
+        _capi.ptr(q), q.stride(0), q.stride(1), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1),
+        n_q // n_kv, _capi.stream_ptr(k.device)), "bgtq_decode_prepare")
+    return q_rot

@@ -44,6 +44,7 @@ class BlockGTQKVManager:
         self.scale = 1.0 / math.sqrt(head_dim)
         self.seq_len = 0
         self._seq_lens = None          # int32 (B,) device tensor when rows are ragged
+        self._lens_src, self._lens_S, self._lens_plus = None, 0, None   # cached _seq_lens + S
 
         self.quantizers = [[None] * n_kv_heads for _ in range(n_layers)]
         self._kernel_args = [[None] * n_kv_heads for _ in range(n_layers)]
@@ -146,18 +147,30 @@ class BlockGTQKVManager:
         li = layer_idx
         S = k_new.shape[2]
         t_pos = self._seq_lens if self._seq_lens is not None else self.seq_len
-        self._encode_kv(li, k_new, v_new, t_pos)
         T = self.seq_len + S
         plans = self._batched_args[li]['plans']
         B = q.shape[0]
         q3 = q.reshape(B, self.n_q, self.hd)
         if q3.dtype != torch.float16:
             q3 = q3.to(torch.float16)
-        if not self.quantizers[li][0]._q_perm_baked:
-            q3 = ops.rotate_q(plans, q3.contiguous(), self.n_kv)
+        if self.quantizers[li][0]._q_perm_baked:
+            self._encode_kv(li, k_new, v_new, t_pos)
+        else:
+            # encode K, V and rotate the queries in one launch
+            self._ensure_storage()
+            k16 = k_new if k_new.dtype == torch.float16 else k_new.to(torch.float16)
+            v16 = v_new if v_new.dtype == torch.float16 else v_new.to(torch.float16)
+            k16 = k16 if k16.stride(-1) == 1 else k16.contiguous()
+            v16 = v16 if v16.stride(-1) == 1 else v16.contiguous()
+            q3 = ops.decode_prepare(
+                plans, k16, v16, q3.contiguous(), self._k_packed[li], self._k_norms[li],
+                self._v_packed[li], self._v_norms[li], t_pos, self._k_row,
+                self._k_norms.shape[-1], self._vpb, self.n_kv, _plan.K_BITPACKED, _plan.V_BITPACKED)
         lens = None
         if self._seq_lens is not None:
-            lens = self._seq_lens + S
+            if self._lens_src is not self._seq_lens or self._lens_S != S:   # one add per step, not per layer
+                self._lens_src, self._lens_S, self._lens_plus = self._seq_lens, S, self._seq_lens + S
+            lens = self._lens_plus
         out = ops.decode_attention(
             plans, q3.contiguous(), self._k_packed[li], self._k_norms[li],
             self._v_packed[li], self._v_norms[li], T, seq_lens=lens, n_splits=self.n_splits,

@@ -178,6 +178,30 @@ int bgtq_rotate_q(const bgtq_head_plan* plans,
                   int n_rows, int n_kv, int gqa, void* stream);
 
 /*
+ * Decode-step preparation in ONE launch: append-encode the new K and V tokens
+ * into their cache slots (as bgtq_encode_k / bgtq_encode_v) and rotate the
+ * queries (as bgtq_rotate_q).  Results are identical to the three separate
+ * calls.  Covers what one layer of a decode step does before attention in
+ * BlockGTQKVManager.append_and_attend (blockgtq/packed_kv_manager.py:269-330:
+ * _compress_and_store K, V, then rotate_q_for_packed_kernel per KV head) and in
+ * BlockGTQProductionCache.encode_and_attend (blockgtq/production_cache.py:207-245).
+ * Arguments have the meaning they have in those three entry points; q has
+ * B rows of n_kv * gqa heads.
+ */
+int bgtq_decode_prepare(const bgtq_head_plan* plans,
+                        const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                        const void* v, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                        int B, int n_kv, int S,
+                        void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                        void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
+                        void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                        void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                        const int32_t* t_pos, int t_pos_scalar,
+                        int k_layout, int v_layout, int quant_mode,
+                        const void* q, int64_t q_sr, int64_t q_sh,
+                        void* q_rot, int64_t qr_sr, int64_t qr_sh, int gqa, void* stream);
+
+/*
  * Kernel selection of bgtq_decode_attn (process-wide; meant for tests and
  * profiling): 0 = automatic (MFMA kernel when the layout allows it, otherwise
  * the layout-agnostic kernel), 1 = always the layout-agnostic kernel,

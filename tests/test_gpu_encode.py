@@ -185,3 +185,41 @@ def test_query_rotation_is_bit_exact(oracle_lib):
         assert np.array_equal(got[:, 4 * h:4 * h + 4].reshape(-1, 128).view(np.uint16), want.view(np.uint16))
     single = qs[1].rotate_q_for_packed_kernel(q[:, 4:8])
     assert np.array_equal(single.cpu().numpy(), got[:, 4:8])
+
+
+@pytest.mark.parametrize("S", [1, 3, 40])
+def test_fused_prepare_equals_the_three_separate_calls(S):
+    """``bgtq_decode_prepare`` (append-encode K, V and rotate Q in one launch) writes the
+    same bytes as ``bgtq_encode_k`` + ``bgtq_encode_v`` + ``bgtq_rotate_q``; S = 40 with
+    B = 2 takes its prefill-sized route."""
+    from blockgtq_amd import ops
+    from blockgtq_amd.quantizer import build_batched_encode_args, encode_k_into, encode_v_into
+    qs = [make_quantizer(seed=70 + h, head=h, device=DEV, max_bits=5)[0] for h in range(2)]
+    args = build_batched_encode_args(qs, device=DEV)
+    B, H, gqa = 2, 2, 4
+    gen = torch.Generator().manual_seed(11 + S)
+    k = torch.randn(B, H, S, 128, generator=gen).half().to(DEV)
+    v = torch.randn(B, H, S, 128, generator=gen).half().to(DEV)
+    q = torch.randn(B, H * gqa, 128, generator=gen).half().to(DEV)
+    kw = (args['max_tpb'] + 3) // 4 * 4
+    ng = args['max_n_groups']
+    pos = torch.tensor([3, 17], dtype=torch.int32, device=DEV)
+
+    def buffers():
+        return (torch.zeros(B, H, 64, kw, dtype=torch.uint8, device=DEV),
+                torch.zeros(B, H, 64, ng, dtype=torch.float16, device=DEV),
+                torch.zeros(B, H, 64, 48, dtype=torch.uint8, device=DEV),
+                torch.zeros(B, H, 64, dtype=torch.float16, device=DEV))
+
+    kp0, kn0, vp0, vn0 = buffers()
+    encode_k_into(args['plans'], k, kp0, kn0, pos, kw, ng, 0)
+    encode_v_into(args['plans'], v, vp0, vn0, pos, 48, 0)
+    q0 = ops.rotate_q(args['plans'], q, H)
+    kp1, kn1, vp1, vn1 = buffers()
+    q1 = ops.decode_prepare(args['plans'], k, v, q, kp1, kn1, vp1, vn1, pos, kw, ng, 48, H, 0, 0)
+    torch.cuda.synchronize()
+    assert kp0.any() and vp0.any()
+    for a, b in ((kp0, kp1), (vp0, vp1), (q0, q1)):
+        assert torch.equal(a, b)
+    assert torch.equal(kn0.view(torch.int16), kn1.view(torch.int16))
+    assert torch.equal(vn0.view(torch.int16), vn1.view(torch.int16))
