@@ -12,10 +12,11 @@
 // passes through vector registers.
 //
 // Dequantisation is table driven.  A "unit" is 8 consecutive codes of one
-// token (bw bytes of the record).  For every bit width <= 4 the work-group
-// builds a pair table in LDS: entry (c0 | c1 << bw) holds the two fp16
-// centroids of a code pair, replicated across LDS banks so that lanes with
-// different indices do not collide (32 copies, 8 for the 256-entry 4-bit table).
+// token (bw bytes of the record).  For every bit width <= 4 the plan carries a
+// pair table that the work-group copies into LDS: entry (c0 | c1 << bw) holds
+// the two fp16 centroids of a code pair, replicated across LDS banks so that
+// lanes with different indices do not collide (32 copies, 8 for the 256-entry
+// 4-bit table).
 // A unit costs one raw read, four {bit-field extract, shift-add, table read}
 // triples and yields the eight fp16 operands of one MFMA k-group.
 //
@@ -55,19 +56,15 @@ constexpr int LDS_LIMIT = 160 * 1024;
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
-constexpr int KLUT1 = 0;                       // 4 entries   x 128 B
-constexpr int KLUT2 = KLUT1 + 4 * 128;         // 16 entries  x 128 B
-constexpr int KLUT3 = KLUT2 + 16 * 128;        // 64 entries  x 128 B
-constexpr int KLUT4 = KLUT3 + 64 * 128;        // 256 entries x 32 B
-constexpr int KRAW = KLUT4 + 256 * 32;         // 4 tables x 256 fp16 (bw 5..8)
-constexpr int VLUT = KRAW + 4 * 512;
+// The first BGTQ_LUT_V + vlut_bytes bytes are a copy of the plan's lut_image.
+constexpr int VLUT = BGTQ_LUT_V;
 constexpr int QROW = 400;                      // one head: zero unit + up to 24 units x 16 B
 __host__ __device__ constexpr int vlut_bytes(int vbw) { return vbw == 4 ? 256 * 32 : (1 << (2 * vbw)) * 128; }
 __host__ __device__ constexpr int steptab_off(int vbw) { return VLUT + vlut_bytes(vbw); }   // [step][lane group] x 32 B
 __host__ __device__ constexpr int qpad_off(int vbw) { return steptab_off(vbw) + MAX_STEPS * 4 * 32; }
 __host__ __device__ constexpr int waves_off(int vbw) { return qpad_off(vbw) + 16 * QROW; }
 constexpr int WAVE_NORM_BYTES = BGTQ_MAX_SEGMENTS * MT * 2 + MT * 4;   // fp16 K norms [seg][token], fp32 V norms
-constexpr int INIT_SCRATCH = 768 + 4096 + 16 * D * 2;
+constexpr int INIT_SCRATCH = MAX_STEPS * 4 * 32 + 256 + 16 * D * 2;
 
 struct TileLayout {
     int kt, vt, knr, vnr, kbuf;    // bytes of the K, V, K-norm, V-norm areas; K + both norm areas
@@ -279,103 +276,50 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const int step_tiles = nw * MT;
     int tile = t0 + wave * MT;
     int v_loads = 0;                 // loads of the V tile issued after the current K tile
-    if (tile < t1) issue_k(tile, 0);
-    TRACE(1);
 
-    // ---- init 1: plan header, step schedule, codebooks and queries into LDS scratch --
-    int* hdr_s = (int*)scratch;                           // first 56 ints of the plan
-    int* stp_s = (int*)(scratch + 256);                   // n_steps, 3 pad, step[12][8]
-    uint16_t* vcb_s = (uint16_t*)(scratch + 704);         // [16] V centroids
-    uint16_t* cb_s = (uint16_t*)(scratch + 768);          // [8][256] K codebooks
-    uint16_t* q_s = (uint16_t*)(scratch + 768 + 4096);    // [16][128] rotated queries
-    for (int i = tid; i < 56; i += nthr) hdr_s[i] = ((const int*)&P)[i];
-    for (int i = tid; i < 4 + MAX_STEPS * 8; i += nthr) stp_s[i] = (&P.n_steps)[i];
-    for (int i = tid; i < 8; i += nthr) ((uint32_t*)vcb_s)[i] = ((const uint32_t*)P.v_lut_f16)[i];
-    for (int i = tid; i < BGTQ_MAX_SEGMENTS * 128; i += nthr)
-        ((uint32_t*)cb_s)[i] = ((const uint32_t*)&P.k_codebook_f16[0][0])[i];
+    // ---- init: tables, step parameters, query units -------------------------------------
+    // The pair tables come ready-made from the plan and are copied into LDS by DMA, each
+    // wave taking every nw-th KB; the first K tile follows right behind them.
+    {
+        const uint8_t* img = (const uint8_t*)P.lut_image;
+        constexpr int total = BGTQ_LUT_V + vlut_bytes(VBW);
+        for (int cc = wave; cc * 1024 < total; cc += nw)
+            if ((int)voff + cc * 1024 < total)
+                dma16<0>(voff, uniform_ptr(img + cc * 1024), __builtin_amdgcn_readfirstlane(smem_lds + cc * 1024));
+    }
+    int k0_loads = 0;
+    if (tile < t1) k0_loads = issue_k(tile, 0);
+    TRACE(1);
+    uint32_t* st_raw = (uint32_t*)scratch;                // steptab as stored in the plan
+    int* qu_s = (int*)(scratch + MAX_STEPS * 4 * 32);     // qunit_dim[32], qunit_len[32]
+    uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 4 * 32 + 256);   // [16][128] rotated queries
+    for (int i = tid; i < MAX_STEPS * 4 * 8; i += nthr) st_raw[i] = (&P.steptab[0][0][0])[i];
+    for (int i = tid; i < 64; i += nthr) qu_s[i] = P.qunit_dim[i];     // qunit_len follows qunit_dim
     for (int i = tid; i < 16 * D / 2; i += nthr) {
         int hq = i / (D / 2), d2 = i - hq * (D / 2);
         uint32_t v = 0;
         if (hq < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + hq) * a.q_sh + d2 * 2);
         ((uint32_t*)q_s)[i] = v;
     }
+    const int n_seg = min(P.n_seg, BGTQ_MAX_SEGMENTS);
+    const int n_steps = min(P.n_steps, MAX_STEPS);
+    const int n_packed = min(P.n_packed_steps, n_steps);   // raw-byte steps (bw >= 5) come last
     __syncthreads();
     TRACE(2);
-    const int n_seg = min(hdr_s[0], BGTQ_MAX_SEGMENTS);
-    const int* seg_bw = hdr_s + 8;
-    const int* seg_start = hdr_s + 16;
-    const int* seg_len = hdr_s + 24;
-    const int n_steps = min(stp_s[0], MAX_STEPS);
-    int n_packed = 0;                                      // raw-byte steps (bw >= 5) come last
-    for (int m = 0; m < n_steps; m++) n_packed += stp_s[4 + m * 8 + 2] != 0;
-
-    // ---- init 2: pair tables ---------------------------------------------------------
-    for (int s = 0; s < n_seg; s++) {
-        const int bw = seg_bw[s];
-        if (bw <= 4) {
-            const int n = 1 << (2 * bw);
-            const int rsh = bw == 4 ? 3 : 5;               // log2 of the replication factor
-            uint8_t* tb = smem + (bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : KLUT4);
-            for (int i = tid; i < (n << rsh); i += nthr) {
-                int e = i >> rsh;
-                uint32_t v = (uint32_t)cb_s[s * 256 + (e & ((1 << bw) - 1))] |
-                             ((uint32_t)cb_s[s * 256 + (e >> bw)] << 16);
-                *(uint32_t*)(tb + i * 4) = v;
-            }
-        } else {
-            // every byte value needs a finite entry: the last unit of a segment also
-            // decodes bytes of its neighbour (their products meet a zero query)
-            uint16_t* tb = (uint16_t*)(smem + KRAW) + (bw - 5) * 256;
-            for (int i = tid; i < 256; i += nthr) tb[i] = i < (1 << bw) ? cb_s[s * 256 + i] : (uint16_t)0;
-        }
+    for (int i = tid; i < n_steps * 4; i += nthr) {        // the row offset depends on the cache's alignment
+        const uint32_t* r = st_raw + i * 8;
+        const uint32_t o = kph + r[0];
+        steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2], r[3]};
+        steptab[i * 2 + 1] = (uint4){r[4], r[5], r[6], r[7]};
     }
-    {
-        constexpr int n = 1 << (2 * VBW);
-        constexpr int rsh = VBW == 4 ? 3 : 5;
-        for (int i = tid; i < (n << rsh); i += nthr) {
-            int e = i >> rsh;
-            uint32_t v = (uint32_t)vcb_s[e & ((1 << VBW) - 1)] | ((uint32_t)vcb_s[e >> VBW] << 16);
-            *(uint32_t*)(vlut + i * 4) = v;
-        }
+    for (int i = tid; i < 16 * (QROW / 4); i += nthr) {     // query units, zero padded
+        const int hd = i / (QROW / 4), rem = i - hd * (QROW / 4), uid = rem >> 2, pp = rem & 3;
+        const int d0 = qu_s[uid] + 2 * pp, len = qu_s[32 + uid];
+        const uint16_t* row = q_s + hd * D;
+        const uint32_t lo = 2 * pp < len ? row[d0] : 0, hi = 2 * pp + 1 < len ? row[d0 + 1] : 0;
+        ((uint32_t*)qpad)[i] = lo | (hi << 16);
     }
-    // ---- init 3: per (step, lane group) parameters and the padded query units -------------
-    // plan step m: {byte offset of unit 0, bytes per unit, bits per pair (0 = raw bytes), bw,
-    //               segment, last-of-segment, real units, first dim}
-    for (int i = tid; i < n_steps * 4; i += nthr) {
-        const int m = i >> 2, g = i & 3;
-        const int* sp = stp_s + 4 + m * 8;
-        const int bw = sp[3], nu = sp[6];
-        int ub = 0;
-        for (int j = 0; j < m; j++) ub += stp_s[4 + j * 8 + 6];
-        const uint32_t o = kph + (uint32_t)sp[0] + (uint32_t)min(g, nu - 1) * (uint32_t)sp[1];
-        uint4 e0, e1;
-        e0.x = o & ~3u;                                              // aligned byte offset in the row
-        e0.y = o & 3u;                                               // byte shift of the unit
-        e0.z = bw == 1 ? KLUT1 : bw == 2 ? KLUT2 : bw == 3 ? KLUT3 : bw == 4 ? KLUT4
-                                                            : KRAW + (bw - 5) * 512;
-        e0.w = bw == 4 ? 7 * 4 : bw <= 3 ? 31 * 4 : 0;               // bank replica mask
-        e1.x = (uint32_t)sp[2];
-        e1.y = bw == 4 ? 5 : 7;                                      // log2 of the table entry stride
-        e1.z = (uint32_t)sp[4] * (MT * 2);                           // norm row of the segment
-        e1.w = g < nu ? (uint32_t)(1 + ub + g) * 16 : 0;             // byte offset of the query unit
-        steptab[i * 2] = e0;
-        steptab[i * 2 + 1] = e1;
-    }
-    if (tid < 64) ((uint32_t*)qpad)[(tid >> 2) * (QROW / 4) + (tid & 3)] = 0;      // unit 0 is all zero (one wave is enough)
-    for (int i = tid; i < n_steps * 256; i += nthr) {
-        const int p = i & 3, hd = (i >> 2) & 15, g = (i >> 6) & 3, m = i >> 8;
-        const int* sp = stp_s + 4 + m * 8;
-        if (g < sp[6]) {
-            int ub = 0;
-            for (int j = 0; j < m; j++) ub += stp_s[4 + j * 8 + 6];
-            const int uid = 1 + ub + g;
-            const int dd = sp[7] + 8 * g + 2 * p;
-            const int end = seg_start[sp[4]] + seg_len[sp[4]];
-            const uint16_t* row = q_s + hd * D;
-            uint32_t lo = dd < end ? row[dd] : 0, hi = dd + 1 < end ? row[dd + 1] : 0;
-            if (uid < QROW / 16) ((uint32_t*)qpad)[hd * (QROW / 4) + uid * 4 + p] = lo | (hi << 16);
-        }
-    }
+    wait_loads(k0_loads);                                   // this wave's share of the tables has landed
     __syncthreads();                                        // scratch is dead from here
     if (tile < t1) v_loads = issue_v(tile);
     TRACE(4);

@@ -37,7 +37,14 @@ PLAN_DTYPE = np.dtype([
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
     ('n_steps', '<i4'), ('reserved1', '<i4', (3,)), ('step', '<i4', (MAX_STEPS, 8)),
+    ('n_packed_steps', '<i4'), ('reserved2', '<i4', (3,)),
+    ('steptab', '<u4', (MAX_STEPS, 4, 8)), ('qunit_dim', '<i4', (32,)), ('qunit_len', '<i4', (32,)),
+    ('lut_image', '<u4', (29184 // 4,)),
 ], align=True)
+
+# byte offsets inside lut_image (BGTQ_LUT_* of include/bgtq.h)
+LUT_K = {1: 0, 2: 512, 3: 2560, 4: 10752}
+LUT_KRAW, LUT_V, LUT_IMAGE_BYTES = 18944, 20992, 29184
 
 
 def segment_bytes(bw: int, length: int) -> int:
@@ -53,22 +60,68 @@ def segment_bytes(bw: int, length: int) -> int:
     return length
 
 
+def _pair_table(cb16: np.ndarray, bw: int) -> np.ndarray:
+    """Bank-replicated pair table of one code width: entry (c0 | c1 << bw)."""
+    e = np.arange(1 << (2 * bw))
+    pairs = cb16[e & ((1 << bw) - 1)].astype(np.uint32) | (cb16[e >> bw].astype(np.uint32) << 16)
+    return np.repeat(pairs, 8 if bw == 4 else 32)
+
+
 def fill_decode_steps(p) -> None:
-    """Derive the MFMA step schedule of the bit-packed K record from the
-    segment table already stored in plan ``p`` (a 0-d structured array)."""
-    m = 0
+    """Derive the MFMA step schedule of the bit-packed K record, its LDS-ready
+    form and the pair tables from the segment table, codebooks and V LUT
+    already stored in plan ``p`` (a 0-d structured array)."""
+    m, n_packed, unit = 0, 0, 1
+    p['step'][...] = 0
+    p['steptab'][...] = 0
+    p['qunit_dim'][...] = 0
+    p['qunit_len'][...] = 0
     for s in range(int(p['n_seg'])):
         bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
+        start, end = int(p['seg_start'][s]), int(p['seg_start'][s]) + ln
         n_units = (ln + 7) // 8
         unit_bytes = bw if bw <= 4 else 8
         for u0 in range(0, n_units, 4):
             if m >= MAX_STEPS:
                 raise ValueError("segment table needs more MFMA steps than the plan holds")
-            p['step'][m] = (int(p['seg_pack_off'][s]) + u0 * unit_bytes, unit_bytes,
-                            2 * bw if bw <= 4 else 0, bw, s, int(u0 + 4 >= n_units),
-                            min(4, n_units - u0), int(p['seg_start'][s]) + u0 * 8)
+            nu = min(4, n_units - u0)
+            off0 = int(p['seg_pack_off'][s]) + u0 * unit_bytes
+            p['step'][m] = (off0, unit_bytes, 2 * bw if bw <= 4 else 0, bw, s,
+                            int(u0 + 4 >= n_units), nu, start + u0 * 8)
+            for g in range(4):
+                gg = min(g, nu - 1)
+                table = LUT_K[bw] if bw <= 4 else LUT_KRAW + (bw - 5) * 512
+                mask = 7 * 4 if bw == 4 else (31 * 4 if bw <= 3 else 0)
+                q_off = 0
+                if g < nu:
+                    d0 = start + (u0 + g) * 8
+                    p['qunit_dim'][unit], p['qunit_len'][unit] = d0, min(8, end - d0)
+                    q_off = 16 * unit
+                    unit += 1
+                p['steptab'][m, g] = (off0 + gg * unit_bytes, 0, table, mask,
+                                      2 * bw if bw <= 4 else 0, 5 if bw == 4 else 7, s * 128, q_off)
+            n_packed += bw <= 4
             m += 1
     p['n_steps'] = m
+    p['n_packed_steps'] = n_packed
+
+    img = np.zeros(LUT_IMAGE_BYTES // 4, dtype=np.uint32)
+    for s in range(int(p['n_seg'])):
+        bw = int(p['seg_bw'][s])
+        cb = p['k_codebook_f16'][s]
+        if bw <= 4:
+            t = _pair_table(cb, bw)
+            img[LUT_K[bw] // 4:LUT_K[bw] // 4 + t.size] = t
+        else:
+            raw = np.zeros(256, dtype=np.uint16)
+            raw[:1 << bw] = cb[:1 << bw]
+            o = (LUT_KRAW + (bw - 5) * 512) // 4
+            img[o:o + 128] = raw.view(np.uint32)
+    vb = int(p['v_bits'])
+    if 1 <= vb <= 4:
+        t = _pair_table(p['v_lut_f16'], vb)
+        img[LUT_V // 4:LUT_V // 4 + t.size] = t
+    p['lut_image'] = img
 
 
 def build_head_plan(quantizer) -> np.ndarray:

@@ -29,6 +29,14 @@ extern "C" {
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
 #define BGTQ_MAX_STEPS     12    /* MFMA steps of one K record, see bgtq_head_plan.step */
+/* byte offsets inside bgtq_head_plan.lut_image (= LDS offsets in the decode kernel) */
+#define BGTQ_LUT_K1      0                       /* 4 entries   x 32 replicas */
+#define BGTQ_LUT_K2      512                     /* 16 entries  x 32 replicas */
+#define BGTQ_LUT_K3      2560                    /* 64 entries  x 32 replicas */
+#define BGTQ_LUT_K4      10752                   /* 256 entries x 8 replicas  */
+#define BGTQ_LUT_KRAW    18944                   /* 4 tables x 256 fp16       */
+#define BGTQ_LUT_V       20992                   /* V pair table, up to 8192 B */
+#define BGTQ_LUT_IMAGE_BYTES 29184
 
 /* error codes (negative); positive return values are hipError_t */
 #define BGTQ_OK            0
@@ -96,6 +104,35 @@ typedef struct bgtq_head_plan {
     int32_t  n_steps;
     int32_t  reserved1[3];
     int32_t  step[BGTQ_MAX_STEPS][8];
+
+    /*
+     * The same schedule in the form the MFMA decode kernel copies into LDS, built
+     * on the host so that a work-group starts streaming right away.
+     *
+     * steptab[m][g] (step m, lane group g = unit g of the step, units past the
+     * step's last real unit repeat that unit and point at query unit 0):
+     *   [0] byte offset of the unit in the record   [1] 0
+     *   [2] byte offset of the unit's table in lut_image   [3] bank-replica mask
+     *       (lane*4 & mask selects the replica)
+     *   [4] bits per code pair (0: raw bytes)        [5] log2 of the table's entry stride
+     *   [6] byte offset of the segment's norm row, segment * 128
+     *   [7] byte offset of the unit's query operand, 16 * query unit
+     * Query units: unit 0 is all zero; unit u >= 1 covers packed dims
+     * [qunit_dim[u], qunit_dim[u] + qunit_len[u]), zero padded to 8 dims.
+     *
+     * lut_image: pair tables, entry (c0 | c1 << bw) = fp16 centroid pair
+     * (c0 in the low half), every entry replicated over consecutive dwords so
+     * that lanes with different codes hit different LDS banks:
+     *   K bw 1..3 at BGTQ_LUT_K1/K2/K3, 32 replicas; K bw 4 at BGTQ_LUT_K4, 8 replicas;
+     *   K bw 5..8: 256 single fp16 entries each at BGTQ_LUT_KRAW + (bw - 5) * 512
+     *   (0 beyond 2^bw); V table for v_bits at BGTQ_LUT_V (replicas as for K).
+     */
+    int32_t  n_packed_steps;       /* steps with bw <= 4 (they come first) */
+    int32_t  reserved2[3];
+    uint32_t steptab[BGTQ_MAX_STEPS][4][8];
+    int32_t  qunit_dim[32];
+    int32_t  qunit_len[32];
+    uint32_t lut_image[BGTQ_LUT_IMAGE_BYTES / 4];
 } bgtq_head_plan;
 
 /* sizeof(bgtq_head_plan) as the library was compiled; the host mirror checks it. */

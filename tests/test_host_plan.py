@@ -210,6 +210,68 @@ def test_plan_struct_mirrors_the_quantizer():
     assert np.allclose(p['v_rot'].reshape(128, 128), p['v_rot_T'].reshape(128, 128).T)
 
 
+@pytest.mark.parametrize("seed,min_bits,max_bits,budget", [(9, 1, 7, 200), (4, 0, 4, 128), (5, 1, 5, 192)])
+def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, budget):
+    """The MFMA step schedule and the LDS table image in the plan, checked against what
+    they stand for: every packed dim of every segment is read exactly once through a
+    query unit, unit byte offsets walk each segment's stream, and a pair-table entry
+    (c0 | c1 << bw) holds the two fp16 centroids, in every bank replica."""
+    from blockgtq_amd import plan as P
+    q, _ = make_quantizer(seed=seed, min_bits=min_bits, max_bits=max_bits, budget=budget)
+    p = q.plan()[0]
+    n_seg, n_steps = int(p['n_seg']), int(p['n_steps'])
+    assert 1 <= n_steps <= P.MAX_STEPS
+    seen = np.zeros(128, dtype=int)
+    unit_of_seg = {s: 0 for s in range(n_seg)}
+    n_packed = 0
+    for m in range(n_steps):
+        off0, ub, pw, bw, s, last, nu, d0 = (int(x) for x in p['step'][m])
+        assert bw == int(p['seg_bw'][s]) and ub == (bw if bw <= 4 else 8) and pw == (2 * bw if bw <= 4 else 0)
+        n_packed += bw <= 4
+        assert n_packed == m + 1 or bw > 4           # raw-byte steps come last
+        for g in range(4):
+            e = [int(x) for x in p['steptab'][m, g]]
+            gg = min(g, nu - 1)
+            u = unit_of_seg[s] + gg
+            assert e[0] == int(p['seg_pack_off'][s]) + u * ub
+            assert e[4] == pw and e[6] == s * 128
+            if g < nu:
+                uid = e[7] // 16
+                assert uid >= 1 and e[7] % 16 == 0
+                a, ln = int(p['qunit_dim'][uid]), int(p['qunit_len'][uid])
+                assert a == int(p['seg_start'][s]) + u * 8
+                assert ln == min(8, int(p['seg_start'][s]) + int(p['seg_len'][s]) - a)
+                seen[a:a + ln] += 1
+            else:
+                assert e[7] == 0                     # padding lanes meet the all-zero query unit
+        unit_of_seg[s] += nu
+        assert last == (unit_of_seg[s] * 8 >= int(p['seg_len'][s]))
+    assert int(p['n_packed_steps']) == n_packed
+    z = int(p['n_zero_dims'])
+    assert (seen[z:] == 1).all() and (seen[:z] == 0).all()
+    img = p['lut_image']
+    for s in range(n_seg):
+        bw = int(p['seg_bw'][s])
+        cb = p['k_codebook_f16'][s]
+        if bw <= 4:
+            rep = 8 if bw == 4 else 32
+            t = img[P.LUT_K[bw] // 4:][:(1 << 2 * bw) * rep].reshape(-1, rep)
+            assert (t == t[:, :1]).all()
+            for c0 in range(1 << bw):
+                for c1 in range(1 << bw):
+                    assert int(t[c0 | (c1 << bw), 0]) == int(cb[c0]) | (int(cb[c1]) << 16)
+        else:
+            raw = img[(P.LUT_KRAW + (bw - 5) * 512) // 4:][:128].view(np.uint16)
+            assert np.array_equal(raw[:1 << bw], cb[:1 << bw]) and not raw[1 << bw:].any()
+    vb = int(p['v_bits'])
+    rep = 8 if vb == 4 else 32
+    tv = img[P.LUT_V // 4:][:(1 << 2 * vb) * rep].reshape(-1, rep)
+    vl = p['v_lut_f16']
+    for c0 in range(1 << vb):
+        for c1 in range(1 << vb):
+            assert (tv[c0 | (c1 << vb)] == (int(vl[c0]) | (int(vl[c1]) << 16))).all()
+
+
 # ---------------------------------------------------------------- V packing
 @pytest.mark.parametrize("bits", [1, 2, 3, 4])
 def test_v_packing_matches_a_plain_bit_stream(bits):
