@@ -44,6 +44,7 @@ typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
 constexpr int D = BGTQ_D;
@@ -51,6 +52,7 @@ constexpr int MT = 64;             // tokens per wave tile = 4 MFMA row blocks
 constexpr int NBLK = MT / 16;
 constexpr int MAX_STEPS = BGTQ_MAX_STEPS;
 constexpr int MAX_WAVES = 8;
+constexpr int KB = 2;              // K tile buffers per wave: 2 = fetched a whole tile ahead, 1 = refilled right after QK^T
 constexpr int MAX_KN = 8;          // norm columns per token row the staging area can hold
 constexpr int LDS_LIMIT = 160 * 1024;
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
@@ -73,21 +75,34 @@ __host__ __device__ inline TileLayout tile_layout(int krow, int vrow, int kn_st)
     TileLayout t;
     t.kt = (MT * krow + 32 + 15) & ~15;
     t.vt = (MT * vrow + 32 + 15) & ~15;
-    t.knr = (MT * kn_st * 2 + 16 + 15) & ~15;
+    t.knr = (MT * kn_st * 2 + 16 + 16 + 15) & ~15;     // phase + the 8-column over-read of the last row
     t.vnr = MT * 2 + 16;
     t.kbuf = t.kt + t.knr + t.vnr;
     return t;
 }
 
-__device__ inline uint32_t lds_u32(const uint8_t* base, uint32_t off) {
-    return *(const uint32_t*)(base + off);
+// (a & mask) | c in one instruction; the mask travels in a scalar register
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t c) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(c));
+    return r;
 }
 
-// 16 bytes per lane from sbase + voff + IMM into LDS at lds_addr + lane * 16 + IMM.
-template <int IMM>
-__device__ __forceinline__ void dma16(uint32_t voff, const uint8_t* sbase, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3\n"
-                 :: "v"(voff), "s"(sbase), "s"(lds_addr), "n"(IMM) : "memory", "m0");
+// Read through an absolute LDS address.  Going through the `smem` symbol instead
+// costs one extra add per access (the symbol's address is only known at link time).
+template <class T>
+__device__ __forceinline__ T lds_at(uint32_t addr) {
+    return *(const __attribute__((address_space(3))) T*)(uintptr_t)addr;
+}
+
+// 16 bytes per lane from sbase + voff into LDS at lds_addr + lane * 16, for the lanes
+// set in `lanes`.  The execution mask is switched inside the block, so the copy needs
+// no divergent branch around it.
+__device__ __forceinline__ void dma16(uint32_t voff, const uint8_t* sbase, uint32_t lds_addr, uint64_t lanes) {
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0\n"
+                 : "=&s"(saved) : "v"(voff), "s"(sbase), "s"(lds_addr), "s"(lanes) : "memory", "m0");
 }
 
 __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
@@ -100,28 +115,19 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
 // Copies the aligned 16-byte pieces of [src_al, src_al + total) to LDS.  Pieces
 // are aligned, so a piece that holds at least one wanted byte never crosses into
 // a page the range itself does not touch.  Exactly dma_count(total) load
-// instructions are issued (lane 0 takes part in every one of them).
+// instructions are issued: every 1 KB chunk but the last runs with all lanes,
+// the last one with the lanes whose piece still starts inside the range.
 __device__ __forceinline__ int dma_count(int total) { return (total + 1023) >> 10; }
 
 template <int NCH>
 __device__ __forceinline__ void dma_region(const uint8_t* src_al, uint32_t lds_addr, int total, uint32_t voff) {
     src_al = uniform_ptr(src_al);
     lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    const int nch = dma_count(total);
+    const uint64_t last = __builtin_amdgcn_ballot_w64((int)voff < total - (nch - 1) * 1024);
 #pragma unroll
-    for (int c = 0; c < NCH; c++) {
-        if (c * 1024 < total) {
-            if ((int)voff + c * 1024 < total) {
-                const uint8_t* sb = src_al + (c >> 2) * 4096;
-                const uint32_t la = lds_addr + (c >> 2) * 4096;
-                switch (c & 3) {
-                case 0: dma16<0>(voff, sb, la); break;
-                case 1: dma16<1024>(voff, sb, la); break;
-                case 2: dma16<2048>(voff, sb, la); break;
-                default: dma16<3072>(voff, sb, la); break;
-                }
-            }
-        }
-    }
+    for (int c = 0; c < NCH; c++)
+        if (c < nch) dma16(voff, src_al + c * 1024, lds_addr + c * 1024, c == nch - 1 ? last : ~0ull);
 }
 
 // Waits until at most n of the loads issued so far are still in flight.
@@ -143,51 +149,16 @@ __device__ __forceinline__ void wait_loads(int n) {
     }
 }
 
-// U consecutive packed steps, straight line.  Per (step, lane group) the table
-// holds {aligned row offset, byte shift, pair table, bank mask} and
-// {bits per pair, log2 entry stride, norm row offset, query unit offset}.
-// Every step starts from a zero accumulator and is scaled by the fp16 group norm
-// of its token rows in fp32, so segments never mix before the norm is applied.
-template <int U>
-__device__ __forceinline__ void k_packed_steps(float4v (&S)[NBLK], const uint8_t* smem, const uint4* st,
-                                               const uint8_t* qrow, uint32_t kbase, uint32_t kstride,
-                                               uint32_t lane4, const uint8_t* nrm) {
-#pragma unroll
-    for (int u = 0; u < U; u++) {
-        const uint4 e0 = st[u * 8], e1 = st[u * 8 + 1];
-        const half8 Q = *(const half8*)(qrow + e1.w);
-        const uint32_t oa = kbase + e0.x;
-        const uint32_t lb = (lane4 & e0.w) | e0.z;
-        const uint32_t pw = e1.x, pw2 = pw * 2, pw3 = pw * 3, tsh = e1.y;
-#pragma unroll
-        for (int k = 0; k < NBLK; k++) {
-            const uint32_t ad = oa + k * kstride;
-            const uint32_t lo = lds_u32(smem, ad), hi = lds_u32(smem, ad + 4);
-            const uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, e0.y);
-            const uint32_t i0 = __builtin_amdgcn_ubfe(raw, 0, pw), i1 = __builtin_amdgcn_ubfe(raw, pw, pw);
-            const uint32_t i2 = __builtin_amdgcn_ubfe(raw, pw2, pw), i3 = __builtin_amdgcn_ubfe(raw, pw3, pw);
-            const uint4 w = {lds_u32(smem, (i0 << tsh) + lb), lds_u32(smem, (i1 << tsh) + lb),
-                             lds_u32(smem, (i2 << tsh) + lb), lds_u32(smem, (i3 << tsh) + lb)};
-            const float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, w), Q,
-                                                                     (float4v){0, 0, 0, 0}, 0, 0, 0);
-            const half4v n4 = *(const half4v*)(nrm + e1.z + k * 32);
-#pragma unroll
-            for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[r], d[r], S[k][r]);
-        }
-    }
-}
-
 // One step of raw byte codes (bw 5..8): one table read per code.
-__device__ __forceinline__ void k_raw_step(float4v (&S)[NBLK], const uint8_t* smem, const uint4* st,
-                                           const uint8_t* qrow, uint32_t kbase, uint32_t kstride,
-                                           const uint8_t* nrm) {
-    const uint4 e0 = st[0], e1 = st[1];
-    const half8 Q = *(const half8*)(qrow + e1.w);
+__device__ __forceinline__ void k_raw_step(float4v (&S)[NBLK], uint32_t st, uint32_t qrow, uint32_t kbase,
+                                           uint32_t kstride, uint32_t nrm) {
+    const uint4v e0 = lds_at<uint4v>(st), e1 = lds_at<uint4v>(st + 16);
+    const half8 Q = lds_at<half8>(qrow + e1.w);
     const uint32_t oa = kbase + e0.x;
 #pragma unroll
     for (int k = 0; k < NBLK; k++) {
         const uint32_t ad = oa + k * kstride;
-        const uint32_t lo = lds_u32(smem, ad), hi = lds_u32(smem, ad + 4), hi2 = lds_u32(smem, ad + 8);
+        const uint32_t lo = lds_at<uint32_t>(ad), hi = lds_at<uint32_t>(ad + 4), hi2 = lds_at<uint32_t>(ad + 8);
         const uint32_t r0 = __builtin_amdgcn_alignbyte(hi, lo, e0.y);
         const uint32_t r1 = __builtin_amdgcn_alignbyte(hi2, hi, e0.y);
         half8 A;
@@ -195,10 +166,10 @@ __device__ __forceinline__ void k_raw_step(float4v (&S)[NBLK], const uint8_t* sm
         for (int e = 0; e < 8; e++) {
             const uint32_t r = e < 4 ? r0 : r1;
             const uint32_t byte = (r >> ((e & 3) * 8)) & 0xFF;
-            A[e] = __builtin_bit_cast(_Float16, *(const uint16_t*)(smem + e0.z + byte * 2));
+            A[e] = __builtin_bit_cast(_Float16, lds_at<uint16_t>(e0.z + byte * 2));
         }
         const float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Q, (float4v){0, 0, 0, 0}, 0, 0, 0);
-        const half4v n4 = *(const half4v*)(nrm + e1.z + k * 32);
+        const half4v n4 = lds_at<half4v>(nrm + e1.z + k * 32);
 #pragma unroll
         for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[r], d[r], S[k][r]);
     }
@@ -209,7 +180,7 @@ __device__ unsigned long long* g_trace;
 #define TRACE(slot)                                                                              \
     do {                                                                                         \
         if (lane == 0 && (slot) < 64)                                                            \
-            g_trace[(((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + wave) * 64 + (slot)] = \
+            g_trace[(((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + wave) * 64 + (slot)] = \
                 __builtin_readcyclecounter();                                                    \
     } while (0)
 #else
@@ -238,13 +209,12 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     constexpr int vrow = 16 * VBW;
     const int kn_st = (int)a.kn_st;
     const TileLayout tl = tile_layout(krow, vrow, kn_st);
-    uint8_t* vlut = smem + VLUT;
     uint4* steptab = (uint4*)(smem + steptab_off(VBW));
     uint8_t* qpad = smem + qpad_off(VBW);
     const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
-    const uint32_t kbufs_off = waves_off(VBW);                                   // [2][nw] K + norm buffers
-    const uint32_t vbuf_off = kbufs_off + 2 * nw * tl.kbuf + wave * tl.vt;        // [nw] V buffers
-    const uint32_t norm_off = kbufs_off + nw * (2 * tl.kbuf + tl.vt) + wave * WAVE_NORM_BYTES;
+    const uint32_t kbufs_off = waves_off(VBW);                                   // [KB][nw] K + norm buffers
+    const uint32_t vbuf_off = kbufs_off + KB * nw * tl.kbuf + wave * tl.vt;        // [nw] V buffers
+    const uint32_t norm_off = kbufs_off + nw * (KB * tl.kbuf + tl.vt) + wave * WAVE_NORM_BYTES;
     uint8_t* kn_h = smem + norm_off;                                 // fp16 [segment][token]
     float* vn_f = (float*)(kn_h + BGTQ_MAX_SEGMENTS * MT * 2);       // fp32 [token]
     uint8_t* scratch = smem + kbufs_off + nw * tl.kbuf;              // everything past the first K buffers is idle during init
@@ -284,8 +254,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         const uint8_t* img = (const uint8_t*)P.lut_image;
         constexpr int total = BGTQ_LUT_V + vlut_bytes(VBW);
         for (int cc = wave; cc * 1024 < total; cc += nw)
-            if ((int)voff + cc * 1024 < total)
-                dma16<0>(voff, uniform_ptr(img + cc * 1024), __builtin_amdgcn_readfirstlane(smem_lds + cc * 1024));
+            dma16(voff, uniform_ptr(img + cc * 1024), __builtin_amdgcn_readfirstlane(smem_lds + cc * 1024),
+                  __builtin_amdgcn_ballot_w64((int)voff + cc * 1024 < total));
     }
     int k0_loads = 0;
     if (tile < t1) k0_loads = issue_k(tile, 0);
@@ -301,7 +271,6 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         if (hq < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + hq) * a.q_sh + d2 * 2);
         ((uint32_t*)q_s)[i] = v;
     }
-    const int n_seg = min(P.n_seg, BGTQ_MAX_SEGMENTS);
     const int n_steps = min(P.n_steps, MAX_STEPS);
     const int n_packed = min(P.n_packed_steps, n_steps);   // raw-byte steps (bw >= 5) come last
     __syncthreads();
@@ -309,8 +278,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     for (int i = tid; i < n_steps * 4; i += nthr) {        // the row offset depends on the cache's alignment
         const uint32_t* r = st_raw + i * 8;
         const uint32_t o = kph + r[0];
-        steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2], r[3]};
-        steptab[i * 2 + 1] = (uint4){r[4], r[5], r[6], r[7]};
+        steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2] + smem_lds, r[3]};     // table as an absolute LDS address
+        steptab[i * 2 + 1] = (uint4){r[4], r[5], r[6] * MT / 64, r[7]};   // norm rows are MT tokens long here
     }
     for (int i = tid; i < 16 * (QROW / 4); i += nthr) {     // query units, zero padded
         const int hd = i / (QROW / 4), rem = i - hd * (QROW / 4), uid = rem >> 2, pp = rem & 3;
@@ -329,15 +298,16 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 
     const float c2 = a.scale * 1.44269504088896340736f;      // logits go through exp2
     const uint32_t lane4 = (uint32_t)lane * 4;
-    const uint32_t vbank = VBW == 4 ? (lane4 & 28u) : (lane4 & 124u);
+    const uint32_t vbank = smem_lds + (VBW == 4 ? (lane4 & 28u) : (lane4 & 124u));   // V table replica of this lane (LDS is 128-byte aligned)
     constexpr int vshift = VBW == 4 ? 5 : 7;
     const uint32_t rowoff = (uint32_t)li * krow;
     const uint32_t kstride = 16u * krow;
     const uint32_t vc = vph + (uint32_t)li * VBW;
-    const uint32_t vbase = vbuf_off + (vc & ~3u) + (uint32_t)lg * 4 * vrow, v_sh = vc & 3u;
-    const uint4* stl = steptab + lg * 2;
-    const uint8_t* qrow = qpad + li * QROW;
-    const uint8_t* nrm = kn_h + lg * 8;
+    const uint32_t vbase = smem_lds + vbuf_off + (vc & ~3u) + (uint32_t)lg * 4 * vrow, v_sh = vc & 3u;
+    const uint32_t stl = smem_lds + steptab_off(VBW) + lg * 32;          // absolute LDS addresses from here on
+    const uint32_t qrow = smem_lds + qpad_off(VBW) + li * QROW;
+    const uint32_t nrm = smem_lds + norm_off + lg * 8;
+    const uint32_t vnf = smem_lds + norm_off + BGTQ_MAX_SEGMENTS * MT * 2;
 
     float m_ref = -INFINITY;        // reference of head li, in exp2 units; never below a score seen
     float l_part = 0.f;             // this lane's share of the softmax denominator
@@ -349,27 +319,30 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     for (; tile < t1; tile += step_tiles, which ^= 1) {
         const int nt = min(MT, t1 - tile);
         const bool more = tile + step_tiles < t1;
-        const uint32_t kbuf = kbufs_off + (which * nw + wave) * tl.kbuf;
+        const uint32_t kbuf = kbufs_off + ((KB == 2 ? which : 0) * nw + wave) * tl.kbuf;
         TRACE(8 + trace_j * 8 + 0);
         wait_loads(v_loads);                                 // K records and norms of this tile are in LDS
         __builtin_amdgcn_wave_barrier();
         TRACE(8 + trace_j * 8 + 1);
         // ---- norms of the tile: lane = token; read raw, start the next K tile, then store
         //      them as fp16 [segment][token] and fp32 V norms -------------------------------------
+        // All 8 columns are moved whatever the head's segment count: columns past the row end
+        // read neighbouring bytes of the staging area, land in rows no step refers to, and the
+        // copy stays free of branches.
         uint16_t nraw[BGTQ_MAX_SEGMENTS];
         {
-            const uint8_t* kraw = smem + kbuf + tl.kt + knph + (uint32_t)lane * kn_st * 2;
+            const uint32_t kraw = smem_lds + kbuf + tl.kt + knph + (uint32_t)lane * kn_st * 2;
 #pragma unroll
-            for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++)
-                if (s < n_seg) nraw[s] = *(const uint16_t*)(kraw + s * 2);
+            for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) nraw[s] = lds_at<uint16_t>(kraw + s * 2);
         }
-        const uint16_t vraw = *(const uint16_t*)(smem + kbuf + tl.kt + tl.knr + vnph + lane * 2);
+        const uint16_t vraw = lds_at<uint16_t>(smem_lds + kbuf + tl.kt + tl.knr + vnph + lane * 2);
         int k_loads = 0;
-        if (more) k_loads = issue_k(tile + step_tiles, which ^ 1);
+        if (KB == 2 && more) k_loads = issue_k(tile + step_tiles, which ^ 1);
+        if (MT == 64 || lane < MT) {
 #pragma unroll
-        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++)
-            if (s < n_seg) *(uint16_t*)(kn_h + (s * MT + lane) * 2) = nraw[s];
-        vn_f[lane] = lane < nt ? bgtq_h2f(vraw) : 0.f;
+            for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) *(uint16_t*)(kn_h + (s * MT + lane) * 2) = nraw[s];
+            vn_f[lane] = lane < nt ? bgtq_h2f(vraw) : 0.f;
+        }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
         TRACE(8 + trace_j * 8 + 2);
@@ -379,13 +352,77 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 #pragma unroll
         for (int k = 0; k < NBLK; k++) S[k] = (float4v){0, 0, 0, 0};
         {
-            const uint32_t kbase = kbuf + rowoff;
-            int m = 0;
-            for (; m + 4 <= n_packed; m += 4) k_packed_steps<4>(S, smem, stl + m * 8, qrow, kbase, kstride, lane4, nrm);
-            if (m + 2 <= n_packed) { k_packed_steps<2>(S, smem, stl + m * 8, qrow, kbase, kstride, lane4, nrm); m += 2; }
-            if (m < n_packed) { k_packed_steps<1>(S, smem, stl + m * 8, qrow, kbase, kstride, lane4, nrm); m += 1; }
-            for (; m < n_steps; m++) k_raw_step(S, smem, stl + m * 8, qrow, kbase, kstride, nrm);
+            // Software pipeline over the packed steps: while the table reads of step m are
+            // in flight, the parameters, raw codes and query unit of step m+1 are fetched.
+            // The scheduling barriers keep the compiler from folding the stages back into
+            // one dependent chain per row block.
+            const uint32_t kbase = smem_lds + kbuf + rowoff;
+            uint4v e0 = lds_at<uint4v>(stl), e1 = lds_at<uint4v>(stl + 16);
+            uint32_t rlo[NBLK] = {}, rhi[NBLK] = {};
+            half8 Q = {};
+            if (n_packed > 0) {
+                const uint32_t oa = kbase + e0.x;
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) {
+                    rlo[k] = lds_at<uint32_t>(oa + k * kstride);
+                    rhi[k] = lds_at<uint32_t>(oa + k * kstride + 4);
+                }
+                Q = lds_at<half8>(qrow + e1.w);
+            }
+            for (int m = 0; m < n_packed; m++) {
+                const int mn = min(m + 1, n_steps - 1);
+                const uint4v f0 = lds_at<uint4v>(stl + mn * 128), f1 = lds_at<uint4v>(stl + mn * 128 + 16);   // A: parameters of the next step
+                __builtin_amdgcn_sched_barrier(0);
+                // B: bit fields -> table reads of this step, norms of its segment
+                const uint32_t lb = (lane4 & e0.w) | e0.z;
+                const uint32_t pw = e1.x, pw2 = pw * 2, pw3 = pw * 3, tsh = e1.y;
+                uint4v w[NBLK];
+                half4v n4[NBLK];
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) {
+                    const uint32_t raw = __builtin_amdgcn_alignbyte(rhi[k], rlo[k], e0.y);
+                    const uint32_t i0 = __builtin_amdgcn_ubfe(raw, 0, pw), i1 = __builtin_amdgcn_ubfe(raw, pw, pw);
+                    const uint32_t i2 = __builtin_amdgcn_ubfe(raw, pw2, pw), i3 = __builtin_amdgcn_ubfe(raw, pw3, pw);
+#ifdef BGTQ_EXPERIMENT_NOKLUT
+                    w[k] = (uint4v){(i0 << tsh) + lb, (i1 << tsh) + lb, (i2 << tsh) + lb, (i3 << tsh) + lb};
+#else
+                    w[k] = (uint4v){lds_at<uint32_t>((i0 << tsh) + lb), lds_at<uint32_t>((i1 << tsh) + lb),
+                                   lds_at<uint32_t>((i2 << tsh) + lb), lds_at<uint32_t>((i3 << tsh) + lb)};
+#endif
+                }
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) n4[k] = lds_at<half4v>(nrm + e1.z + k * 32);
+                __builtin_amdgcn_sched_barrier(0);
+                // C: raw codes and query unit of the next step
+                uint32_t nlo[NBLK], nhi[NBLK];
+                const uint32_t oan = kbase + f0.x;
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) {
+                    nlo[k] = lds_at<uint32_t>(oan + k * kstride);
+                    nhi[k] = lds_at<uint32_t>(oan + k * kstride + 4);
+                }
+                const half8 Qn = lds_at<half8>(qrow + f1.w);
+                __builtin_amdgcn_sched_barrier(0);
+                // D: one MFMA per row block from a zero accumulator, scaled by the fp16 group
+                //    norm of its token rows in fp32
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) {
+                    const float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, w[k]), Q,
+                                                                             (float4v){0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[k][r], d[r], S[k][r]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                e0 = f0;
+                e1 = f1;
+                Q = Qn;
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) { rlo[k] = nlo[k]; rhi[k] = nhi[k]; }
+            }
+            TRACE(8 + trace_j * 8 + 6);
+            for (int m = n_packed; m < n_steps; m++) k_raw_step(S, stl + m * 128, qrow, kbase, kstride, nrm);
         }
+        if (KB == 1 && more) k_loads = issue_k(tile + step_tiles, 0);   // all reads of the K buffer are done
         TRACE(8 + trace_j * 8 + 3);
 
         // ---- online softmax: lane (head li, group lg) holds tokens 16k + 4lg + r ------
@@ -420,40 +457,57 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         wait_loads(k_loads);                                 // the V records of this tile are in LDS
         __builtin_amdgcn_wave_barrier();
 
+        // values: lane (j = li, group lg) decodes unit j of its 8 tokens per half tile.  Raw
+        // codes are fetched one half ahead; the exponentials run while the table reads fly.
+        uint32_t vlo[8], vhi[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            const int tk = (r >> 2) * 16 + (r & 3);                       // + 4lg, folded into vbase
+            vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
+            vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
+        }
 #pragma unroll
         for (int half = 0; half < NBLK / 2; half++) {
-            // P * v_norm is formed in fp32 and rounded to fp16 once
-            half8 Pm;
-            {
-                const float4v vlo = *(const float4v*)(vn_f + half * 32 + lg * 4);        // tokens 4lg .. 4lg+3
-                const float4v vhi = *(const float4v*)(vn_f + half * 32 + 16 + lg * 4);   // tokens 16+4lg ..
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int k = half * 2 + (e >> 1), r = (e & 1) * 2;
-                    const float p0 = __builtin_amdgcn_exp2f(fmaf(S[k][r], c2, -m_ref));
-                    const float p1 = __builtin_amdgcn_exp2f(fmaf(S[k][r + 1], c2, -m_ref));
-                    l_part += p0 + p1;
-                    const float4v vn4 = (e >> 1) ? vhi : vlo;
-                    const float2v pv = {p0 * vn4[r], p1 * vn4[r + 1]};
-                    const half2v ph = __builtin_convertvector(pv, half2v);
-                    Pm[2 * e] = ph[0];
-                    Pm[2 * e + 1] = ph[1];
-                }
-            }
-            // values: lane (j = li, group lg) decodes unit j of its 8 tokens
+            const float4v vn_lo = lds_at<float4v>(vnf + (half * 32 + lg * 4) * 4);        // tokens 4lg .. 4lg+3
+            const float4v vn_hi = lds_at<float4v>(vnf + (half * 32 + 16 + lg * 4) * 4);   // tokens 16+4lg ..
             uint32_t W[8][4];
 #pragma unroll
             for (int r = 0; r < 8; r++) {
-                const int tk = half * 32 + (r >> 2) * 16 + (r & 3);      // + 4lg, folded into vbase
-                const uint32_t ad = vbase + (uint32_t)tk * vrow;
-                const uint32_t lo = lds_u32(smem, ad), hi = lds_u32(smem, ad + 4);
-                const uint32_t raw = __builtin_amdgcn_alignbyte(hi, lo, v_sh);
+                const uint32_t raw = __builtin_amdgcn_alignbyte(vhi[r], vlo[r], v_sh);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const uint32_t idx = __builtin_amdgcn_ubfe(raw, e * 2 * VBW, 2 * VBW);
-                    W[r][e] = lds_u32(vlut, (idx << vshift) + vbank);
+                    // shift the pair field to its place in the table address, then one and-or
+                    // merges the bank replica (the compiler would spend an and plus an add)
+                    constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
+                    const int fp = e * 2 * VBW;
+                    const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
+                    W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank) + VLUT);   // + VLUT rides in the offset field
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (half + 1 < NBLK / 2) {
+#pragma unroll
+                for (int r = 0; r < 8; r++) {
+                    const int tk = (half + 1) * 32 + (r >> 2) * 16 + (r & 3);
+                    vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
+                    vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
+                }
+            }
+            // P * v_norm is formed in fp32 and rounded to fp16 once
+            half8 Pm;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int k = half * 2 + (e >> 1), r = (e & 1) * 2;
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(S[k][r], c2, -m_ref));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(S[k][r + 1], c2, -m_ref));
+                l_part += p0 + p1;
+                const float4v vn4 = (e >> 1) ? vn_hi : vn_lo;
+                const float2v pv = {p0 * vn4[r], p1 * vn4[r + 1]};
+                const half2v ph = __builtin_convertvector(pv, half2v);
+                Pm[2 * e] = ph[0];
+                Pm[2 * e + 1] = ph[1];
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 half8 Bv;
@@ -467,6 +521,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                 }
                 acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Pm, Bv, acc[e], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();     // V buffer and norm areas are rewritten from here on
@@ -516,7 +571,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 // LDS bytes of a work-group of nw waves
 size_t mfma_smem_bytes(int vbw, int krow, int vrow, int kn_st, int nw) {
     const TileLayout tl = tile_layout(krow, vrow, kn_st);
-    size_t need = (size_t)waves_off(vbw) + (size_t)nw * (2 * tl.kbuf + tl.vt + WAVE_NORM_BYTES);
+    size_t need = (size_t)waves_off(vbw) + (size_t)nw * (KB * tl.kbuf + tl.vt + WAVE_NORM_BYTES);
     size_t scratch = (size_t)waves_off(vbw) + (size_t)nw * tl.kbuf + INIT_SCRATCH;
     size_t merge = (size_t)nw * (32 + 16 * D) * 4;
     size_t s = need > scratch ? need : scratch;
