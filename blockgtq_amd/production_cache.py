@@ -90,15 +90,23 @@ class BlockGTQProductionCache:
         li = layer_idx
         S = k.shape[2]
         t_pos = self._seq_lens if self._seq_lens is not None else self.seq_len
-        self._encode_batched(li, k, v, t_pos)
         T = self.seq_len + S
         plans = self.batched_args[li]['plans']
         B = q.shape[0]
         q3 = q.reshape(B, self.nq, self.hd)
         if q3.dtype != torch.float16:
             q3 = q3.to(torch.float16)
-        if not self.quantizers[li][0]._q_perm_baked:
-            q3 = ops.rotate_q(plans, q3.contiguous(), self.nkv)
+        if self.quantizers[li][0]._q_perm_baked:
+            self._encode_batched(li, k, v, t_pos)
+        else:                        # encode K, V and rotate the queries in one launch
+            k16 = k if k.dtype == torch.float16 else k.to(torch.float16)
+            v16 = v if v.dtype == torch.float16 else v.to(torch.float16)
+            k16 = k16 if k16.stride(-1) == 1 else k16.contiguous()
+            v16 = v16 if v16.stride(-1) == 1 else v16.contiguous()
+            q3 = ops.decode_prepare(
+                plans, k16, v16, q3.contiguous(), self.k_packed[li], self.k_norms[li],
+                self.v_packed[li], self.v_norms[li], t_pos, self.k_bytes_per_tok, self.max_ng,
+                self.vpb, self.nkv, self._k_layout, self._v_layout)
         lens = self._seq_lens + S if self._seq_lens is not None else None
         out = ops.decode_attention(
             plans, q3.contiguous(), self.k_packed[li], self.k_norms[li],
