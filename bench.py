@@ -42,16 +42,17 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_baseline(mgr, w, q_rot_layer0, seconds):
+def cpu_baseline(mgr, w, q_rot_layer0, seconds, packed_lens):
     """Time the CPU checker on (batch row, KV head) pairs of layer 0 until about
-    ``seconds`` of wall time are spent; scale to a full layer."""
+    ``seconds`` of wall time are spent; scale to a full layer.  ``packed_lens[b]`` is
+    the number of packed tokens row b attends to."""
     import numpy as np
     import oracle
     from concurrent.futures import ThreadPoolExecutor
 
     oracle.build()
     cores = min(os.cpu_count() or 1, 16)
-    T = mgr.seq_len
+    T = max(packed_lens)
     li = 0
     kp = mgr._k_packed[li, :, :, :T].cpu().numpy()
     kn = mgr._k_norms[li, :, :, :T].cpu().numpy()
@@ -65,9 +66,10 @@ def cpu_baseline(mgr, w, q_rot_layer0, seconds):
     def one(bh):
         b, h = bh
         q8 = mgr.quantizers[li][h]
+        n = packed_lens[b]
         oracle.decode_attn(plans[h:h + 1], qr[b, h * gqa:(h + 1) * gqa],
-                           kp[b, h][:, :q8._total_packed_bytes], kn[b, h][:, :max(q8._n_groups, 1)],
-                           vp[b, h], vn[b, h], n_splits=1)
+                           kp[b, h][:n, :q8._total_packed_bytes], kn[b, h][:n, :max(q8._n_groups, 1)],
+                           vp[b, h][:n], vn[b, h][:n], n_splits=1)
 
     one(pairs[0])                                   # page in
     done, t0 = 0, time.perf_counter()
@@ -79,7 +81,7 @@ def cpu_baseline(mgr, w, q_rot_layer0, seconds):
     dt = time.perf_counter() - t0
     per_layer_us = dt / done * len(pairs) * 1e6
     return {"value": per_layer_us, "unit": "us/layer/step", "cores": cores, "kind": "port",
-            "sample": f"{done} (batch row, KV head) attention calls of layer 0 at T={T} "
+            "sample": f"{done} (batch row, KV head) packed-attention calls of layer 0 at up to T={T} "
                       f"({done / len(pairs):.2f} layer-steps), scalar C checker, {cores} threads"}
 
 
@@ -115,6 +117,10 @@ def main():
     qs = [wl.draw_q(w, li, dev, T) for li in range(L)]
     kvs = [wl.draw_kv(w, energies[li], 1, 10_000_000 + li, dev, pos0=T) for li in range(L)]
     n_splits = args.splits or ops.default_splits(w.batch, w.n_kv, T + 1)
+    if not args.splits and (w.seq_lens is not None or w.window):
+        n_splits = max(n_splits, min(4 * n_splits, (T + 511) // 512))      # ragged rows: finer partitions
+    if mgr.buffered and mgr._seq_lens is None:
+        mgr.set_seq_lens(seq_lens)
     mgr.n_splits = n_splits
     outs = [None] * L
 
@@ -156,7 +162,12 @@ def main():
               for li in range(L)]
     part_out, part_lse = mgr._ws.get(w.batch, w.n_q, n_splits, dev)
     lib = _capi.lib()
-    lens_dev = mgr._seq_lens
+    # tokens of the packed cache each row attends to once this step's token is in
+    fp16_rows = (mgr.n_sink + mgr.window) if mgr.buffered else 0
+    packed_lens = [max(t + 1 - fp16_rows, 0) for t in seq_lens]
+    ragged = mgr.buffered or w.seq_lens is not None
+    lens_dev = torch.tensor(packed_lens, dtype=torch.int32, device=dev) if ragged else None
+    Tk = max(packed_lens)
 
     def attn_only(li):
         _capi.check(lib.bgtq_decode_attn(
@@ -165,7 +176,7 @@ def main():
             _capi.ptr(mgr._k_norms[li]), *mgr._k_norms[li].stride()[:3],
             _capi.ptr(mgr._v_packed[li]), *mgr._v_packed[li].stride()[:3], mgr._vpb,
             _capi.ptr(mgr._v_norms[li]), *mgr._v_norms[li].stride()[:3],
-            _capi.ptr(lens_dev), T + 1, w.batch, w.n_kv, mgr.gqa_ratio, n_splits,
+            _capi.ptr(lens_dev), Tk, w.batch, w.n_kv, mgr.gqa_ratio, n_splits,
             _capi.ptr(part_out), _capi.ptr(part_lse), _plan.K_BITPACKED, _plan.V_BITPACKED,
             mgr.scale, _capi.stream_ptr()), "bgtq_decode_attn")
 
@@ -198,6 +209,7 @@ def main():
                    "head_dim": w.head_dim, "batch": w.batch, "context": T,
                    "k_bits_avg": w.k_bits, "v_bits": w.v_bits, "n_splits": n_splits,
                    "k_layout": "bit-packed", "v_layout": "bit-packed",
+                   "fp16_sink_tokens": mgr.n_sink, "fp16_recent_window": mgr.window,
                    "step": "append(encode K,V) + rotate Q + attention + merge, per layer",
                    "graph": graph is not None},
         "tokens_per_s": round(tokens_per_s, 1),
@@ -211,7 +223,7 @@ def main():
                      "avg_launch_us": round(attn_us, 3)},
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(mgr, w, q_rots[0], args.cpu_seconds)
+        out["cpu_baseline"] = cpu_baseline(mgr, w, q_rots[0], args.cpu_seconds, packed_lens)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -88,6 +88,10 @@ def decode_attention(plans: torch.Tensor, q_rot: torch.Tensor,
     L = _capi.lib()
     if n_splits <= 0:
         n_splits = L.bgtq_default_splits(B, n_kv, max(T, 1))
+        if seq_lens is not None:
+            # ragged rows: smaller partitions let the short rows' compute units pick up
+            # pieces of the long rows
+            n_splits = max(n_splits, min(4 * n_splits, (T + 511) // 512))
     ws = workspace or _default_ws
     part_out, part_lse = ws.get(B, n_q, n_splits, q_rot.device)
     st = _capi.stream_ptr(q_rot.device)
@@ -149,3 +153,29 @@ def decode_prepare(plans: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q: tor
         _capi.ptr(q), q.stride(0), q.stride(1), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1),
         n_q // n_kv, _capi.stream_ptr(k.device)), "bgtq_decode_prepare")
     return q_rot
+
+
+@torch.no_grad()
+def window_attention(q: torch.Tensor, kbuf: torch.Tensor, vbuf: torch.Tensor,
+                     lens: Optional[torch.Tensor], n_kv: int, scale: Optional[float] = None):
+    """Dense fp16 attention partial over buffered (unquantised) tokens.
+
+    q (B, n_q, D) fp16 ORIGINAL queries; kbuf / vbuf (B, n_kv, W, D) fp16 with a
+    common layout; ``lens`` int32 device tensor (B,) of valid rows or None.
+    Returns (partial (B, n_q, D) fp32, lse (B, n_q) fp32) for ``decode_attention``'s
+    ``extra_out`` / ``extra_lse``."""
+    _capi.require_cuda(q, "q")
+    assert q.dtype == torch.float16 and q.stride(-1) == 1
+    assert kbuf.dtype == torch.float16 and vbuf.dtype == torch.float16
+    assert kbuf.shape == vbuf.shape and kbuf.stride() == vbuf.stride() and kbuf.stride(-1) == 1
+    B, n_q, D = q.shape
+    W = kbuf.shape[2]
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    po = torch.empty((B, n_q, D), dtype=torch.float32, device=q.device)
+    pl = torch.empty((B, n_q), dtype=torch.float32, device=q.device)
+    _capi.check(_capi.lib().bgtq_window_attn(
+        _capi.ptr(q), q.stride(0), q.stride(1), _capi.ptr(kbuf), _capi.ptr(vbuf),
+        kbuf.stride(0), kbuf.stride(1), kbuf.stride(2), _capi.ptr(lens), W,
+        B, n_kv, n_q // n_kv, scale, _capi.ptr(po), _capi.ptr(pl), _capi.stream_ptr(q.device)),
+        "bgtq_window_attn")
+    return po, pl

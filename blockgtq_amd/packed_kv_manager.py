@@ -13,6 +13,13 @@ partition); nothing loops over heads and nothing is captured into graphs
 because no step needs a per-head kernel variant.  Per-row sequence lengths are
 supported (``set_seq_lens``) for ragged batches; by default every row shares
 ``seq_len`` as in the reference.
+
+With ``n_sink`` / ``recent_window`` set, the manager keeps the three-region
+layout of the reference's buffered mode (blockgtq/unaccelerated.py:163-244, block
+size 1): the first ``n_sink`` tokens and the most recent ``recent_window`` tokens
+stay fp16 in a small per-layer buffer, everything between lives in the packed
+cache.  Every append moves the token that falls out of the window into the packed
+cache; attention runs over the packed part and the buffer and merges the two.
 """
 import math
 
@@ -28,7 +35,8 @@ class BlockGTQKVManager:
     def __init__(self, n_layers: int, n_q_heads: int, n_kv_heads: int,
                  head_dim: int, max_seq_len: int, batch_size: int = 1,
                  k_avg_bits: float = 3.0, v_bits: int = 3, device='cuda',
-                 min_bits: int = 1, max_bits: int = 8, rotation_threshold: int = 2):
+                 min_bits: int = 1, max_bits: int = 8, rotation_threshold: int = 2,
+                 n_sink: int = 0, recent_window: int = 0):
         self.n_layers = n_layers
         self.n_q = n_q_heads
         self.n_kv = n_kv_heads
@@ -54,6 +62,13 @@ class BlockGTQKVManager:
         self._k_packed = self._k_norms = self._v_packed = self._v_norms = None
         self._ws = ops.Workspace()
         self.n_splits = 0              # partitions per (row, KV head); 0 = library default
+        # with-buffer mode: fp16 sink tokens + ring of recent tokens, (L, B, n_kv, n_sink + window, D)
+        self.n_sink, self.window = int(n_sink), int(recent_window)
+        self.buffered = self.window > 0
+        if self.n_sink and not self.buffered:
+            raise ValueError("n_sink needs recent_window > 0")
+        self._buf_k = self._buf_v = None
+        self._step_src, self._step_idx = None, None     # per-step index tensors of the buffered append
 
     # ------------------------------------------------------------ calibration
     def calibrate(self, layer_idx: int, q_data: torch.Tensor, k_data: torch.Tensor):
@@ -101,6 +116,10 @@ class BlockGTQKVManager:
         self._k_norms = torch.zeros(*shape, ng, dtype=torch.float16, device=dev)
         self._v_packed = torch.zeros(*shape, self._vpb, dtype=torch.uint8, device=dev)
         self._v_norms = torch.zeros(*shape, dtype=torch.float16, device=dev)
+        if self.buffered:
+            bshape = (self.n_layers, self.B, self.n_kv, self.n_sink + self.window, self.hd)
+            self._buf_k = torch.zeros(bshape, dtype=torch.float16, device=dev)
+            self._buf_v = torch.zeros(bshape, dtype=torch.float16, device=dev)
 
     def set_seq_lens(self, seq_lens):
         """Per-row visible lengths (ragged batch); ``None`` returns to one shared length."""
@@ -139,11 +158,86 @@ class BlockGTQKVManager:
             self._encode_kv(li, k, v, 0)
         self.seq_len = T
 
+    # ------------------------------------------------------- with-buffer mode
+    @torch.no_grad()
+    def fill_buffered(self, layer_idx: int, k: torch.Tensor, v: torch.Tensor, lens=None):
+        """Load a layer's prefix in with-buffer mode.  k, v (B, n_kv, Tmax, D) post-RoPE; row b
+        holds ``lens[b]`` tokens (all ``Tmax`` when ``lens`` is None), each at least
+        ``n_sink + recent_window`` long.  Call ``set_seq_lens(lens)`` afterwards."""
+        assert self.buffered
+        self._ensure_storage()
+        li, ns, w = layer_idx, self.n_sink, self.window
+        B, _, Tmax, _ = k.shape
+        dev = k.device
+        lens_t = (torch.full((B,), Tmax, dtype=torch.long, device=dev) if lens is None
+                  else torch.as_tensor(lens, dtype=torch.long).to(dev))
+        assert int(lens_t.min()) >= ns + w and int(lens_t.max()) <= Tmax
+        k16, v16 = k.to(torch.float16), v.to(torch.float16)
+        if Tmax - w > ns:          # tokens between sink and window, packed index = position - n_sink
+            self._encode_kv(li, k16[:, :, ns:Tmax - w], v16[:, :, ns:Tmax - w], 0)
+        self._buf_k[li, :, :, :ns] = k16[:, :, :ns]
+        self._buf_v[li, :, :, :ns] = v16[:, :, :ns]
+        pos = lens_t[:, None] - w + torch.arange(w, device=dev)[None, :]           # (B, w) positions
+        slot = ns + (pos - ns) % w
+        ar = torch.arange(B, device=dev)[:, None]
+        self._buf_k[li][ar, :, slot] = k16[ar, :, pos]
+        self._buf_v[li][ar, :, slot] = v16[ar, :, pos]
+
+    def _buffered_step_indices(self):
+        """Index tensors of one buffered append, shared by all layers of a step."""
+        if self._step_src is self._seq_lens:
+            return self._step_idx
+        ns, w = self.n_sink, self.window
+        p = self._seq_lens.to(torch.long)                  # position of the token being appended
+        rel = p - ns
+        slot = torch.where(p < ns, p, ns + rel.clamp(min=0) % w)
+        flush = rel >= w                                    # the slot holds a token that leaves the window
+        scratch_row = self.max_T - 1                        # records of rows that flush nothing go here
+        t_flush = torch.where(flush, rel - w, torch.full_like(rel, scratch_row)).to(torch.int32)
+        packed_len = (p + 1 - ns - w).clamp(min=0).to(torch.int32)
+        buf_len = (p + 1).clamp(max=ns + w).to(torch.int32)
+        ar = torch.arange(self.B, device=p.device)
+        self._step_src = self._seq_lens
+        self._step_idx = (ar, slot, t_flush, packed_len, buf_len)
+        return self._step_idx
+
+    @torch.no_grad()
+    def _append_and_attend_buffered(self, li, q, k_new, v_new):
+        assert k_new.shape[2] == 1, "with-buffer decode appends one token per sequence"
+        self._ensure_storage()
+        if self._seq_lens is None:
+            self.set_seq_lens([self.seq_len] * self.B)
+        assert self.seq_len + 1 - self.n_sink - self.window < self.max_T - 1
+        ar, slot, t_flush, packed_len, buf_len = self._buffered_step_indices()
+        plans = self._batched_args[li]['plans']
+        B = q.shape[0]
+        q3 = q.reshape(B, self.n_q, self.hd).to(torch.float16).contiguous()
+        bk, bv = self._buf_k[li], self._buf_v[li]
+        old_k = bk[ar, :, slot].unsqueeze(2)                # (B, n_kv, 1, D): tokens leaving the window
+        old_v = bv[ar, :, slot].unsqueeze(2)
+        q_rot = ops.decode_prepare(
+            plans, old_k, old_v, q3, self._k_packed[li], self._k_norms[li],
+            self._v_packed[li], self._v_norms[li], t_flush, self._k_row,
+            self._k_norms.shape[-1], self._vpb, self.n_kv, _plan.K_BITPACKED, _plan.V_BITPACKED)
+        bk[ar, :, slot] = k_new[:, :, 0].to(torch.float16)
+        bv[ar, :, slot] = v_new[:, :, 0].to(torch.float16)
+        ext_out, ext_lse = ops.window_attention(q3, bk, bv, buf_len, self.n_kv, self.scale)
+        T = max(self.seq_len + 1 - self.n_sink - self.window, 1)
+        out = ops.decode_attention(
+            plans, q_rot, self._k_packed[li], self._k_norms[li],
+            self._v_packed[li], self._v_norms[li], T, seq_lens=packed_len, n_splits=self.n_splits,
+            k_layout=_plan.K_BITPACKED, v_layout=_plan.V_BITPACKED, scale=self.scale,
+            k_row_width=self._k_row, v_row_width=self._vpb, workspace=self._ws,
+            extra_out=ext_out, extra_lse=ext_lse)
+        return out.unsqueeze(2)
+
     # ----------------------------------------------------------------- decode
     @torch.no_grad()
     def append_and_attend(self, layer_idx: int, q: torch.Tensor,
                           k_new: torch.Tensor, v_new: torch.Tensor) -> torch.Tensor:
         """q (B, n_q, 1, D), k_new / v_new (B, n_kv, S, D) -> (B, n_q, 1, D) fp16."""
+        if self.buffered:
+            return self._append_and_attend_buffered(layer_idx, q, k_new, v_new)
         li = layer_idx
         S = k_new.shape[2]
         t_pos = self._seq_lens if self._seq_lens is not None else self.seq_len

@@ -35,6 +35,8 @@ class Workload:
     student_t_nu: Optional[int] = None
     seed: int = 1234
     head_dim: int = 128
+    n_sink: int = 0                   # with-buffer setting: fp16 sink tokens ...
+    window: int = 0                   # ... and fp16 recent window next to the packed cache
     extra: dict = field(default_factory=dict)
 
 
@@ -49,6 +51,18 @@ WORKLOADS = {
                                   k_bits=2.0, v_bits=2, min_bits=0, max_bits=4,
                                   student_t_nu=4, seed=1236),
 }
+
+
+def _ragged_lens(batch: int, lo: int, hi: int, seed: int) -> List[int]:
+    gen = torch.Generator().manual_seed(seed)
+    return [int(x) for x in torch.randint(lo, hi + 1, (batch,), generator=gen)]
+
+
+# Qwen3-8B geometry, ragged batch in the with-buffer setting: K3V3 packed cache plus 4 fp16
+# sink tokens and a 128-token fp16 recent window, one append per sequence per step
+WORKLOADS["qwen3_8b_b32_ragged_buffered"] = Workload(
+    "qwen3_8b_b32_ragged_buffered", 36, 32, 8, 32, 16384, 1e6, seed=1237,
+    seq_lens=_ragged_lens(32, 1024, 16384, 1237), n_sink=4, window=128)
 
 
 def calibrate_layer(w: Workload, layer: int, device):
@@ -74,7 +88,8 @@ def build_manager(w: Workload, device, max_T: Optional[int] = None, n_layers: Op
     L = n_layers or w.n_layers
     mgr = BlockGTQKVManager(L, w.n_q, w.n_kv, w.head_dim, max_T or (w.context + 16),
                             batch_size=w.batch, k_avg_bits=w.k_bits, v_bits=w.v_bits,
-                            device=device, min_bits=w.min_bits, max_bits=w.max_bits)
+                            device=device, min_bits=w.min_bits, max_bits=w.max_bits,
+                            n_sink=w.n_sink, recent_window=w.window)
     energies = []
     for li in range(L):
         qs, e = calibrate_layer(w, li, device)
@@ -115,6 +130,14 @@ def draw_q(w: Workload, layer: int, device, position: int):
 
 def fill_cache(mgr: BlockGTQKVManager, w: Workload, energies, device, chunk: int = 8192):
     """Encode ``w.context`` synthetic tokens per row into every layer of ``mgr``."""
+    if mgr.buffered:
+        lens = w.seq_lens or [w.context] * w.batch
+        for li in range(mgr.n_layers):
+            k, v = draw_kv(w, energies[li], max(lens), li * 4096, device)
+            mgr.fill_buffered(li, k, v, lens)
+            del k, v
+        mgr.set_seq_lens(lens)
+        return
     for li in range(mgr.n_layers):
         for lo in range(0, w.context, chunk):
             n = min(chunk, w.context - lo)
@@ -133,7 +156,9 @@ def algorithmic_bytes_per_layer(mgr: BlockGTQKVManager, layer: int, seq_lens) ->
     total = 0
     vb = mgr._vpb
     for T_b in seq_lens:
+        fp16_rows = min(T_b, mgr.n_sink + mgr.window) if mgr.buffered else 0
         for q8 in mgr.quantizers[layer]:
-            total += T_b * (q8._total_packed_bytes + 2 * q8._n_groups + vb + 2)
+            total += (T_b - fp16_rows) * (q8._total_packed_bytes + 2 * q8._n_groups + vb + 2)
+            total += fp16_rows * mgr.hd * 2 * 2            # fp16 K and V rows of the buffer
     total += len(seq_lens) * mgr.n_q * mgr.hd * 2 * 2
     return total

@@ -269,3 +269,59 @@ def test_window_partial_merges_like_one_softmax(oracle_lib):
             want = wgt[0] * torch.tensor(ref_p[b, hq]).double() + wgt[1] * w_out
             assert (out[b, hq].double().cpu() - want).abs().max() < TOL
             assert abs(float(lse[b, hq]) - float(torch.logsumexp(a, 0))) < LSE_TOL
+
+
+def test_with_buffer_manager_keeps_sink_and_window_in_fp16(oracle_lib):
+    """Ragged batch with 4 fp16 sink tokens and a 16-token fp16 recent window: after a few
+    appends the output equals one softmax over [sink | dequantised middle | recent], where the
+    middle tokens went through the packers exactly once, when they left the window."""
+    from blockgtq_amd.packed_kv_manager import BlockGTQKVManager
+    ns, win, B, H, gqa, L = 4, 16, 3, 2, 4, 1
+    lens0 = [40, 21, 33]                         # row 1 starts with one packed token, others more
+    steps = 5
+    qs, ens = zip(*[make_quantizer(seed=90 + h, head=h, device=DEV, max_bits=5) for h in range(H)])
+    mgr = BlockGTQKVManager(L, H * gqa, H, 128, 128, batch_size=B, device=DEV, n_sink=ns, recent_window=win)
+    mgr.set_quantizers(0, list(qs))
+    Tmax = max(lens0) + steps
+    hist_k = np.zeros((B, H, Tmax, 128), np.float16)
+    hist_v = np.zeros((B, H, Tmax, 128), np.float16)
+    for b in range(B):
+        for h in range(H):
+            k, v, _ = make_kv(ens[h], Tmax, seed=500 + 10 * b + h)
+            hist_k[b, h], hist_v[b, h] = k, v
+    k0 = torch.tensor(hist_k[:, :, :max(lens0)]).to(DEV)
+    v0 = torch.tensor(hist_v[:, :, :max(lens0)]).to(DEV)
+    # rows shorter than the padded prefix: their tail positions come from their own history
+    # later, so hand every row its own first lens0[b] tokens and let the padding be ignored
+    mgr.fill_buffered(0, k0, v0, lens0)
+    mgr.set_seq_lens(lens0)
+    lens = list(lens0)
+    plans_np = mgr._batched_args[0]['plans_np']
+    gen = torch.Generator().manual_seed(77)
+    for step in range(steps):
+        q = torch.randn(B, H * gqa, 1, 128, generator=gen).half().to(DEV)
+        k1 = torch.tensor(np.stack([hist_k[b, :, lens[b]] for b in range(B)])[:, :, None]).to(DEV)
+        v1 = torch.tensor(np.stack([hist_v[b, :, lens[b]] for b in range(B)])[:, :, None]).to(DEV)
+        out = mgr.append_and_attend(0, q, k1, v1)[:, :, 0].float().cpu().numpy()
+        mgr.increment_seq_len()
+        lens = [t + 1 for t in lens]
+        qn = q[:, :, 0].cpu().numpy()
+        for b in range(B):
+            T = lens[b]
+            for h in range(H):
+                pl = plans_np[h:h + 1]
+                mid = slice(ns, T - win)
+                codes, raw, _ = oracle_lib.encode_k(pl, hist_k[b, h, mid])
+                kd = oracle_lib.dequant_k(pl, codes, oracle_lib.f2h(raw[:, :max(int(pl['n_seg'][0]), 1)]))
+                vc, vn = oracle_lib.encode_v(pl, hist_v[b, h, mid])
+                vd = oracle_lib.dequant_v(pl, vc, vn).astype(np.float64) @ pl['v_rot'][0].reshape(128, 128).astype(np.float64)
+                fp = np.r_[0:ns, T - win:T]
+                qh = qn[b, h * gqa:(h + 1) * gqa]
+                q_rot = oracle_lib.rotate_q(pl, qh).astype(np.float64)
+                logits = np.concatenate([q_rot @ kd.astype(np.float64).T,
+                                         qh.astype(np.float64) @ hist_k[b, h, fp].astype(np.float64).T], 1) / np.sqrt(128)
+                p = np.exp(logits - logits.max(1, keepdims=True))
+                p /= p.sum(1, keepdims=True)
+                ref = p @ np.concatenate([vd, hist_v[b, h, fp].astype(np.float64)], 0)
+                got = out[b, h * gqa:(h + 1) * gqa]
+                assert np.abs(got - ref).max() < TOL, (step, b, h, np.abs(got - ref).max())
