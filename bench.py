@@ -25,6 +25,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per attention launch from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy
+# kernel of known size (profiles/decode_mfma_kernel_<workload>_hbm_traffic.txt); valid for the
+# workload's own context, batch and default partition count only.
+MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 65.13e6}
 
 
 def parse():
@@ -39,6 +43,9 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run a device-to-device copy of this many MiB (a kernel of known HBM "
+                         "traffic, to calibrate FETCH_SIZE / WRITE_SIZE counter readings)")
     return ap.parse_args()
 
 
@@ -129,6 +136,14 @@ def main():
         for li in range(L):
             outs[li] = mgr.append_and_attend(li, qs[li], kvs[li][0], kvs[li][1])
 
+    if args.copy_probe_mib:
+        src = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # --- warm up eagerly, then capture the step once -----------------------
     step()
     torch.cuda.synchronize()
@@ -218,7 +233,9 @@ def main():
         "setup_s": round(setup_s, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "decode attention",
+                     "traffic": (MEASURED_TRAFFIC_BYTES.get(w.name)
+                                 if not (args.context or args.splits) else None),
+                     "kernel": "decode attention",
                      "algorithmic_bytes_per_launch": int(alg_bytes),
                      "avg_launch_us": round(attn_us, 3)},
     }
