@@ -265,6 +265,9 @@ int launch_generic(const DecodeArgs& a, hipStream_t st) {
 // One work-group per (batch row, query head).  Thread j first takes part in
 // finding the global maximum and the weight of every partition (partitions are
 // spread over the threads, weights parked in LDS), then owns output dim j.
+// Every global load that does not depend on a computed value (the first batch of
+// partial vectors, this thread's column of the un-rotation) is issued up front,
+// so the kernel pays for about one memory round trip.
 __global__ __launch_bounds__(D) void lse_reduce_kernel(
     const bgtq_head_plan* plans, const float* part_out, const float* part_lse, int n_splits,
     const float* extra_out, const float* extra_lse, int n_extra,
@@ -278,11 +281,17 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     const float* pl = part_lse + row * n_splits;
     const float* el = extra_lse ? extra_lse + row * n_extra : nullptr;
     const float* R = plans[hq / gqa].v_rot;
-    // the first rows of the un-rotation do not depend on anything computed here
-    constexpr int PF = 16;
-    float rpre[PF];
+    const float* po = part_out + row * n_splits * D + j;
+
+    constexpr int NB = 16;                     // partial vectors fetched before anything else
+    float pv[NB];
 #pragma unroll
-    for (int k = 0; k < PF; k++) rpre[k] = unrotate ? R[k * D + j] : 0.f;
+    for (int i = 0; i < NB; i++) pv[i] = po[(size_t)min(i, n_splits - 1) * D];
+    float rcol[D];                             // this thread's column of the un-rotation
+    if (unrotate) {
+#pragma unroll
+        for (int k = 0; k < D; k++) rcol[k] = R[k * D + j];
+    }
 
     float m = -INFINITY;
     for (int c = j; c < n_splits; c += D) { float l = pl[c]; wgt[c] = l; m = fmaxf(m, l); }
@@ -300,8 +309,15 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     for (int c = j; c < n_splits; c += D) { float l = wgt[c]; wgt[c] = (l == -INFINITY) ? 0.f : __expf(l - m); }
     __syncthreads();
     float den = 0.f, accp = 0.f, acce = 0.f;
-    const float* po = part_out + row * n_splits * D + j;
-    int c = 0;
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        if (i < n_splits) {
+            const float w = wgt[i];
+            den += w;
+            if (w != 0.f) accp += w * pv[i];
+        }
+    }
+    int c = NB;
     for (; c + 8 <= n_splits; c += 8) {
         float v[8];
 #pragma unroll
@@ -331,14 +347,7 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
         __syncthreads();
         float r = 0.f;
 #pragma unroll
-        for (int k = 0; k < PF; k++) r += vec[k] * rpre[k];
-        for (int k0 = PF; k0 < D; k0 += 16) {
-            float rr[16];
-#pragma unroll
-            for (int i = 0; i < 16; i++) rr[i] = R[(k0 + i) * D + j];
-#pragma unroll
-            for (int i = 0; i < 16; i++) r += vec[k0 + i] * rr[i];
-        }
+        for (int k = 0; k < D; k++) r += vec[k] * rcol[k];
         res = r;
     }
     out[b * o_sb + hq * o_sh + j] = bgtq_f2h((res + acce) / den);

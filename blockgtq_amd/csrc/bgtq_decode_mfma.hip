@@ -58,13 +58,16 @@ constexpr int LDS_LIMIT = 160 * 1024;
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
-// The first BGTQ_LUT_V + vlut_bytes bytes are a copy of the plan's lut_image.
-constexpr int VLUT = BGTQ_LUT_V;
+// LDS starts with the V pair table (8 KB reserved, so that an entry address is the table
+// offset OR-ed with field and bank bits), then a copy of the plan's K tables (kimg bytes:
+// lut_image up to BGTQ_LUT_V, or lut_image_mixed up to BGTQ_LUTM_V for the mixed K layout).
 constexpr int QROW = 400;                      // one head: zero unit + up to 24 units x 16 B
+constexpr int VTAB_BYTES = 8192;
+__host__ __device__ constexpr int kimg_bytes(int k_layout) { return k_layout == BGTQ_K_MIXED ? BGTQ_LUTM_V : BGTQ_LUT_V; }
 __host__ __device__ constexpr int vlut_bytes(int vbw) { return vbw == 4 ? 256 * 32 : (1 << (2 * vbw)) * 128; }
-__host__ __device__ constexpr int steptab_off(int vbw) { return VLUT + vlut_bytes(vbw); }   // [step][lane group] x 32 B
-__host__ __device__ constexpr int qpad_off(int vbw) { return steptab_off(vbw) + MAX_STEPS * 4 * 32; }
-__host__ __device__ constexpr int waves_off(int vbw) { return qpad_off(vbw) + 16 * QROW; }
+__host__ __device__ constexpr int steptab_off(int kimg) { return VTAB_BYTES + kimg; }   // [step][lane group] x 32 B
+__host__ __device__ constexpr int qpad_off(int kimg) { return steptab_off(kimg) + MAX_STEPS * 4 * 32; }
+__host__ __device__ constexpr int waves_off(int kimg) { return qpad_off(kimg) + 16 * QROW; }
 constexpr int WAVE_NORM_BYTES = BGTQ_MAX_SEGMENTS * MT * 2 + MT * 4;   // fp16 K norms [seg][token], fp32 V norms
 constexpr int INIT_SCRATCH = MAX_STEPS * 4 * 32 + 256 + 16 * D * 2;
 
@@ -209,10 +212,12 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     constexpr int vrow = 16 * VBW;
     const int kn_st = (int)a.kn_st;
     const TileLayout tl = tile_layout(krow, vrow, kn_st);
-    uint4* steptab = (uint4*)(smem + steptab_off(VBW));
-    uint8_t* qpad = smem + qpad_off(VBW);
+    const bool kmix = a.k_layout == BGTQ_K_MIXED, vnib = a.v_layout == BGTQ_V_NIBBLE;
+    const int kimg = kimg_bytes(a.k_layout);             // LDS offset of the V table
+    uint4* steptab = (uint4*)(smem + steptab_off(kimg));
+    uint8_t* qpad = smem + qpad_off(kimg);
     const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
-    const uint32_t kbufs_off = waves_off(VBW);                                   // [KB][nw] K + norm buffers
+    const uint32_t kbufs_off = waves_off(kimg);                                   // [KB][nw] K + norm buffers
     const uint32_t vbuf_off = kbufs_off + KB * nw * tl.kbuf + wave * tl.vt;        // [nw] V buffers
     const uint32_t norm_off = kbufs_off + nw * (KB * tl.kbuf + tl.vt) + wave * WAVE_NORM_BYTES;
     uint8_t* kn_h = smem + norm_off;                                 // fp16 [segment][token]
@@ -251,11 +256,21 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     // The pair tables come ready-made from the plan and are copied into LDS by DMA, each
     // wave taking every nw-th KB; the first K tile follows right behind them.
     {
-        const uint8_t* img = (const uint8_t*)P.lut_image;
-        constexpr int total = BGTQ_LUT_V + vlut_bytes(VBW);
-        for (int cc = wave; cc * 1024 < total; cc += nw)
-            dma16(voff, uniform_ptr(img + cc * 1024), __builtin_amdgcn_readfirstlane(smem_lds + cc * 1024),
-                  __builtin_amdgcn_ballot_w64((int)voff + cc * 1024 < total));
+        // V table of the value layout in use at LDS offset 0, K tables of the record layout
+        // in use behind it; the chunks of both are dealt round-robin to the waves
+        const uint8_t* vimg = vnib ? (const uint8_t*)P.lut_image_mixed + BGTQ_LUTM_V
+                                   : (const uint8_t*)P.lut_image + BGTQ_LUT_V;
+        const uint8_t* kimg_src = (const uint8_t*)(kmix ? P.lut_image_mixed : P.lut_image);
+        constexpr int vch = (vlut_bytes(VBW) + 1023) >> 10;
+        const int kch = (kimg + 1023) >> 10;
+        for (int cc = wave; cc < vch + kch; cc += nw) {
+            const bool isv = cc < vch;
+            const int o = (isv ? cc : cc - vch) * 1024;
+            const int left = (isv ? vlut_bytes(VBW) : kimg) - o;
+            dma16(voff, uniform_ptr((isv ? vimg : kimg_src) + o),
+                  __builtin_amdgcn_readfirstlane(smem_lds + (isv ? 0 : VTAB_BYTES) + o),
+                  __builtin_amdgcn_ballot_w64((int)voff < left));
+        }
     }
     int k0_loads = 0;
     if (tile < t1) k0_loads = issue_k(tile, 0);
@@ -263,22 +278,24 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     uint32_t* st_raw = (uint32_t*)scratch;                // steptab as stored in the plan
     int* qu_s = (int*)(scratch + MAX_STEPS * 4 * 32);     // qunit_dim[32], qunit_len[32]
     uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 4 * 32 + 256);   // [16][128] rotated queries
-    for (int i = tid; i < MAX_STEPS * 4 * 8; i += nthr) st_raw[i] = (&P.steptab[0][0][0])[i];
-    for (int i = tid; i < 64; i += nthr) qu_s[i] = P.qunit_dim[i];     // qunit_len follows qunit_dim
+    const uint32_t* st_src = kmix ? &P.steptab_mixed[0][0][0] : &P.steptab[0][0][0];
+    const int32_t* qu_src = kmix ? P.qunit_dim_mixed : P.qunit_dim;     // qunit_len follows qunit_dim
+    for (int i = tid; i < MAX_STEPS * 4 * 8; i += nthr) st_raw[i] = st_src[i];
+    for (int i = tid; i < 64; i += nthr) qu_s[i] = qu_src[i];
     for (int i = tid; i < 16 * D / 2; i += nthr) {
         int hq = i / (D / 2), d2 = i - hq * (D / 2);
         uint32_t v = 0;
         if (hq < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + hq) * a.q_sh + d2 * 2);
         ((uint32_t*)q_s)[i] = v;
     }
-    const int n_steps = min(P.n_steps, MAX_STEPS);
-    const int n_packed = min(P.n_packed_steps, n_steps);   // raw-byte steps (bw >= 5) come last
+    const int n_steps = min(kmix ? P.n_steps_mixed : P.n_steps, MAX_STEPS);
+    const int n_packed = min(kmix ? P.n_packed_steps_mixed : P.n_packed_steps, n_steps);   // raw-byte steps come last
     __syncthreads();
     TRACE(2);
     for (int i = tid; i < n_steps * 4; i += nthr) {        // the row offset depends on the cache's alignment
         const uint32_t* r = st_raw + i * 8;
         const uint32_t o = kph + r[0];
-        steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2] + smem_lds, r[3]};     // table as an absolute LDS address
+        steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2] + smem_lds + VTAB_BYTES, r[3]};     // table as an absolute LDS address
         steptab[i * 2 + 1] = (uint4){r[4], r[5], r[6] * MT / 64, r[7]};   // norm rows are MT tokens long here
     }
     for (int i = tid; i < 16 * (QROW / 4); i += nthr) {     // query units, zero padded
@@ -298,14 +315,16 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 
     const float c2 = a.scale * 1.44269504088896340736f;      // logits go through exp2
     const uint32_t lane4 = (uint32_t)lane * 4;
-    const uint32_t vbank = smem_lds + (VBW == 4 ? (lane4 & 28u) : (lane4 & 124u));   // V table replica of this lane (LDS is 128-byte aligned)
+    // V table replica of this lane.  The table sits at the very start of LDS (this kernel has
+    // no static LDS, the launcher checks that), so field bits OR-ed in never meet the base.
+    const uint32_t vbank = smem_lds + (VBW == 4 ? (lane4 & 28u) : (lane4 & 124u));
     constexpr int vshift = VBW == 4 ? 5 : 7;
     const uint32_t rowoff = (uint32_t)li * krow;
     const uint32_t kstride = 16u * krow;
     const uint32_t vc = vph + (uint32_t)li * VBW;
     const uint32_t vbase = smem_lds + vbuf_off + (vc & ~3u) + (uint32_t)lg * 4 * vrow, v_sh = vc & 3u;
-    const uint32_t stl = smem_lds + steptab_off(VBW) + lg * 32;          // absolute LDS addresses from here on
-    const uint32_t qrow = smem_lds + qpad_off(VBW) + li * QROW;
+    const uint32_t stl = smem_lds + steptab_off(kimg) + lg * 32;         // absolute LDS addresses from here on
+    const uint32_t qrow = smem_lds + qpad_off(kimg) + li * QROW;
     const uint32_t nrm = smem_lds + norm_off + lg * 8;
     const uint32_t vnf = smem_lds + norm_off + BGTQ_MAX_SEGMENTS * MT * 2;
 
@@ -481,7 +500,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                     constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
                     const int fp = e * 2 * VBW;
                     const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
-                    W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank) + VLUT);   // + VLUT rides in the offset field
+                    W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -569,10 +588,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 }
 
 // LDS bytes of a work-group of nw waves
-size_t mfma_smem_bytes(int vbw, int krow, int vrow, int kn_st, int nw) {
+size_t mfma_smem_bytes(int k_layout, int krow, int vrow, int kn_st, int nw) {
+    const int woff = waves_off(kimg_bytes(k_layout));
     const TileLayout tl = tile_layout(krow, vrow, kn_st);
-    size_t need = (size_t)waves_off(vbw) + (size_t)nw * (KB * tl.kbuf + tl.vt + WAVE_NORM_BYTES);
-    size_t scratch = (size_t)waves_off(vbw) + (size_t)nw * tl.kbuf + INIT_SCRATCH;
+    size_t need = (size_t)woff + (size_t)nw * (KB * tl.kbuf + tl.vt + WAVE_NORM_BYTES);
+    size_t scratch = (size_t)woff + (size_t)nw * tl.kbuf + INIT_SCRATCH;
     size_t merge = (size_t)nw * (32 + 16 * D) * 4;
     size_t s = need > scratch ? need : scratch;
     return s > merge ? s : merge;
@@ -584,16 +604,22 @@ int launch(const DecodeArgs& a, hipStream_t st) {
     const int part = (a.T + a.n_splits - 1) / a.n_splits;
     int nw = (part + MT - 1) / MT;
     nw = nw < 1 ? 1 : nw > MAX_WAVES ? MAX_WAVES : nw;
-    while (nw > 1 && mfma_smem_bytes(VBW, a.k_row_width, a.v_row_width, (int)a.kn_st, nw) > (size_t)LDS_LIMIT) nw--;
-    const size_t smem = mfma_smem_bytes(VBW, a.k_row_width, a.v_row_width, (int)a.kn_st, nw);
+    while (nw > 1 && mfma_smem_bytes(a.k_layout, a.k_row_width, a.v_row_width, (int)a.kn_st, nw) > (size_t)LDS_LIMIT) nw--;
+    const size_t smem = mfma_smem_bytes(a.k_layout, a.k_row_width, a.v_row_width, (int)a.kn_st, nw);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
     auto kern = decode_mfma_kernel<VBW>;
-    static size_t attr_set = 0;              // largest size the attribute was raised to
-    if (smem > attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_LIMIT);
+    static int ready = 0;                    // 1: usable, -1: not usable
+    if (ready == 0) {
+        // the kernel addresses its V table as "LDS offset 0": that holds only while it has
+        // no static LDS in front of the dynamic block
+        hipFuncAttributes fa;
+        hipError_t e = hipFuncGetAttributes(&fa, (const void*)kern);
         if (e != hipSuccess) return (int)e;
-        attr_set = LDS_LIMIT;
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_LIMIT);
+        if (e != hipSuccess) return (int)e;
+        ready = fa.sharedSizeBytes == 0 ? 1 : -1;
     }
+    if (ready < 0) return BGTQ_EUNSUPPORTED;
     dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)a.B);
     hipLaunchKernelGGL(kern, grid, dim3(nw * 64), smem, st, a);
     return bgtq_launch_status();
@@ -609,7 +635,6 @@ extern "C" int bgtq_debug_set_trace(void* buf) {
 
 int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     // layout requirements of the fast path; anything else takes the generic kernel
-    if (a.k_layout != BGTQ_K_BITPACKED || a.v_layout != BGTQ_V_BITPACKED) return BGTQ_EUNSUPPORTED;
     if (a.gqa > 16 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
     if ((a.kp_st & 3) || (a.kp_sb & 3) || (a.kp_sh & 3) || ((uintptr_t)a.kp & 3)) return BGTQ_EUNSUPPORTED;
     if ((a.vp_st & 3) || (a.vp_sb & 3) || (a.vp_sh & 3) || ((uintptr_t)a.vp & 3)) return BGTQ_EUNSUPPORTED;
@@ -617,7 +642,8 @@ int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     if (a.k_row_width < 4 || a.k_row_width > 128) return BGTQ_EUNSUPPORTED;
     if (a.vn_st != 1 || a.kn_st < 1 || a.kn_st > MAX_KN) return BGTQ_EUNSUPPORTED;
     if ((a.q_sb & 1) || (a.q_sh & 1) || ((uintptr_t)a.q & 3)) return BGTQ_EUNSUPPORTED;
-    // a bit-packed V record of 128 dims is 16 bytes per bit of code width
+    if (a.v_layout == BGTQ_V_NIBBLE && a.v_row_width != 64) return BGTQ_EUNSUPPORTED;
+    // a bit-packed V record of 128 dims is 16 bytes per bit of code width, a nibble record 64
     switch (a.v_row_width) {
     case 16: return launch<1>(a, stream);
     case 32: return launch<2>(a, stream);

@@ -13,6 +13,8 @@
 // byte j while packing.  The rotation matrix is read once per work-group
 // (coalesced across j, served from L2) and reused for all ROWS rows out of
 // registers; rows are staged in LDS so the k-loop reads them as broadcasts.
+#include <type_traits>
+
 #include "bgtq_common.h"
 
 namespace {
@@ -53,40 +55,96 @@ __device__ inline unsigned stream_byte(const uint8_t* codes, int len, int bw, in
     return out;
 }
 
+// Plan tables a work-group needs, copied to LDS with one burst of independent loads:
+// every later table access is an LDS read instead of one more dependent trip to memory.
+struct StagedK {
+    int hdr[56];                 // n_seg .. seg_identity, as at the start of bgtq_head_plan
+    int group_of[D];
+    int head_perm[D];
+    float lut_offset[D];
+    float lut_inv_scale[D];
+    uint8_t code_lut[BGTQ_MAX_SEGMENTS * BGTQ_LUT_BINS];
+    float centroids[BGTQ_MAX_SEGMENTS * 32];   // first 32 levels of every segment (bw <= 5)
+};
+struct StagedV {
+    int v_bits;
+    float centroids[16];
+    float boundaries[16];
+};
+constexpr int H_NSEG = 0, H_NZERO = 1, H_NOPACK_START = 4, H_NOPACK_LEN = 5, H_VBITS = 6;
+constexpr int H_BW = 8, H_START = 16, H_LEN = 24, H_PACK_OFF = 32, H_IDENT = 48;
+
 template <int ROWS, bool IS_V>
 __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, const int h) {
     __shared__ float xs[ROWS][D];
     __shared__ float nrm[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ float nrm_out[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ uint8_t cds[ROWS][D];
+    __shared__ uint16_t xraw[ROWS][D];
+    __shared__ typename std::conditional<IS_V, StagedV, StagedK>::type sp;
 
     const int j = threadIdx.x;
     const bgtq_head_plan& P = a.plans[h];
     const int64_t N = (int64_t)a.B * a.S;
     const int64_t row0 = (int64_t)bx * ROWS;
-
-    // ---- per-thread static data -------------------------------------------
-    const int n_seg = IS_V ? 1 : P.n_seg;
-    const int g = IS_V ? 0 : P.group_of[j];
-    int gs = 0, ge = D, ident = 0;
-    if (!IS_V) {
-        if (g >= 0) { gs = P.seg_start[g]; ge = gs + P.seg_len[g]; ident = P.seg_identity[g]; }
-        else        { gs = 0; ge = 0; }
-    }
     const float* RT = IS_V ? P.v_rot_T : P.k_rot_T;
-    const int src_dim = IS_V ? j : P.head_perm[j];
 
-    // ---- 1. load (gather by head_perm for K), fp16 -> fp32 -----------------
+    // ---- 0. one burst: plan tables, the raw rows, and (V) the rotation column -------------
+    if constexpr (IS_V) {
+        if (j == 0) sp.v_bits = P.v_bits;
+        if (j < 16) { sp.centroids[j] = P.v_centroids[j]; sp.boundaries[j] = P.v_boundaries[j]; }
+    } else {
+        if (j < 56) sp.hdr[j] = ((const int*)&P)[j];
+        sp.group_of[j] = P.group_of[j];
+        sp.head_perm[j] = P.head_perm[j];
+        sp.lut_offset[j] = P.lut_offset[j];
+        sp.lut_inv_scale[j] = P.lut_inv_scale[j];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            ((uint32_t*)sp.code_lut)[j + i * NT] = ((const uint32_t*)&P.code_lut[0][0])[j + i * NT];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int e = j + i * NT;                        // segment e / 32, level e % 32
+            sp.centroids[e] = P.k_centroids[e >> 5][e & 31];
+        }
+    }
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
         int64_t n = row0 + r;
-        float v = 0.f;
+        uint16_t v = 0;
         if (n < N) {
             int64_t b = n / a.S, s = n - b * a.S;
-            v = bgtq_h2f(a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + src_dim]);
+            v = a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + j];
         }
-        xs[r][j] = v;
+        xraw[r][j] = v;
     }
+    // Decode append is latency bound: V's rotation column does not depend on anything, so
+    // the whole of it is requested now; K's depends on the group range and follows below.
+    constexpr int PF = ROWS == 2 ? (IS_V ? D : 32) : 0;
+    float rpre[PF > 0 ? PF : 1];
+    if constexpr (IS_V && PF > 0) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) rpre[i] = RT[i * D + j];
+    }
+    __syncthreads();
+
+    // ---- per-thread static data -------------------------------------------
+    int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
+    if constexpr (!IS_V) {
+        n_seg = sp.hdr[H_NSEG];
+        g = sp.group_of[j];
+        src_dim = sp.head_perm[j];
+        if (g >= 0) { gs = sp.hdr[H_START + g]; ge = gs + sp.hdr[H_LEN + g]; ident = sp.hdr[H_IDENT + g]; }
+        else        { gs = 0; ge = 0; }
+        if (PF > 0 && !(ident || g < 0)) {
+#pragma unroll
+            for (int i = 0; i < PF; i++) rpre[i] = RT[min(gs + i, ge - 1) * D + j];
+        }
+    }
+
+    // ---- 1. gather by head_perm (K), fp16 -> fp32 ------------------------------
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xraw[r][src_dim]);
     __syncthreads();
 
     // ---- 2. group norms: thread (r, grp) runs one sequential chain ---------
@@ -94,8 +152,8 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
         float n = 0.f;
         if (gg < n_seg) {
-            int s = IS_V ? 0 : P.seg_start[gg];
-            int e = IS_V ? D : s + P.seg_len[gg];
+            int s = 0, e = D;
+            if constexpr (!IS_V) { s = sp.hdr[H_START + gg]; e = s + sp.hdr[H_LEN + gg]; }
             float ss = 0.f;
 #pragma unroll 8
             for (int k = s; k < e; k++) ss = __builtin_fmaf(xs[r][k], xs[r][k], ss);
@@ -130,8 +188,15 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     } else {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) y[r] = 0.f;
-        constexpr int RB = 16;
-        for (int k0 = gs; k0 < ge; k0 += RB) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {          // entries fetched at the top of the kernel
+            if (gs + i < ge) {
+#pragma unroll
+                for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][gs + i], rpre[i], y[r]);
+            }
+        }
+        constexpr int RB = IS_V ? 32 : 16;
+        for (int k0 = gs + PF; k0 < ge; k0 += RB) {
             float rt[RB];
 #pragma unroll
             for (int i = 0; i < RB; i++) rt[i] = RT[min(k0 + i, ge - 1) * D + j];
@@ -151,22 +216,29 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     for (int r = 0; r < ROWS; r++) {
         int code = 0;
         if (IS_V) {
-            int nb = (1 << P.v_bits) - 1;
-            for (int b = 0; b < nb; b++) code += (y[r] > P.v_boundaries[b]) ? 1 : 0;
+            if constexpr (IS_V) {
+                int nb = (1 << sp.v_bits) - 1;
+                for (int b = 0; b < nb; b++) code += (y[r] > sp.boundaries[b]) ? 1 : 0;
+            }
         } else if (g >= 0) {
-            if (a.quant_mode == BGTQ_QUANT_EXACT) {
-                int nb = (1 << P.seg_bw[g]) - 1;
-                for (int b = 0; b < nb; b++) code += (P.k_boundaries[g][b] < y[r]) ? 1 : 0;
-            } else {
-                float t = (y[r] - P.lut_offset[j]) * P.lut_inv_scale[j];
-                t = fminf(fmaxf(t, 0.0f), (float)(BGTQ_LUT_BINS - 1));
-                code = P.code_lut[g][(int)t];
+            if constexpr (!IS_V) {
+                if (a.quant_mode == BGTQ_QUANT_EXACT) {
+                    int nb = (1 << sp.hdr[H_BW + g]) - 1;
+                    for (int b = 0; b < nb; b++) code += (P.k_boundaries[g][b] < y[r]) ? 1 : 0;
+                } else {
+                    float t = (y[r] - sp.lut_offset[j]) * sp.lut_inv_scale[j];
+                    t = fminf(fmaxf(t, 0.0f), (float)(BGTQ_LUT_BINS - 1));
+                    code = sp.code_lut[g * BGTQ_LUT_BINS + (int)t];
+                }
             }
         }
         cds[r][j] = (uint8_t)code;
         // centroid of the chosen code for the norm correction below; it is parked in xs
         // after the barrier (other threads may still be reading xs in their rotation)
-        if (need_cent) y[r] = IS_V ? P.v_centroids[code] : (g >= 0 ? P.k_centroids[g][code] : 0.f);
+        if (need_cent) {
+            if constexpr (IS_V) y[r] = sp.centroids[code];
+            else y[r] = g < 0 ? 0.f : code < 32 ? sp.centroids[g * 32 + code] : P.k_centroids[g][code];
+        }
     }
     __syncthreads();
     if (need_cent) {
@@ -191,7 +263,8 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
                 float cn = __builtin_sqrtf(cs + 1e-20f);
                 out = n / (cn > 1e-10f ? cn : 1.0f);
             } else if (a.layout == BGTQ_K_MIXED || a.corrected) {
-                int s = P.seg_start[gg], e = s + P.seg_len[gg];
+                int s = 0, e = 0;
+                if constexpr (!IS_V) { s = sp.hdr[H_START + gg]; e = s + sp.hdr[H_LEN + gg]; }
                 float cs = 0.f;
                 for (int k = s; k < e; k++) {
                     float c = xs[r][k];
@@ -240,20 +313,20 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     if (j >= a.row_width) return;
     int mode = 0;        // 0: zero fill, 1: bit stream, 2: raw byte copy
     int c0 = 0, clen = 0, bw = 1, idx = 0;
-    if (IS_V) {
-        bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : P.v_bits;
+    if constexpr (IS_V) {
+        bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : sp.v_bits;
         if (j < bgtq_seg_bytes(bw, D)) { mode = 1; c0 = 0; clen = D; idx = j; }
     } else if (a.layout == BGTQ_K_MIXED) {
-        int z = P.n_zero_dims;
-        int nib = (P.nopack_start - z) >> 1;
-        if (j < nib)                     { mode = 1; bw = 4; c0 = z; clen = P.nopack_start - z; idx = j; }
-        else if (j < nib + P.nopack_len) { mode = 2; c0 = P.nopack_start + (j - nib); }
+        int z = sp.hdr[H_NZERO], nps = sp.hdr[H_NOPACK_START];
+        int nib = (nps - z) >> 1;
+        if (j < nib)                             { mode = 1; bw = 4; c0 = z; clen = nps - z; idx = j; }
+        else if (j < nib + sp.hdr[H_NOPACK_LEN]) { mode = 2; c0 = nps + (j - nib); }
     } else {
-        for (int s = 0; s < P.n_seg; s++) {
-            int off = P.seg_pack_off[s], sb = P.seg_bw[s], sl = P.seg_len[s];
+        for (int s = 0; s < n_seg; s++) {
+            int off = sp.hdr[H_PACK_OFF + s], sb = sp.hdr[H_BW + s], sl = sp.hdr[H_LEN + s];
             if (j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
-                if (sb >= 5) { mode = 2; c0 = P.seg_start[s] + (j - off); }
-                else         { mode = 1; bw = sb; c0 = P.seg_start[s]; clen = sl; idx = j - off; }
+                if (sb >= 5) { mode = 2; c0 = sp.hdr[H_START + s] + (j - off); }
+                else         { mode = 1; bw = sb; c0 = sp.hdr[H_START + s]; clen = sl; idx = j - off; }
             }
         }
     }

@@ -40,11 +40,15 @@ PLAN_DTYPE = np.dtype([
     ('n_packed_steps', '<i4'), ('reserved2', '<i4', (3,)),
     ('steptab', '<u4', (MAX_STEPS, 4, 8)), ('qunit_dim', '<i4', (32,)), ('qunit_len', '<i4', (32,)),
     ('lut_image', '<u4', (29184 // 4,)),
+    ('n_steps_mixed', '<i4'), ('n_packed_steps_mixed', '<i4'), ('reserved3', '<i4', (2,)),
+    ('steptab_mixed', '<u4', (MAX_STEPS, 4, 8)), ('qunit_dim_mixed', '<i4', (32,)),
+    ('qunit_len_mixed', '<i4', (32,)), ('lut_image_mixed', '<u4', (43008 // 4,)),
 ], align=True)
 
 # byte offsets inside lut_image (BGTQ_LUT_* of include/bgtq.h)
 LUT_K = {1: 0, 2: 512, 3: 2560, 4: 10752}
 LUT_KRAW, LUT_V, LUT_IMAGE_BYTES = 18944, 20992, 29184
+LUTM_KRAW, LUTM_V, LUTM_IMAGE_BYTES = 32768, 34816, 43008      # BGTQ_LUTM_*
 
 
 def segment_bytes(bw: int, length: int) -> int:
@@ -122,6 +126,63 @@ def fill_decode_steps(p) -> None:
         t = _pair_table(p['v_lut_f16'], vb)
         img[LUT_V // 4:LUT_V // 4 + t.size] = t
     p['lut_image'] = img
+    _fill_mixed_tables(p)
+
+
+def _byte_pair_table(cb16: np.ndarray, bw: int) -> np.ndarray:
+    """Pair table indexed by a byte that holds two codes as nibbles (low nibble first)."""
+    b = np.arange(256)
+    lo, hi = b & 15, b >> 4
+    ok = (lo < (1 << bw)) & (hi < (1 << bw))
+    pairs = cb16[np.where(ok, lo, 0)].astype(np.uint32) | (cb16[np.where(ok, hi, 0)].astype(np.uint32) << 16)
+    return np.repeat(np.where(ok, pairs, 0).astype(np.uint32), 8)
+
+
+def _fill_mixed_tables(p) -> None:
+    """Step schedule, query units and table image of the mixed K / nibble V layouts."""
+    m, n_packed, unit, n_ptab = 0, 0, 1, 0
+    p['steptab_mixed'][...] = 0
+    p['qunit_dim_mixed'][...] = 0
+    p['qunit_len_mixed'][...] = 0
+    img = np.zeros(LUTM_IMAGE_BYTES // 4, dtype=np.uint32)
+    for s in range(int(p['n_seg'])):
+        bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
+        start, end = int(p['seg_start'][s]), int(p['seg_start'][s]) + ln
+        n_units = (ln + 7) // 8
+        unit_bytes = 4 if bw <= 4 else 8
+        cb = p['k_codebook_f16'][s]
+        if bw <= 4:
+            table = n_ptab * 8192                 # at most 4 distinct widths <= 4 bits
+            img[table // 4:table // 4 + 2048] = _byte_pair_table(cb, bw)
+            n_ptab += 1
+        else:
+            table = LUTM_KRAW + (bw - 5) * 512
+            raw = np.zeros(256, dtype=np.uint16)
+            raw[:1 << bw] = cb[:1 << bw]
+            img[table // 4:table // 4 + 128] = raw.view(np.uint32)
+        for u0 in range(0, n_units, 4):
+            if m >= MAX_STEPS:
+                raise ValueError("segment table needs more MFMA steps than the plan holds")
+            nu = min(4, n_units - u0)
+            off0 = int(p['seg_mixed_off'][s]) + u0 * unit_bytes
+            for g in range(4):
+                gg = min(g, nu - 1)
+                q_off = 0
+                if g < nu:
+                    d0 = start + (u0 + g) * 8
+                    p['qunit_dim_mixed'][unit], p['qunit_len_mixed'][unit] = d0, min(8, end - d0)
+                    q_off = 16 * unit
+                    unit += 1
+                p['steptab_mixed'][m, g] = (off0 + gg * unit_bytes, 0, table, 7 * 4 if bw <= 4 else 0,
+                                            8 if bw <= 4 else 0, 5, s * 128, q_off)
+            n_packed += bw <= 4
+            m += 1
+    p['n_steps_mixed'] = m
+    p['n_packed_steps_mixed'] = n_packed
+    vb = int(p['v_bits'])
+    if 1 <= vb <= 4:
+        img[LUTM_V // 4:LUTM_V // 4 + 2048] = _byte_pair_table(p['v_lut_f16'], vb)
+    p['lut_image_mixed'] = img
 
 
 def build_head_plan(quantizer) -> np.ndarray:

@@ -37,6 +37,11 @@ extern "C" {
 #define BGTQ_LUT_KRAW    18944                   /* 4 tables x 256 fp16       */
 #define BGTQ_LUT_V       20992                   /* V pair table, up to 8192 B */
 #define BGTQ_LUT_IMAGE_BYTES 29184
+/* the same for lut_image_mixed */
+#define BGTQ_LUTM_K0     0                       /* up to 4 packed segments x 256 entries x 8 replicas */
+#define BGTQ_LUTM_KRAW   32768
+#define BGTQ_LUTM_V      34816
+#define BGTQ_LUTM_IMAGE_BYTES 43008
 
 /* error codes (negative); positive return values are hipError_t */
 #define BGTQ_OK            0
@@ -133,6 +138,23 @@ typedef struct bgtq_head_plan {
     int32_t  qunit_dim[32];
     int32_t  qunit_len[32];
     uint32_t lut_image[BGTQ_LUT_IMAGE_BYTES / 4];
+
+    /*
+     * The same three tables for the mixed K layout (nibbles of every code of at most
+     * 4 bits, then raw bytes) and the nibble V layout.  A pair of codes is one
+     * byte there, so each packed segment gets its own 256-entry table indexed by
+     * that byte (entry = centroids of the low and the high nibble, 0 where a
+     * nibble is not a code of the segment), 8 replicas: the i-th packed segment at
+     * BGTQ_LUTM_K0 + i * 8192, raw-byte tables at BGTQ_LUTM_KRAW + (bw - 5) * 512,
+     * the byte-indexed V table at BGTQ_LUTM_V.
+     */
+    int32_t  n_steps_mixed;
+    int32_t  n_packed_steps_mixed;
+    int32_t  reserved3[2];
+    uint32_t steptab_mixed[BGTQ_MAX_STEPS][4][8];
+    int32_t  qunit_dim_mixed[32];
+    int32_t  qunit_len_mixed[32];
+    uint32_t lut_image_mixed[BGTQ_LUTM_IMAGE_BYTES / 4];
 } bgtq_head_plan;
 
 /* sizeof(bgtq_head_plan) as the library was compiled; the host mirror checks it. */

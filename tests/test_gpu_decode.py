@@ -325,3 +325,25 @@ def test_with_buffer_manager_keeps_sink_and_window_in_fp16(oracle_lib):
                 ref = p @ np.concatenate([vd, hist_v[b, h, fp].astype(np.float64)], 0)
                 got = out[b, h * gqa:(h + 1) * gqa]
                 assert np.abs(got - ref).max() < TOL, (step, b, h, np.abs(got - ref).max())
+
+
+@pytest.mark.parametrize("k_layout,v_layout,vb", [(0, 0, 3), (1, 1, 3), (1, 0, 4), (0, 1, 2), (1, 1, 4)])
+def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, vb):
+    """With the layout-agnostic kernel switched off, the MFMA kernel must accept bit-packed
+    and mixed K records and bit-packed and nibble V records in any combination."""
+    from blockgtq_amd import _capi
+    lib = _capi.lib()
+    args, qs, q_rot, kp, kn, vp, vn = _build(192, 1, 6, vb, 2, 4, 2, 333, seed=7 + 3 * k_layout + v_layout,
+                                             k_layout=k_layout, v_layout=v_layout)
+    ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
+                              vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), [333] * 2, 4,
+                              k_layout, v_layout, vb)
+    assert lib.bgtq_set_decode_path(2) == 0
+    try:
+        for ns in (1, 4):
+            out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 333, n_splits=ns,
+                                            k_layout=k_layout, v_layout=v_layout, return_lse=True)
+            assert np.abs(out.float().cpu().numpy() - ref).max() < TOL
+            assert np.abs(lse.cpu().numpy() - ref_lse).max() < LSE_TOL
+    finally:
+        lib.bgtq_set_decode_path(0)
