@@ -42,17 +42,28 @@ struct EncodeArgs {
     int corrected;              // K codes path: emit corrected norms
 };
 
-// LSB-first stream of bw-bit codes -> byte `idx`; codes past `len` read as 0.
-__device__ inline unsigned stream_byte(const uint8_t* codes, int len, int bw, int idx) {
-    unsigned out = 0;
-#pragma unroll
-    for (int b = 0; b < 8; b++) {
-        int bit = idx * 8 + b;
-        int ci = bit / bw;
-        unsigned c = ci < len ? codes[ci] : 0u;
-        out |= ((c >> (bit - ci * bw)) & 1u) << b;
+// Byte `idx` of the LSB-first stream of bw-bit codes (bw <= 4) covers the codes
+// first .. first + n - 1, the first of them from its bit `skip` on.  None of this depends
+// on the row, so a thread works it out once and reuses it for every row of the tile.
+struct StreamSlot { int first, n, skip; };
+__device__ inline StreamSlot stream_slot(int len, int bw, int idx) {
+    const int bit0 = idx * 8;
+    int first, skip;
+    switch (bw) {                               // constant divisors: no integer division at run time
+    case 1: first = bit0; skip = 0; break;
+    case 2: first = bit0 >> 1; skip = 0; break;
+    case 3: first = bit0 / 3; skip = bit0 - first * 3; break;
+    default: first = bit0 >> 2; skip = 0; break;
     }
-    return out;
+    int last = (bit0 + 7) / (bw == 3 ? 3 : 1);
+    if (bw != 3) last = (bit0 + 7) >> (bw == 1 ? 0 : bw == 2 ? 1 : 2);
+    last = min(last, len - 1);
+    return {first, last - first + 1, skip};
+}
+__device__ inline unsigned stream_byte(const uint8_t* codes, StreamSlot s, int bw) {
+    unsigned w = 0;
+    for (int i = 0; i < s.n; i++) w |= (unsigned)codes[s.first + i] << (i * bw);
+    return (w >> s.skip) & 0xFFu;
 }
 
 // Plan tables a work-group needs, copied to LDS with one burst of independent loads:
@@ -75,8 +86,9 @@ constexpr int H_NSEG = 0, H_NZERO = 1, H_NOPACK_START = 4, H_NOPACK_LEN = 5, H_V
 constexpr int H_BW = 8, H_START = 16, H_LEN = 24, H_PACK_OFF = 32, H_IDENT = 48;
 
 template <int ROWS, bool IS_V>
-__device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, const int h) {
-    __shared__ float xs[ROWS][D];
+__device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, const int h,
+                                            const int64_t n_tiles, const int tile_stride) {
+    __shared__ __align__(16) float xs[ROWS][D];
     __shared__ float nrm[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ float nrm_out[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ uint8_t cds[ROWS][D];
@@ -86,10 +98,10 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     const int j = threadIdx.x;
     const bgtq_head_plan& P = a.plans[h];
     const int64_t N = (int64_t)a.B * a.S;
-    const int64_t row0 = (int64_t)bx * ROWS;
     const float* RT = IS_V ? P.v_rot_T : P.k_rot_T;
 
-    // ---- 0. one burst: plan tables, the raw rows, and (V) the rotation column -------------
+    // ---- 0. one burst: plan tables, the first tile's raw rows, and (V) the rotation column ----
+    // A work-group stages the plan once and then walks tiles bx, bx + tile_stride, ...
     if constexpr (IS_V) {
         if (j == 0) sp.v_bits = P.v_bits;
         if (j < 16) { sp.centroids[j] = P.v_centroids[j]; sp.boundaries[j] = P.v_boundaries[j]; }
@@ -108,18 +120,24 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             sp.centroids[e] = P.k_centroids[e >> 5][e & 31];
         }
     }
+    uint16_t xr[ROWS];                 // raw rows of the tile about to be processed
+    auto fetch_rows = [&](int64_t tile) {
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        int64_t n = row0 + r;
-        uint16_t v = 0;
-        if (n < N) {
-            int64_t b = n / a.S, s = n - b * a.S;
-            v = a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + j];
+        for (int r = 0; r < ROWS; r++) {
+            int64_t n = tile * ROWS + r;
+            uint16_t v = 0;
+            if (n < N) {
+                int64_t b = n / a.S, s = n - b * a.S;
+                v = a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + j];
+            }
+            xr[r] = v;
         }
-        xraw[r][j] = v;
-    }
-    // Decode append is latency bound: V's rotation column does not depend on anything, so
-    // the whole of it is requested now; K's depends on the group range and follows below.
+    };
+    fetch_rows(bx);
+    // Decode append (2-row tiles) is latency bound: this thread's column of the rotation is
+    // requested before anything else is known, V's whole dense column right away, the first 32
+    // entries of K's group range once the plan is in LDS.  16-row tiles fetch per tile instead
+    // (unrolled prefetched entries would run masked for every row of every tile).
     constexpr int PF = ROWS == 2 ? (IS_V ? D : 32) : 0;
     float rpre[PF > 0 ? PF : 1];
     if constexpr (IS_V && PF > 0) {
@@ -142,7 +160,35 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
 
-    // ---- 1. gather by head_perm (K), fp16 -> fp32 ------------------------------
+    // ---- pack geometry of output byte j (row independent) ------------------------
+    int mode = 0;        // 0: zero fill, 1: bit stream, 2: raw byte copy
+    int c0 = 0, clen = 0, bw = 1, idx = 0;
+    if constexpr (IS_V) {
+        bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : sp.v_bits;
+        if (j < bgtq_seg_bytes(bw, D)) { mode = 1; c0 = 0; clen = D; idx = j; }
+    } else if (a.layout == BGTQ_K_MIXED) {
+        int z = sp.hdr[H_NZERO], nps = sp.hdr[H_NOPACK_START];
+        int nib = (nps - z) >> 1;
+        if (j < nib)                             { mode = 1; bw = 4; c0 = z; clen = nps - z; idx = j; }
+        else if (j < nib + sp.hdr[H_NOPACK_LEN]) { mode = 2; c0 = nps + (j - nib); }
+    } else {
+        for (int s = 0; s < n_seg; s++) {
+            int off = sp.hdr[H_PACK_OFF + s], sb = sp.hdr[H_BW + s], sl = sp.hdr[H_LEN + s];
+            if (j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
+                if (sb >= 5) { mode = 2; c0 = sp.hdr[H_START + s] + (j - off); }
+                else         { mode = 1; bw = sb; c0 = sp.hdr[H_START + s]; clen = sl; idx = j - off; }
+            }
+        }
+    }
+    const StreamSlot slot = mode == 1 ? stream_slot(clen, bw, idx) : StreamSlot{0, 0, 0};
+
+    for (int64_t tile = bx; tile < n_tiles; tile += tile_stride) {
+    const int64_t row0 = tile * ROWS;
+    // ---- 1. rows to LDS, next tile's rows on their way, gather by head_perm (K) -------------
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) xraw[r][j] = xr[r];
+    __syncthreads();
+    if (tile + tile_stride < n_tiles) fetch_rows(tile + tile_stride);
 #pragma unroll
     for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xraw[r][src_dim]);
     __syncthreads();
@@ -200,11 +246,27 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             float rt[RB];
 #pragma unroll
             for (int i = 0; i < RB; i++) rt[i] = RT[min(k0 + i, ge - 1) * D + j];
+            if (IS_V) {
+                // dense rotation: the range is the whole row, so the row values can be
+                // read four at a time (same chain order)
 #pragma unroll
-            for (int i = 0; i < RB; i++) {
-                if (k0 + i < ge) {
+                for (int i = 0; i < RB; i += 4) {
 #pragma unroll
-                    for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][k0 + i], rt[i], y[r]);
+                    for (int r = 0; r < ROWS; r++) {
+                        const float4 x4 = *(const float4*)&xs[r][k0 + i];
+                        y[r] = __builtin_fmaf(x4.x, rt[i], y[r]);
+                        y[r] = __builtin_fmaf(x4.y, rt[i + 1], y[r]);
+                        y[r] = __builtin_fmaf(x4.z, rt[i + 2], y[r]);
+                        y[r] = __builtin_fmaf(x4.w, rt[i + 3], y[r]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RB; i++) {
+                    if (k0 + i < ge) {
+#pragma unroll
+                        for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][k0 + i], rt[i], y[r]);
+                    }
                 }
             }
         }
@@ -294,11 +356,10 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             if (row0 + r < N && gg < a.norm_width)
                 a.norms_f32_out[(row0 + r) * a.norm_width + gg] = nrm_out[r][gg];
         }
-        return;
     }
 
     // ---- 7b. cache norms --------------------------------------------------------
-    if (j < ROWS * BGTQ_MAX_SEGMENTS) {
+    if (!a.codes_out && j < ROWS * BGTQ_MAX_SEGMENTS) {
         int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
         int64_t n = row0 + r;
         int width = IS_V ? 1 : a.norm_width;
@@ -310,42 +371,27 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
 
     // ---- 8. pack: thread j produces output byte j of every row ---------------
-    if (j >= a.row_width) return;
-    int mode = 0;        // 0: zero fill, 1: bit stream, 2: raw byte copy
-    int c0 = 0, clen = 0, bw = 1, idx = 0;
-    if constexpr (IS_V) {
-        bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : sp.v_bits;
-        if (j < bgtq_seg_bytes(bw, D)) { mode = 1; c0 = 0; clen = D; idx = j; }
-    } else if (a.layout == BGTQ_K_MIXED) {
-        int z = sp.hdr[H_NZERO], nps = sp.hdr[H_NOPACK_START];
-        int nib = (nps - z) >> 1;
-        if (j < nib)                             { mode = 1; bw = 4; c0 = z; clen = nps - z; idx = j; }
-        else if (j < nib + sp.hdr[H_NOPACK_LEN]) { mode = 2; c0 = nps + (j - nib); }
-    } else {
-        for (int s = 0; s < n_seg; s++) {
-            int off = sp.hdr[H_PACK_OFF + s], sb = sp.hdr[H_BW + s], sl = sp.hdr[H_LEN + s];
-            if (j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
-                if (sb >= 5) { mode = 2; c0 = sp.hdr[H_START + s] + (j - off); }
-                else         { mode = 1; bw = sb; c0 = sp.hdr[H_START + s]; clen = sl; idx = j - off; }
-            }
+    if (!a.codes_out && j < a.row_width) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            int64_t n = row0 + r;
+            if (n >= N) break;
+            int64_t b = n / a.S, s = n - b * a.S;
+            int64_t t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            unsigned v = 0;
+            if (mode == 1)      v = stream_byte(&cds[r][c0], slot, bw);
+            else if (mode == 2) v = cds[r][c0];
+            a.packed[b * a.p_sb + h * a.p_sh + t * a.p_st + j] = (uint8_t)v;
         }
     }
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        int64_t n = row0 + r;
-        if (n >= N) break;
-        int64_t b = n / a.S, s = n - b * a.S;
-        int64_t t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
-        unsigned v = 0;
-        if (mode == 1)      v = stream_byte(&cds[r][c0], clen, bw, idx);
-        else if (mode == 2) v = cds[r][c0];
-        a.packed[b * a.p_sb + h * a.p_sh + t * a.p_st + j] = (uint8_t)v;
+    __syncthreads();            // the tile buffers are rewritten by the next tile
     }
 }
 
 template <int ROWS, bool IS_V>
 __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
-    encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y);
+    const int64_t N = (int64_t)a.B * a.S;
+    encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y, (N + ROWS - 1) / ROWS, gridDim.x);
 }
 
 template <bool IS_V>
@@ -359,7 +405,11 @@ int launch_encode(const EncodeArgs& a, hipStream_t st) {
         dim3 grid((unsigned)((N + 1) / 2), (unsigned)a.n_kv);
         hipLaunchKernelGGL((encode_kernel<2, IS_V>), grid, dim3(NT), 0, st, a);
     } else {
-        dim3 grid((unsigned)((N + 15) / 16), (unsigned)a.n_kv);
+        // a work-group stages its head's plan once and walks several tiles: about 10
+        // work-groups per CU in total
+        int64_t tiles = (N + 15) / 16;
+        int64_t want = (256 * 10 + a.n_kv - 1) / a.n_kv;
+        dim3 grid((unsigned)(tiles < want ? tiles : want), (unsigned)a.n_kv);
         hipLaunchKernelGGL((encode_kernel<16, IS_V>), grid, dim3(NT), 0, st, a);
     }
     return bgtq_launch_status();
@@ -411,10 +461,10 @@ __global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs a
     int bid = blockIdx.x;
     const int nk = k_tiles * ak.n_kv, nv = v_tiles * av.n_kv;
     if (bid < nk) {
-        encode_rows<2, false>(ak, bid % k_tiles, bid / k_tiles);
+        encode_rows<2, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles);
     } else if (bid < nk + nv) {
         bid -= nk;
-        encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles);
+        encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles);
     } else {
         bid -= nk + nv;
         rotate_q_row(aq, bid / aq.n_q, bid % aq.n_q);
