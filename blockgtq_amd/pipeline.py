@@ -158,3 +158,31 @@ class BlockGTQPipeline:
         if k_proj_bias is not None:
             k_proj_bias[lo:hi] = k_proj_bias[lo:hi].clone()[perm]
         self._perm_baked = True
+
+    @torch.no_grad()
+    def compress_decompress(self, k: torch.Tensor) -> torch.Tensor:
+        """Quantise-then-reconstruct ``k`` (..., D) in plain torch on ``k``'s
+        plan device: permute, per-group norm, rotate, nearest centroid,
+        renormalise the reconstruction per group, undo rotation and permutation
+        (blockgtq/block_gtq_pipeline.py:309-357).  Coordinates of 0-bit blocks
+        come back as 0, and so does a group whose input norm is 0 (as in the
+        packed record, which stores that norm; the reference's multi-group
+        branch rescales such a group by 1 instead)."""
+        assert self._calibrated
+        hd = self.head_dim
+        x = k.reshape(-1, hd).float()
+        if not self._perm_baked:
+            x = x[:, self._head_perm]
+        live = (self._group_of >= 0)
+        gidx = self._group_of.clamp(min=0)
+        norms_g = torch.sqrt((x * x) @ self._group_mask)
+        safe_g = torch.where(norms_g > 0, norms_g, torch.ones_like(norms_g))
+        per_pos = safe_g[:, gidx]
+        y = (x / per_pos) @ self._block_rot_T
+        idx_t = torch.searchsorted(self._pos_boundaries, y.T.contiguous())
+        idx_t = idx_t.clamp(max=self._pos_centroids.shape[1] - 1)
+        y_hat = self._pos_centroids[self._row_idx, idx_t].T.contiguous()
+        yh_g = torch.sqrt((y_hat * y_hat) @ self._group_mask)
+        yh_safe = torch.where(yh_g > 1e-10, yh_g, torch.ones_like(yh_g))
+        y_hat = y_hat / yh_safe[:, gidx] * norms_g[:, gidx] * live
+        return (y_hat @ self._block_rot_unperm).reshape(*k.shape[:-1], hd)

@@ -54,6 +54,9 @@ class BlockGTQProductionCache:
         self.v_norms = torch.zeros(*shape, dtype=torch.float16, device=device)
         self._ws = ops.Workspace()
         self.n_splits = 0              # partitions per (row, KV head); 0 = library default
+        # K cell search: the reference's 256-bin table (blockgtq/quantizer.py:841-850);
+        # plan.QUANT_EXACT gives the nearest centroid of the unpacked torch path
+        self.quant_mode = _plan.QUANT_LUT256
 
     # ---------------------------------------------------------------- encode
     def _encode_batched(self, layer_idx, k, v, t_pos):
@@ -67,7 +70,7 @@ class BlockGTQProductionCache:
         if v16.stride(-1) != 1:
             v16 = v16.contiguous()
         encode_k_into(plans, k16, self.k_packed[li], self.k_norms[li], t_pos,
-                      self.k_bytes_per_tok, self.max_ng, self._k_layout)
+                      self.k_bytes_per_tok, self.max_ng, self._k_layout, self.quant_mode)
         encode_v_into(plans, v16, self.v_packed[li], self.v_norms[li], t_pos,
                       self.vpb, self._v_layout)
 
@@ -106,7 +109,7 @@ class BlockGTQProductionCache:
             q3 = ops.decode_prepare(
                 plans, k16, v16, q3.contiguous(), self.k_packed[li], self.k_norms[li],
                 self.v_packed[li], self.v_norms[li], t_pos, self.k_bytes_per_tok, self.max_ng,
-                self.vpb, self.nkv, self._k_layout, self._v_layout)
+                self.vpb, self.nkv, self._k_layout, self._v_layout, self.quant_mode)
         lens = self._seq_lens + S if self._seq_lens is not None else None
         out = ops.decode_attention(
             plans, q3.contiguous(), self.k_packed[li], self.k_norms[li],

@@ -347,3 +347,35 @@ def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, v
             assert np.abs(lse.cpu().numpy() - ref_lse).max() < LSE_TOL
     finally:
         lib.bgtq_set_decode_path(0)
+
+
+def test_production_cache_tracks_the_unpacked_torch_path():
+    """No checker involved: the cache's output against softmax attention in fp64
+    over K round-tripped by the plain-torch pipeline and V round-tripped by the
+    torch V quantizer (same tables, different arithmetic and no byte format)."""
+    from blockgtq_amd import BlockGTQPipeline, BlockGTQProductionCache
+    from blockgtq_amd.calibration import build_quantizers
+    gen = torch.Generator().manual_seed(8)
+    nkv, nq, T = 2, 8, 700
+    en = wl.syn.block_energies(nkv, 64, gen)
+    amp = torch.cat([en.sqrt(), en.sqrt()], -1).unsqueeze(1)
+    layer_data = {0: {'q': torch.randn(nkv, 1024, 128, generator=gen) * amp,
+                      'k': torch.randn(nkv, 256, 128, generator=gen) * amp}}
+    quantizers, ba, ka = build_quantizers(layer_data, 1, nkv, 128, device=DEV)
+    cache = BlockGTQProductionCache(quantizers, ba, ka, 1, nkv, nq, 128, T + 8, device=DEV)
+    cache.quant_mode = P.QUANT_EXACT       # the 256-bin table moves codes near cell edges (1e-2 here)
+    k = (torch.randn(1, nkv, T + 1, 128, generator=gen) * amp).half().to(DEV)
+    v = torch.randn(1, nkv, T + 1, 128, generator=gen).half().to(DEV)
+    q = (torch.randn(1, nq, 1, 128, generator=gen) * amp.repeat_interleave(4, 0).unsqueeze(0) * 0.3).half().to(DEV)
+    cache._encode_batched(0, k[:, :, :T], v[:, :, :T], 0)
+    cache.seq_len = T
+    out = cache.encode_and_attend(0, q, k[:, :, T:], v[:, :, T:])[0, :, 0].double().cpu()
+    for hi in range(nkv):
+        q8 = quantizers[0][hi]
+        pipe = BlockGTQPipeline(128, rotation_threshold=q8.rotation_threshold, device=DEV)
+        pipe.set_allocation(q8.bit_allocation)
+        k_hat = pipe.compress_decompress(k[0, hi].float()).double().cpu()
+        v_hat = q8._v_quantizer.dequantize(*q8._v_quantizer.quantize(v[0, hi].float())).double().cpu()
+        qh = q[0, hi * 4:(hi + 1) * 4, 0].double().cpu()
+        ref = torch.softmax(qh @ k_hat.T / 128 ** 0.5, -1) @ v_hat
+        assert (out[hi * 4:(hi + 1) * 4] - ref).abs().max() < TOL
