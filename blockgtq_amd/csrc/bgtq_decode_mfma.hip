@@ -48,11 +48,20 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
 constexpr int D = BGTQ_D;
-constexpr int MT = 64;             // tokens per wave tile = 4 MFMA row blocks
+#ifndef BGTQ_MT
+#define BGTQ_MT 64
+#endif
+#ifndef BGTQ_MAX_WAVES
+#define BGTQ_MAX_WAVES 8
+#endif
+#ifndef BGTQ_KB
+#define BGTQ_KB 2
+#endif
+constexpr int MT = BGTQ_MT;        // tokens per wave tile = MT / 16 MFMA row blocks
 constexpr int NBLK = MT / 16;
 constexpr int MAX_STEPS = BGTQ_MAX_STEPS;
-constexpr int MAX_WAVES = 8;
-constexpr int KB = 2;              // K tile buffers per wave: 2 = fetched a whole tile ahead, 1 = refilled right after QK^T
+constexpr int MAX_WAVES = BGTQ_MAX_WAVES;
+constexpr int KB = BGTQ_KB;         // K tile buffers per wave: 2 = fetched a whole tile ahead, 1 = refilled right after QK^T
 constexpr int MAX_KN = 8;          // norm columns per token row the staging area can hold
 constexpr int LDS_LIMIT = 160 * 1024;
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
@@ -189,6 +198,16 @@ __device__ unsigned long long* g_trace;
 #else
 #define TRACE(slot) do {} while (0)
 #endif
+#ifdef BGTQ_TRACE
+#define TRACE_WALL(slot)                                                                         \
+    do {                                                                                         \
+        if (lane == 0)                                                                           \
+            g_trace[(((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + wave) * 64 + (slot)] = \
+                __builtin_amdgcn_s_memrealtime();                                                \
+    } while (0)
+#else
+#define TRACE_WALL(slot) do {} while (0)
+#endif
 
 template <int VBW>
 __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs a) {
@@ -206,6 +225,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     chunk = (chunk + MT - 1) / MT * MT;
     const int t0 = min(c * chunk, T), t1 = min(t0 + chunk, T);
     TRACE(0);
+    TRACE_WALL(6);
 
     // ---- LDS carve-up --------------------------------------------------------
     const int krow = a.k_row_width;
@@ -371,72 +391,107 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 #pragma unroll
         for (int k = 0; k < NBLK; k++) S[k] = (float4v){0, 0, 0, 0};
         {
-            // Software pipeline over the packed steps: while the table reads of step m are
-            // in flight, the parameters, raw codes and query unit of step m+1 are fetched.
-            // The scheduling barriers keep the compiler from folding the stages back into
-            // one dependent chain per row block.
+            // Software pipeline over the packed steps.  The iteration that multiplies step m
+            // first forms the table addresses of step m+1 (from raw codes and parameters read
+            // one iteration earlier), issues the MFMAs of step m, then fetches parameters and
+            // raw codes of step m+2 together with the query unit and norms of step m+1, and
+            // last the table words of step m+1.  Every LDS read is consumed one iteration
+            // after it was issued and every register set is rewritten only after its last
+            // reader has issued, so the loop carries no copies.  The small reads go first
+            // because the counter of outstanding LDS reads saturates at 15: the next iteration
+            // can then wait for them while most table reads are still in flight.
             const uint32_t kbase = smem_lds + kbuf + rowoff;
-            uint4v e0 = lds_at<uint4v>(stl), e1 = lds_at<uint4v>(stl + 16);
-            uint32_t rlo[NBLK] = {}, rhi[NBLK] = {};
-            half8 Q = {};
-            if (n_packed > 0) {
-                const uint32_t oa = kbase + e0.x;
+            const int last = n_packed - 1;
+            uint4v e0, e1;                                  // parameters of the step whose addresses are formed next
+            uint32_t xoff;                                  // raw-code offset of the step fetched next
+            uint32_t rlo[NBLK], rhi[NBLK];                  // raw codes
+            uint32_t ad[NBLK][4], qad, nad;                 // table, query-unit and norm addresses
+            uint4v w[NBLK];                                 // table words = the MFMA A operands
+            half8 Q;
+            half4v n4[NBLK];
+            auto params = [&](int m) {
+                const uint32_t at = stl + (uint32_t)min(m, last) * 128;
+                e0 = lds_at<uint4v>(at);
+                e1 = lds_at<uint4v>(at + 16);
+            };
+            auto raw_offset = [&](int m) { return lds_at<uint32_t>(stl + (uint32_t)min(m, last) * 128); };
+            auto raws = [&](uint32_t off) {
+                const uint32_t oa = kbase + off;
 #pragma unroll
                 for (int k = 0; k < NBLK; k++) {
                     rlo[k] = lds_at<uint32_t>(oa + k * kstride);
                     rhi[k] = lds_at<uint32_t>(oa + k * kstride + 4);
                 }
-                Q = lds_at<half8>(qrow + e1.w);
-            }
-            for (int m = 0; m < n_packed; m++) {
-                const int mn = min(m + 1, n_steps - 1);
-                const uint4v f0 = lds_at<uint4v>(stl + mn * 128), f1 = lds_at<uint4v>(stl + mn * 128 + 16);   // A: parameters of the next step
-                __builtin_amdgcn_sched_barrier(0);
-                // B: bit fields -> table reads of this step, norms of its segment
+            };
+            auto addresses = [&]() {                        // bit fields -> table addresses
                 const uint32_t lb = (lane4 & e0.w) | e0.z;
                 const uint32_t pw = e1.x, pw2 = pw * 2, pw3 = pw * 3, tsh = e1.y;
-                uint4v w[NBLK];
-                half4v n4[NBLK];
 #pragma unroll
                 for (int k = 0; k < NBLK; k++) {
                     const uint32_t raw = __builtin_amdgcn_alignbyte(rhi[k], rlo[k], e0.y);
-                    const uint32_t i0 = __builtin_amdgcn_ubfe(raw, 0, pw), i1 = __builtin_amdgcn_ubfe(raw, pw, pw);
-                    const uint32_t i2 = __builtin_amdgcn_ubfe(raw, pw2, pw), i3 = __builtin_amdgcn_ubfe(raw, pw3, pw);
+                    ad[k][0] = (__builtin_amdgcn_ubfe(raw, 0, pw) << tsh) + lb;
+                    ad[k][1] = (__builtin_amdgcn_ubfe(raw, pw, pw) << tsh) + lb;
+                    ad[k][2] = (__builtin_amdgcn_ubfe(raw, pw2, pw) << tsh) + lb;
+                    ad[k][3] = (__builtin_amdgcn_ubfe(raw, pw3, pw) << tsh) + lb;
+                }
+                qad = qrow + e1.w;
+                nad = nrm + e1.z;
+            };
+            auto operands = [&]() {                         // query unit and norms of the segment
+                Q = lds_at<half8>(qad);
+#pragma unroll
+                for (int k = 0; k < NBLK; k++) n4[k] = lds_at<half4v>(nad + k * 32);
+            };
+            auto tables = [&]() {                           // table words
+#pragma unroll
+                for (int k = 0; k < NBLK; k++)
 #ifdef BGTQ_EXPERIMENT_NOKLUT
-                    w[k] = (uint4v){(i0 << tsh) + lb, (i1 << tsh) + lb, (i2 << tsh) + lb, (i3 << tsh) + lb};
+                    w[k] = (uint4v){ad[k][0], ad[k][1], ad[k][2], ad[k][3]};
 #else
-                    w[k] = (uint4v){lds_at<uint32_t>((i0 << tsh) + lb), lds_at<uint32_t>((i1 << tsh) + lb),
-                                   lds_at<uint32_t>((i2 << tsh) + lb), lds_at<uint32_t>((i3 << tsh) + lb)};
+                    w[k] = (uint4v){lds_at<uint32_t>(ad[k][0]), lds_at<uint32_t>(ad[k][1]),
+                                   lds_at<uint32_t>(ad[k][2]), lds_at<uint32_t>(ad[k][3])};
 #endif
-                }
+            };
+            // one MFMA per row block from a zero accumulator, scaled by the fp16 group norm of
+            // its token rows in fp32
+            auto multiply = [&]() {
+                float4v d[NBLK];
 #pragma unroll
-                for (int k = 0; k < NBLK; k++) n4[k] = lds_at<half4v>(nrm + e1.z + k * 32);
+                for (int k = 0; k < NBLK; k++)
+                    d[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, w[k]), Q,
+                                                                  (float4v){0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+                for (int k = 0; k < NBLK; k++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[k][r], d[k][r], S[k][r]);
+            };
+            if (n_packed > 0) {
+                params(0);
+                const uint32_t x1 = raw_offset(1);
+                xoff = raw_offset(2);
+                raws(e0.x);
+                addresses();                                // step 0
                 __builtin_amdgcn_sched_barrier(0);
-                // C: raw codes and query unit of the next step
-                uint32_t nlo[NBLK], nhi[NBLK];
-                const uint32_t oan = kbase + f0.x;
-#pragma unroll
-                for (int k = 0; k < NBLK; k++) {
-                    nlo[k] = lds_at<uint32_t>(oan + k * kstride);
-                    nhi[k] = lds_at<uint32_t>(oan + k * kstride + 4);
-                }
-                const half8 Qn = lds_at<half8>(qrow + f1.w);
+                params(1);                                  // same order as in the loop, so that the
+                raws(x1);                                   // wait at the loop head is the same on
+                operands();                                 // both ways into it
                 __builtin_amdgcn_sched_barrier(0);
-                // D: one MFMA per row block from a zero accumulator, scaled by the fp16 group
-                //    norm of its token rows in fp32
-#pragma unroll
-                for (int k = 0; k < NBLK; k++) {
-                    const float4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, w[k]), Q,
-                                                                             (float4v){0, 0, 0, 0}, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 4; r++) S[k][r] = fmaf((float)n4[k][r], d[r], S[k][r]);
+                tables();
+                for (int m = 0; m < last; m++) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    addresses();                            // step m+1
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply();                             // step m
+                    __builtin_amdgcn_sched_barrier(0);
+                    params(m + 2);
+                    raws(xoff);                             // step m+2
+                    xoff = raw_offset(m + 3);
+                    operands();                             // step m+1
+                    __builtin_amdgcn_sched_barrier(0);
+                    tables();                               // step m+1
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                e0 = f0;
-                e1 = f1;
-                Q = Qn;
-#pragma unroll
-                for (int k = 0; k < NBLK; k++) { rlo[k] = nlo[k]; rhi[k] = nhi[k]; }
+                multiply();
             }
             TRACE(8 + trace_j * 8 + 6);
             for (int m = n_packed; m < n_steps; m++) k_raw_step(S, stl + m * 128, qrow, kbase, kstride, nrm);
@@ -500,7 +555,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                     constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
                     const int fp = e * 2 * VBW;
                     const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
+#ifdef BGTQ_EXPERIMENT_NOVLUT
+                    W[r][e] = and_or(sh, fmask, vbank);
+#else
                     W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
+#endif
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -585,6 +644,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         if (d == 0) a.part_lse[row] = (t1 > t0) ? (m + log2f(den)) * 0.69314718055994530942f : -INFINITY;
     }
     TRACE(62);
+    TRACE_WALL(7);
 }
 
 // LDS bytes of a work-group of nw waves

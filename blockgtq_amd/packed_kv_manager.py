@@ -107,7 +107,7 @@ class BlockGTQKVManager:
         if self._k_packed is not None:
             return
         # Records are padded to a 4-byte multiple so every row starts on a dword.
-        self._k_row = max(4, (self._max_k_packed_bytes + 3) // 4 * 4)
+        self._k_row = _plan.cache_row_bytes(self._max_k_packed_bytes)
         self._vpb = packed_v_bytes(self.hd, self.v_bits)
         ng = max(self._max_n_groups, 1)
         shape = (self.n_layers, self.B, self.n_kv, self.max_T)

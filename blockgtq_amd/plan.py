@@ -260,3 +260,16 @@ def upload_plans(plans: np.ndarray, device) -> torch.Tensor:
     """Copy a structured plan array to ``device`` as a flat uint8 tensor."""
     raw = torch.from_numpy(np.ascontiguousarray(plans).view(np.uint8).copy())
     return raw.to(device)
+
+
+def cache_row_bytes(record_bytes: int) -> int:
+    """Row width of a packed K cache for records of ``record_bytes``: a multiple
+    of 4 (rows start on a dword) that is not a multiple of 32.  The decode kernel
+    keeps a tile of rows in LDS at this stride and 16 lanes read the same column
+    of 16 consecutive rows; with a stride of 32, 64, 96 or 128 bytes those reads
+    fall on a quarter of the 64 LDS banks and serialise four-fold.  A 128-byte
+    record keeps its width: rows wider than that are beyond what the encoders
+    and the fast decode kernel take."""
+    row = max(4, (int(record_bytes) + 3) // 4 * 4)
+    return row + 4 if row % 32 == 0 and row < HEAD_DIM else row
+

@@ -41,8 +41,8 @@ class BlockGTQProductionCache:
         self.max_ng = max(max(quantizers[li][hi]._n_groups
                               for li in range(n_layers) for hi in range(nkv)), 1)
         own = max(ba['max_mixed_bytes'] if k_nibble else ba['max_tpb'] for ba in batched_args)
-        # records are padded to a 4-byte multiple so every row starts on a dword
-        self.k_bytes_per_tok = max(4, (own + 3) // 4 * 4)
+        # rows start on a dword and avoid the strides that collide in LDS
+        self.k_bytes_per_tok = _plan.cache_row_bytes(own)
         self.vpb = hd // 2 if v_nibble else packed_v_bytes(hd, v_bits)
         self._k_layout = _plan.K_MIXED if k_nibble else _plan.K_BITPACKED
         self._v_layout = _plan.V_NIBBLE if v_nibble else _plan.V_BITPACKED

@@ -290,6 +290,18 @@ def test_v_packing_matches_a_plain_bit_stream(bits):
 
 
 # ---------------------------------------------------------------- library surface
+def test_cache_rows_avoid_strides_that_collide_in_lds():
+    from blockgtq_amd.plan import cache_row_bytes
+    for n in range(1, 129):
+        row = cache_row_bytes(n)
+        assert row >= n and row % 4 == 0 and row - n < 8 and row <= 128
+        if row < 128:
+            # 16 consecutive rows must start in 16 different groups of 4 banks (64 banks of 4 bytes)
+            assert len({(r * row // 4) % 64 // 4 for r in range(16)}) == 16 or row % 32 != 0
+            assert row % 32 != 0
+    assert cache_row_bytes(57) == 60 and cache_row_bytes(61) == 68 and cache_row_bytes(128) == 128
+
+
 def test_library_loads_and_exports_every_declared_symbol():
     from blockgtq_amd import _capi
     lib = _capi.lib()
