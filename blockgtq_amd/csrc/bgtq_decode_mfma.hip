@@ -117,29 +117,42 @@ __device__ __forceinline__ void dma16(uint32_t voff, const uint8_t* sbase, uint3
                  : "=&s"(saved) : "v"(voff), "s"(sbase), "s"(lds_addr), "s"(lanes) : "memory", "m0");
 }
 
-__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
-    uint64_t v = (uint64_t)(uintptr_t)p;
-    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+// Same for all 64 lanes of a 1 KB chunk at a compile-time distance from sbase / lds_addr:
+// the instruction offset moves the global and the LDS address together.
+template <int OFF>
+__device__ __forceinline__ void dma_chunk(uint32_t voff, const uint8_t* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3\n"
+                 :: "v"(voff), "s"(sbase), "s"(lds_addr), "n"(OFF) : "memory", "m0");
 }
 
-// Copies the aligned 16-byte pieces of [src_al, src_al + total) to LDS.  Pieces
-// are aligned, so a piece that holds at least one wanted byte never crosses into
-// a page the range itself does not touch.  Exactly dma_count(total) load
-// instructions are issued: every 1 KB chunk but the last runs with all lanes,
-// the last one with the lanes whose piece still starts inside the range.
+// How a byte range [src_al, src_al + total) is cut into 1 KB load instructions: every
+// chunk but the last runs with all lanes, the last one with the lanes whose aligned
+// 16-byte piece still starts inside the range.  Pieces are aligned, so a piece that holds
+// at least one wanted byte never crosses into a page the range itself does not touch.
+struct DmaShape {
+    int nfull;          // chunks before the last
+    uint64_t last;      // lanes of the last chunk
+};
 __device__ __forceinline__ int dma_count(int total) { return (total + 1023) >> 10; }
+__device__ __forceinline__ DmaShape dma_shape(int total, uint32_t voff) {
+    DmaShape d;
+    d.nfull = dma_count(total) - 1;
+    d.last = __builtin_amdgcn_ballot_w64((int)voff < total - d.nfull * 1024);
+    return d;
+}
 
+// Issues the nfull + 1 loads of a range of at most NCH chunks.
 template <int NCH>
-__device__ __forceinline__ void dma_region(const uint8_t* src_al, uint32_t lds_addr, int total, uint32_t voff) {
-    src_al = uniform_ptr(src_al);
-    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
-    const int nch = dma_count(total);
-    const uint64_t last = __builtin_amdgcn_ballot_w64((int)voff < total - (nch - 1) * 1024);
+__device__ __forceinline__ void dma_region(const uint8_t* src_al, uint32_t lds_addr, const DmaShape& d, uint32_t voff) {
 #pragma unroll
-    for (int c = 0; c < NCH; c++)
-        if (c < nch) dma16(voff, src_al + c * 1024, lds_addr + c * 1024, c == nch - 1 ? last : ~0ull);
+    for (int c = 0; c + 1 < NCH; c++)
+        if (c < d.nfull) {
+            if ((c & 3) == 0) dma_chunk<0>(voff, src_al + (c >> 2) * 4096, lds_addr + (c >> 2) * 4096);
+            if ((c & 3) == 1) dma_chunk<1024>(voff, src_al + (c >> 2) * 4096, lds_addr + (c >> 2) * 4096);
+            if ((c & 3) == 2) dma_chunk<2048>(voff, src_al + (c >> 2) * 4096, lds_addr + (c >> 2) * 4096);
+            if ((c & 3) == 3) dma_chunk<3072>(voff, src_al + (c >> 2) * 4096, lds_addr + (c >> 2) * 4096);
+        }
+    dma16(voff, src_al + d.nfull * 1024, lds_addr + d.nfull * 1024, d.last);
 }
 
 // Waits until at most n of the loads issued so far are still in flight.
@@ -209,7 +222,9 @@ __device__ unsigned long long* g_trace;
 #define TRACE_WALL(slot) do {} while (0)
 #endif
 
-template <int VBW>
+// VBW: bits per V code; VST: bytes from one V record to the next (the record itself is
+// 16 * VBW bytes; a padded stride keeps the rows of a tile on different LDS banks)
+template <int VBW, int VST>
 __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -229,7 +244,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 
     // ---- LDS carve-up --------------------------------------------------------
     const int krow = a.k_row_width;
-    constexpr int vrow = 16 * VBW;
+    constexpr int vrow = VST;
     const int kn_st = (int)a.kn_st;
     const TileLayout tl = tile_layout(krow, vrow, kn_st);
     const bool kmix = a.k_layout == BGTQ_K_MIXED, vnib = a.v_layout == BGTQ_V_NIBBLE;
@@ -252,21 +267,30 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const uint32_t kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
     const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
     const uint32_t voff = (uint32_t)lane * 16;
-    // K records and both norm arrays of a tile go to K buffer `which`; returns the loads issued
+    // K records and both norm arrays of a tile go to K buffer `which`; returns the loads issued.
+    // The shapes of a full tile are the same for every tile of the partition.
+    const DmaShape full_k = dma_shape((int)kph + MT * krow, voff), full_kn = dma_shape((int)knph + MT * kn_st * 2, voff);
+    const DmaShape full_vn = dma_shape((int)vnph + MT * 2, voff), full_v = dma_shape((int)vph + MT * vrow, voff);
     auto issue_k = [&](int tile, int which) -> int {
         const int nt = min(MT, t1 - tile);
         const uint32_t buf = smem_lds + kbufs_off + (which * nw + wave) * tl.kbuf;
-        const int bk = (int)kph + nt * krow, bn = (int)knph + nt * kn_st * 2, bv = (int)vnph + nt * 2;
-        dma_region<9>(kp_base - kph + (int64_t)tile * krow, buf, bk, voff);
-        dma_region<2>(kn_base - knph + (int64_t)tile * kn_st * 2, buf + tl.kt, bn, voff);
-        dma_region<1>(vn_base - vnph + (int64_t)tile * 2, buf + tl.kt + tl.knr, bv, voff);
-        return dma_count(bk) + dma_count(bn) + dma_count(bv);
+        DmaShape sk = full_k, sn = full_kn, sv = full_vn;
+        if (nt < MT) {
+            sk = dma_shape((int)kph + nt * krow, voff);
+            sn = dma_shape((int)knph + nt * kn_st * 2, voff);
+            sv = dma_shape((int)vnph + nt * 2, voff);
+        }
+        dma_region<9>(kp_base - kph + (int64_t)tile * krow, buf, sk, voff);
+        dma_region<2>(kn_base - knph + (int64_t)tile * kn_st * 2, buf + tl.kt, sn, voff);
+        dma_region<1>(vn_base - vnph + (int64_t)tile * 2, buf + tl.kt + tl.knr, sv, voff);
+        return sk.nfull + sn.nfull + sv.nfull + 3;
     };
     auto issue_v = [&](int tile) -> int {
         const int nt = min(MT, t1 - tile);
-        const int bv = (int)vph + nt * vrow;
-        dma_region<5>(vp_base - vph + (int64_t)tile * vrow, smem_lds + vbuf_off, bv, voff);
-        return dma_count(bv);
+        DmaShape sv = full_v;
+        if (nt < MT) sv = dma_shape((int)vph + nt * vrow, voff);
+        dma_region<5>(vp_base - vph + (int64_t)tile * vrow, smem_lds + vbuf_off, sv, voff);
+        return sv.nfull + 1;
     };
     const int step_tiles = nw * MT;
     int tile = t0 + wave * MT;
@@ -287,7 +311,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             const bool isv = cc < vch;
             const int o = (isv ? cc : cc - vch) * 1024;
             const int left = (isv ? vlut_bytes(VBW) : kimg) - o;
-            dma16(voff, uniform_ptr((isv ? vimg : kimg_src) + o),
+            dma16(voff, (isv ? vimg : kimg_src) + o,
                   __builtin_amdgcn_readfirstlane(smem_lds + (isv ? 0 : VTAB_BYTES) + o),
                   __builtin_amdgcn_ballot_w64((int)voff < left));
         }
@@ -658,16 +682,16 @@ size_t mfma_smem_bytes(int k_layout, int krow, int vrow, int kn_st, int nw) {
     return s > merge ? s : merge;
 }
 
-template <int VBW>
+template <int VBW, int VST>
 int launch(const DecodeArgs& a, hipStream_t st) {
     // no more waves than the longest partition has tiles
     const int part = (a.T + a.n_splits - 1) / a.n_splits;
     int nw = (part + MT - 1) / MT;
     nw = nw < 1 ? 1 : nw > MAX_WAVES ? MAX_WAVES : nw;
-    while (nw > 1 && mfma_smem_bytes(a.k_layout, a.k_row_width, a.v_row_width, (int)a.kn_st, nw) > (size_t)LDS_LIMIT) nw--;
-    const size_t smem = mfma_smem_bytes(a.k_layout, a.k_row_width, a.v_row_width, (int)a.kn_st, nw);
+    while (nw > 1 && mfma_smem_bytes(a.k_layout, a.k_row_width, VST, (int)a.kn_st, nw) > (size_t)LDS_LIMIT) nw--;
+    const size_t smem = mfma_smem_bytes(a.k_layout, a.k_row_width, VST, (int)a.kn_st, nw);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
-    auto kern = decode_mfma_kernel<VBW>;
+    auto kern = decode_mfma_kernel<VBW, VST>;
     static int ready = 0;                    // 1: usable, -1: not usable
     if (ready == 0) {
         // the kernel addresses its V table as "LDS offset 0": that holds only while it has
@@ -698,17 +722,20 @@ int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     if (a.gqa > 16 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
     if ((a.kp_st & 3) || (a.kp_sb & 3) || (a.kp_sh & 3) || ((uintptr_t)a.kp & 3)) return BGTQ_EUNSUPPORTED;
     if ((a.vp_st & 3) || (a.vp_sb & 3) || (a.vp_sh & 3) || ((uintptr_t)a.vp & 3)) return BGTQ_EUNSUPPORTED;
-    if (a.kp_st != a.k_row_width || a.vp_st != a.v_row_width) return BGTQ_EUNSUPPORTED;   // records contiguous
+    if (a.kp_st != a.k_row_width) return BGTQ_EUNSUPPORTED;   // K records contiguous
     if (a.k_row_width < 4 || a.k_row_width > 128) return BGTQ_EUNSUPPORTED;
     if (a.vn_st != 1 || a.kn_st < 1 || a.kn_st > MAX_KN) return BGTQ_EUNSUPPORTED;
     if ((a.q_sb & 1) || (a.q_sh & 1) || ((uintptr_t)a.q & 3)) return BGTQ_EUNSUPPORTED;
     if (a.v_layout == BGTQ_V_NIBBLE && a.v_row_width != 64) return BGTQ_EUNSUPPORTED;
     // a bit-packed V record of 128 dims is 16 bytes per bit of code width, a nibble record 64
+    // V records follow each other directly, or 4 bytes apart where the record width itself
+    // (32 or 64 bytes) would put the rows of a tile on the same LDS banks
+    const int64_t pad = a.vp_st - a.v_row_width;
     switch (a.v_row_width) {
-    case 16: return launch<1>(a, stream);
-    case 32: return launch<2>(a, stream);
-    case 48: return launch<3>(a, stream);
-    case 64: return launch<4>(a, stream);
+    case 16: return pad == 0 ? launch<1, 16>(a, stream) : BGTQ_EUNSUPPORTED;
+    case 32: return pad == 0 ? launch<2, 32>(a, stream) : pad == 4 ? launch<2, 36>(a, stream) : BGTQ_EUNSUPPORTED;
+    case 48: return pad == 0 ? launch<3, 48>(a, stream) : BGTQ_EUNSUPPORTED;
+    case 64: return pad == 0 ? launch<4, 64>(a, stream) : pad == 4 ? launch<4, 68>(a, stream) : BGTQ_EUNSUPPORTED;
     default: return BGTQ_EUNSUPPORTED;
     }
 }

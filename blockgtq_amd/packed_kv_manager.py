@@ -106,7 +106,8 @@ class BlockGTQKVManager:
     def _ensure_storage(self):
         if self._k_packed is not None:
             return
-        # Records are padded to a 4-byte multiple so every row starts on a dword.
+        # Rows start on a dword and keep clear of the strides that collide in LDS; the V
+        # cache is a view of the first _vpb bytes of its (possibly wider) rows.
         self._k_row = _plan.cache_row_bytes(self._max_k_packed_bytes)
         self._vpb = packed_v_bytes(self.hd, self.v_bits)
         ng = max(self._max_n_groups, 1)
@@ -114,7 +115,8 @@ class BlockGTQKVManager:
         dev = self.device
         self._k_packed = torch.zeros(*shape, self._k_row, dtype=torch.uint8, device=dev)
         self._k_norms = torch.zeros(*shape, ng, dtype=torch.float16, device=dev)
-        self._v_packed = torch.zeros(*shape, self._vpb, dtype=torch.uint8, device=dev)
+        self._v_row = _plan.cache_row_bytes(self._vpb)
+        self._v_packed = torch.zeros(*shape, self._v_row, dtype=torch.uint8, device=dev)[..., :self._vpb]
         self._v_norms = torch.zeros(*shape, dtype=torch.float16, device=dev)
         if self.buffered:
             bshape = (self.n_layers, self.B, self.n_kv, self.n_sink + self.window, self.hd)
@@ -291,7 +293,7 @@ class BlockGTQKVManager:
         """Bytes the packed cache holds for the current length (padding included)."""
         n = self.seq_len * self.n_kv * self.B * self.n_layers
         self._ensure_storage()
-        return n * (self._k_row + self._vpb + self._k_norms.shape[-1] * 2 + 2)
+        return n * (self._k_row + self._v_row + self._k_norms.shape[-1] * 2 + 2)
 
     def fp16_cache_bytes(self) -> int:
         return self.n_layers * self.B * self.n_kv * self.seq_len * self.hd * 2 * 2

@@ -263,7 +263,7 @@ def upload_plans(plans: np.ndarray, device) -> torch.Tensor:
 
 
 def cache_row_bytes(record_bytes: int) -> int:
-    """Row width of a packed K cache for records of ``record_bytes``: a multiple
+    """Row width of a packed K or V cache for records of ``record_bytes``: a multiple
     of 4 (rows start on a dword) that is not a multiple of 32.  The decode kernel
     keeps a tile of rows in LDS at this stride and 16 lanes read the same column
     of 16 consecutive rows; with a stride of 32, 64, 96 or 128 bytes those reads

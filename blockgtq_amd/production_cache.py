@@ -50,7 +50,8 @@ class BlockGTQProductionCache:
         shape = (n_layers, batch_size, nkv, max_T)
         self.k_packed = torch.zeros(*shape, self.k_bytes_per_tok, dtype=torch.uint8, device=device)
         self.k_norms = torch.zeros(*shape, self.max_ng, dtype=torch.float16, device=device)
-        self.v_packed = torch.zeros(*shape, self.vpb, dtype=torch.uint8, device=device)
+        self._v_row = _plan.cache_row_bytes(self.vpb)      # v_packed is a view of the first vpb bytes
+        self.v_packed = torch.zeros(*shape, self._v_row, dtype=torch.uint8, device=device)[..., :self.vpb]
         self.v_norms = torch.zeros(*shape, dtype=torch.float16, device=device)
         self._ws = ops.Workspace()
         self.n_splits = 0              # partitions per (row, KV head); 0 = library default
@@ -126,7 +127,7 @@ class BlockGTQProductionCache:
     # ------------------------------------------------------------ accounting
     def cache_memory_bytes(self) -> int:
         n = self.seq_len * self.nkv * self.n_layers * self.B
-        return n * (self.k_bytes_per_tok + self.vpb + self.max_ng * 2 + 2)
+        return n * (self.k_bytes_per_tok + self._v_row + self.max_ng * 2 + 2)
 
     def fp16_cache_bytes(self) -> int:
         return self.n_layers * self.B * self.nkv * self.seq_len * self.hd * 2 * 2

@@ -338,13 +338,18 @@ def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, v
     ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
                               vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), [333] * 2, 4,
                               k_layout, v_layout, vb)
+    # the same records in rows 4 bytes wider, as the cache classes store 32- and 64-byte records
+    vw = vp.shape[-1]
+    vp_wide = torch.full((*vp.shape[:-1], P.cache_row_bytes(vw)), 0xA5, dtype=torch.uint8, device=DEV)[..., :vw]
+    vp_wide.copy_(vp)
     assert lib.bgtq_set_decode_path(2) == 0
     try:
         for ns in (1, 4):
-            out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 333, n_splits=ns,
-                                            k_layout=k_layout, v_layout=v_layout, return_lse=True)
-            assert np.abs(out.float().cpu().numpy() - ref).max() < TOL
-            assert np.abs(lse.cpu().numpy() - ref_lse).max() < LSE_TOL
+            for vrec in (vp, vp_wide):
+                out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vrec, vn, 333, n_splits=ns,
+                                                k_layout=k_layout, v_layout=v_layout, return_lse=True)
+                assert np.abs(out.float().cpu().numpy() - ref).max() < TOL
+                assert np.abs(lse.cpu().numpy() - ref_lse).max() < LSE_TOL
     finally:
         lib.bgtq_set_decode_path(0)
 
