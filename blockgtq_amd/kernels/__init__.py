@@ -1,4 +1,4 @@
-"""Fused decode attention over the packed cache, reference-compatible entry.
+"""Attention over the packed cache, reference-compatible entries.
 
 ``fused_blockgtq_decode_attention`` keeps the argument list of
 blockgtq/kernels/fused_packed_attention.py:1541-1570 so existing call sites
@@ -124,6 +124,50 @@ def fused_blockgtq_decode_attention(
     return res.unsqueeze(2)
 
 
+@torch.no_grad()
+def fused_blockgtq_prefill_attention(
+    q, k_packed, k_norms, codebook_flat, lut_offset, norm_group, segments,
+    v_codes, v_norms, v_lut,
+    scale=None, block_q=64, block_t=64, v_skip_thresh=0.0, v_norm_scale=None,
+    v_bits=0, v_rotation=None, is_causal=True, q_pos_offset=0,
+    k_nibble=False, v_nibble=False, min_seg_for_dot=16,
+):
+    """Prompt-phase attention of one KV head's query group over its packed cache
+    slice (argument list of blockgtq/kernels/fused_packed_attention.py:2597-2620).
+
+    q (B, gqa, S_q, D) fp16 already permuted + rotated; cache slices as for the
+    decode entry.  Query token s sees records ``t <= q_pos_offset + s`` when
+    ``is_causal``.  Returns (B, gqa, S_q, D) fp16.  The records are dequantised
+    in one pass (``bgtq_dequant_kv``) and the two GEMMs run in the library's
+    fused attention; ``block_q``, ``block_t`` and ``min_seg_for_dot`` tuned the
+    reference kernel and are ignored."""
+    assert q.dim() == 4
+    assert len(segments) <= 8
+    if v_skip_thresh:
+        raise NotImplementedError("v_skip_thresh changes results; not built")
+    if v_norms.dtype != torch.float16:
+        raise NotImplementedError("only fp16 V norms are supported")
+    if not v_nibble and not (1 <= int(v_bits) <= 4):
+        raise NotImplementedError("V must be bit-packed (v_bits 1..4) or nibble-packed")
+    if k_packed.shape[1] != 1:
+        raise NotImplementedError("pass one KV head per call (each head owns its plan)")
+    T = k_packed.shape[2]
+    quant = _QUANTIZER_OF_CODEBOOK.get(codebook_flat.data_ptr()) if codebook_flat.numel() else None
+    if quant is not None:
+        plans = quant.device_plan()
+    else:
+        plans = _plan_from_args(codebook_flat, segments, v_lut, v_rotation,
+                                int(v_bits) if not v_nibble else max(int(v_bits), 1), q.device)
+    if v_norms.dim() == 4:
+        v_norms = v_norms[..., 0]
+    k_hat, v_hat = ops.dequant_kv(
+        plans, k_packed, k_norms, v_codes, v_norms, T,
+        k_layout=_plan.K_MIXED if k_nibble else _plan.K_BITPACKED,
+        v_layout=_plan.V_NIBBLE if v_nibble else _plan.V_BITPACKED)
+    v_rot = None if v_rotation is None else v_rotation.reshape(1, q.shape[-1], q.shape[-1])
+    return ops.prefill_attention(q.to(torch.float16), k_hat, v_hat, v_rot, scale, is_causal, q_pos_offset)
+
+
 def build_segments_from_pack_meta(pack_meta, codebook_flat=None, pos_centroids=None):
     """``[(bw, dim_start, dim_len, pack_off, lut_off, norm_idx)]`` in ascending
     bit width (blockgtq/kernels/fused_packed_attention.py:2763-2787)."""
@@ -135,5 +179,6 @@ def build_segments_from_pack_meta(pack_meta, codebook_flat=None, pos_centroids=N
     return out
 
 
-__all__ = ["fused_blockgtq_decode_attention", "build_segments_from_pack_meta",
+__all__ = ["fused_blockgtq_decode_attention", "fused_blockgtq_prefill_attention",
+           "build_segments_from_pack_meta",
            "register_kernel_args"]

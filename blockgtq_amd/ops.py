@@ -9,6 +9,7 @@ import math
 from typing import Optional
 
 import torch
+import torch.nn.functional as F
 
 from . import _capi, plan as _plan
 
@@ -179,3 +180,67 @@ def window_attention(q: torch.Tensor, kbuf: torch.Tensor, vbuf: torch.Tensor,
         B, n_kv, n_q // n_kv, scale, _capi.ptr(po), _capi.ptr(pl), _capi.stream_ptr(q.device)),
         "bgtq_window_attn")
     return po, pl
+
+
+@torch.no_grad()
+def dequant_kv(plans: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor,
+               v_packed: torch.Tensor, v_norms: torch.Tensor, T: int, *,
+               k_layout: int = _plan.K_BITPACKED, v_layout: int = _plan.V_BITPACKED,
+               k_row_width: Optional[int] = None, v_row_width: Optional[int] = None):
+    """The first ``T`` records of a layer's packed cache as fp16 tensors.
+
+    Inputs as for ``decode_attention``.  Returns ``(k_hat, v_hat)``, both
+    (B, n_kv, T, D) fp16: K in the packed-dim order and rotated space of the
+    records (what ``rotate_q`` queries multiply with), V in its rotated space."""
+    _capi.require_cuda(k_packed, "k_packed")
+    assert k_packed.dtype == torch.uint8 and k_packed.stride(-1) == 1
+    assert v_packed.dtype == torch.uint8 and v_packed.stride(-1) == 1
+    assert k_norms.dtype == torch.float16 and v_norms.dtype == torch.float16
+    B, n_kv = k_packed.shape[:2]
+    assert k_packed.shape[2] >= T and v_packed.shape[2] >= T
+    k_row_width = k_packed.shape[-1] if k_row_width is None else k_row_width
+    v_row_width = v_packed.shape[-1] if v_row_width is None else v_row_width
+    ko = torch.empty((B, n_kv, T, _plan.HEAD_DIM), dtype=torch.float16, device=k_packed.device)
+    vo = torch.empty_like(ko)
+    _capi.check(_capi.lib().bgtq_dequant_kv(
+        _capi.ptr(plans),
+        _capi.ptr(k_packed), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2), k_row_width,
+        _capi.ptr(k_norms), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2),
+        _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), v_row_width,
+        _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
+        B, n_kv, T, k_layout, v_layout,
+        _capi.ptr(ko), ko.stride(0), ko.stride(1), ko.stride(2),
+        _capi.ptr(vo), vo.stride(0), vo.stride(1), vo.stride(2),
+        _capi.stream_ptr(k_packed.device)), "bgtq_dequant_kv")
+    return ko, vo
+
+
+@torch.no_grad()
+def prefill_attention(q_rot: torch.Tensor, k_hat: torch.Tensor, v_hat: torch.Tensor,
+                      v_rot: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                      is_causal: bool = True, q_pos_offset: int = 0) -> torch.Tensor:
+    """Attention of many query tokens over dequantised records.
+
+    q_rot (B, n_q, S, D) fp16 rotated queries; k_hat / v_hat (B, n_kv, T, D) from
+    ``dequant_kv``; ``v_rot`` (n_kv, D, D) fp32 un-rotation or None.  Query
+    token s sees records ``t <= q_pos_offset + s`` when ``is_causal``.  The
+    score/value GEMMs are the library's fused attention; returns (B, n_q, S, D) fp16."""
+    B, n_q, S, D = q_rot.shape
+    n_kv, T = k_hat.shape[1], k_hat.shape[2]
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    if is_causal and q_pos_offset == 0 and S == T:
+        out = F.scaled_dot_product_attention(q_rot, k_hat, v_hat, is_causal=True, scale=scale,
+                                             enable_gqa=True)
+    else:
+        mask = None
+        if is_causal:
+            t = torch.arange(T, device=q_rot.device)
+            mask = t[None, :] <= (q_pos_offset + torch.arange(S, device=q_rot.device))[:, None]
+        out = F.scaled_dot_product_attention(q_rot, k_hat, v_hat, attn_mask=mask, scale=scale,
+                                             enable_gqa=True)
+    if v_rot is not None:
+        gqa = n_q // n_kv
+        o = out.reshape(B, n_kv, gqa * S, D).float() @ v_rot.to(out.device, torch.float32).unsqueeze(0)
+        out = o.reshape(B, n_q, S, D).to(torch.float16)
+    return out
+

@@ -344,6 +344,29 @@ int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
                      int B, int n_kv, int gqa, float scale,
                      float* part_out, float* part_lse, void* stream);
 
+/*
+ * Packed records back to fp16 vectors, all KV heads of a layer in one launch:
+ * the tile dequantisation of the reference's prompt-phase attention kernel
+ * (blockgtq/kernels/fused_packed_attention.py:1876-2594, helpers :1384-1533)
+ * as a pass of its own.  Causal attention of bgtq_rotate_q's queries over
+ * k_out / v_out, followed by the V un-rotation, equals attention over the
+ * packed cache.
+ *   inputs     as for bgtq_decode_attn (same strides, layouts and row widths)
+ *   k_out      fp16 [B][n_kv][T][128] in the packed-dim order and rotated space of
+ *              the records: fp16(codebook[code] * group norm), 0 on 0-bit dims;
+ *              strides ko_sb/ko_sh/ko_st in halves
+ *   v_out      fp16 [B][n_kv][T][128] in rotated V space: fp16(centroid[code] * norm)
+ */
+int bgtq_dequant_kv(const bgtq_head_plan* plans,
+                    const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                    const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                    const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                    const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                    int B, int n_kv, int T, int k_layout, int v_layout,
+                    void* k_out, int64_t ko_sb, int64_t ko_sh, int64_t ko_st,
+                    void* v_out, int64_t vo_sb, int64_t vo_sh, int64_t vo_st,
+                    void* stream);
+
 #ifdef __cplusplus
 }
 #endif

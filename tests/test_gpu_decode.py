@@ -384,3 +384,97 @@ def test_production_cache_tracks_the_unpacked_torch_path():
         qh = q[0, hi * 4:(hi + 1) * 4, 0].double().cpu()
         ref = torch.softmax(qh @ k_hat.T / 128 ** 0.5, -1) @ v_hat
         assert (out[hi * 4:(hi + 1) * 4] - ref).abs().max() < TOL
+
+
+@pytest.mark.parametrize("k_layout,v_layout,vb", [(0, 0, 3), (1, 1, 3), (0, 0, 2), (1, 0, 4)])
+def test_dequantised_records_equal_the_checker_bit_for_bit(oracle_lib, k_layout, v_layout, vb):
+    mn = 0 if vb == 2 else 1
+    args, qs, q_rot, kp, kn, vp, vn = _build(160, mn, 6, vb, 2, 4, 2, 211, seed=40 + vb + k_layout,
+                                             k_layout=k_layout, v_layout=v_layout)
+    T = 209                                   # not a multiple of the kernel's token tile
+    k_hat, v_hat = ops.dequant_kv(args['plans'], kp, kn, vp, vn, T, k_layout=k_layout, v_layout=v_layout)
+    assert k_hat.shape == (2, 2, T, 128) and v_hat.dtype == torch.float16
+    for b in range(2):
+        for h in range(2):
+            pl = args['plans_np'][h:h + 1]
+            ng = int(pl[0]['n_seg'])
+            codes = oracle_lib.unpack_k(pl, kp[b, h, :T].cpu().numpy(), k_layout)
+            ref_k = oracle_lib.dequant_k(pl, codes, kn[b, h, :T, :max(ng, 1)].cpu().numpy())
+            vcodes = oracle_lib.unpack_v(vp[b, h, :T].cpu().numpy(), vb if not v_layout else 4, bool(v_layout))
+            ref_v = oracle_lib.dequant_v(pl, vcodes, vn[b, h, :T].cpu().numpy())
+            # centroid (fp16) x norm (fp16) is exact in fp32, so one rounding on either side
+            assert np.array_equal(k_hat[b, h].cpu().numpy().view(np.uint16), ref_k.astype(np.float16).view(np.uint16))
+            assert np.array_equal(v_hat[b, h].cpu().numpy().view(np.uint16), ref_v.astype(np.float16).view(np.uint16))
+
+
+def _causal_reference(orc, pl, q_rot, kp, kn, vp, vn, k_layout, v_layout, vb, offset, scale=128 ** -0.5):
+    """fp64 attention of q_rot (gqa, S, 128) over one head's records, row s seeing t <= offset + s."""
+    T = kp.shape[0]
+    ng = int(pl[0]['n_seg'])
+    k_hat = orc.dequant_k(pl, orc.unpack_k(pl, kp, k_layout), kn[:, :max(ng, 1)]).astype(np.float64)
+    v_hat = orc.dequant_v(pl, orc.unpack_v(vp, vb if not v_layout else 4, bool(v_layout)), vn).astype(np.float64)
+    logits = q_rot.astype(np.float64) @ k_hat.T * scale
+    S = q_rot.shape[1]
+    mask = np.arange(T)[None, :] <= (offset + np.arange(S))[:, None]
+    logits = np.where(mask[None], logits, -np.inf)
+    p = np.exp(logits - logits.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    return (p @ v_hat) @ pl[0]['v_rot'].reshape(128, 128).astype(np.float64)
+
+
+@pytest.mark.parametrize("k_layout,v_layout", [(0, 0), (1, 1)])
+def test_prompt_attention_over_the_packed_cache(oracle_lib, k_layout, v_layout):
+    """Reference-style per-head entry: whole prompt (S = T), and a later chunk of
+    queries against a longer cache (q_pos_offset)."""
+    from blockgtq_amd.kernels import fused_blockgtq_prefill_attention
+    from helpers import make_kv
+    vb, T, gqa = 3, 150, 4
+    args, qs, _, kp, kn, vp, vn = _build(192, 1, 6, vb, 2, gqa, 1, T, seed=61 + k_layout,
+                                         k_layout=k_layout, v_layout=v_layout)
+    gen = torch.Generator().manual_seed(5)
+    for hi in range(2):
+        q8 = qs[hi]
+        a = q8.build_kernel_args()
+        q = (torch.randn(1, gqa, T, 128, generator=gen) * 0.7).half().to(DEV)
+        q_rot = q8.rotate_q_for_packed_kernel(q)
+        pl = args['plans_np'][hi:hi + 1]
+        sl = lambda x: x[:, hi:hi + 1, :T]
+        for S, off in ((T, 0), (37, T - 37)):
+            out = fused_blockgtq_prefill_attention(
+                q_rot[:, :, T - S:], sl(kp), sl(kn), a['codebook_flat'], a['lut_offset'], a['norm_group'],
+                a['segments_b'], sl(vp), sl(vn), q8.v_lut, v_bits=vb, v_rotation=q8._v_rot,
+                is_causal=True, q_pos_offset=off, k_nibble=bool(k_layout), v_nibble=bool(v_layout))
+            assert out.shape == (1, gqa, S, 128) and out.dtype == torch.float16
+            ref = _causal_reference(oracle_lib, pl, q_rot[0, :, T - S:].cpu().numpy(), kp[0, hi, :T].cpu().numpy(),
+                                    kn[0, hi, :T].cpu().numpy(), vp[0, hi, :T].cpu().numpy(),
+                                    vn[0, hi, :T].cpu().numpy(), k_layout, v_layout, vb, off)
+            assert np.abs(out[0].double().cpu().numpy() - ref).max() < TOL
+
+
+def test_prompt_attention_rows_equal_decode_steps():
+    """Size-independent property through the cache class: row s of the prompt-phase
+    attention is the decode attention of that query over the first s + 1 records."""
+    from blockgtq_amd import BlockGTQProductionCache
+    from blockgtq_amd.calibration import build_quantizers
+    from blockgtq_amd.prefill import packed_prefill_attention
+    gen = torch.Generator().manual_seed(12)
+    nkv, nq, T = 2, 8, 300
+    en = wl.syn.block_energies(nkv, 64, gen)
+    amp = torch.cat([en.sqrt(), en.sqrt()], -1).unsqueeze(1)
+    layer_data = {0: {'q': torch.randn(nkv, 1024, 128, generator=gen) * amp,
+                      'k': torch.randn(nkv, 256, 128, generator=gen) * amp}}
+    quantizers, ba, ka = build_quantizers(layer_data, 1, nkv, 128, device=DEV)
+    cache = BlockGTQProductionCache(quantizers, ba, ka, 1, nkv, nq, 128, T + 8, device=DEV, batch_size=2)
+    k = (torch.randn(2, nkv, T, 128, generator=gen) * amp).half().to(DEV)
+    v = torch.randn(2, nkv, T, 128, generator=gen).half().to(DEV)
+    q = (torch.randn(2, nq, T, 128, generator=gen) * 0.5).half().to(DEV)
+    cache._encode_batched(0, k, v, 0)
+    full = packed_prefill_attention(cache, 0, q, T)
+    assert full.shape == (2, nq, T, 128)
+    plans = ba[0]['plans']
+    for s in (0, 63, 64, 299):
+        q_rot = ops.rotate_q(plans, q[:, :, s].contiguous(), nkv)
+        dec = ops.decode_attention(plans, q_rot, cache.k_packed[0], cache.k_norms[0], cache.v_packed[0],
+                                   cache.v_norms[0], s + 1, k_layout=cache._k_layout, v_layout=cache._v_layout,
+                                   k_row_width=cache.k_bytes_per_tok, v_row_width=cache.vpb)
+        assert (full[:, :, s].float() - dec.float()).abs().max() < TOL
