@@ -65,7 +65,7 @@ class _Timer:
 @torch.no_grad()
 def run(model_name="qwen2.5-3b", batch=4, prompt_len=8192, new_tokens=256, k_bits=3.0, v_bits=3,
         device="cuda:0", seed=1234, n_layers=None, n_calib=256, fp16_baseline=True,
-        max_bits=5, return_logits=False):
+        max_bits=5, return_logits=False, graph=True):
     from . import _capi
     from .calibration import build_quantizers, collect_qk_activations
     from .fp16_baseline import FP16KVCache, fp16_decode_step
@@ -113,31 +113,77 @@ def run(model_name="qwen2.5-3b", batch=4, prompt_len=8192, new_tokens=256, k_bit
         out_logits = {"packed_prefill": logits.float().cpu()}
 
     # ---- packed decode -----------------------------------------------------------------------
+    # The first steps run eagerly (per-layer attention time comes from them); the rest is one
+    # HIP graph of the whole step (model layers, append, attention, merge, greedy pick, position
+    # and length updates) replayed once per token.
     attn = _Timer()
     ea = cache.encode_and_attend
+    n_eager = min(8, new_tokens) if graph else new_tokens
     tok, toks = first, []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(new_tokens):
-        timed = i >= new_tokens - 8           # per-layer attention time from the last steps
+    for i in range(n_eager):
+        timed = i >= n_eager - 8              # per-layer attention time from the last eager steps
         cache.encode_and_attend = (lambda *a, **kw: attn(ea, *a, **kw)) if timed else ea
         pos = torch.full((batch, 1), prompt_len + i, device=device, dtype=torch.long)
         step_logits = production_decode_step(model, tok, pos, cache)
         if return_logits and i == 0:
             out_logits["packed_step0"] = step_logits.float().cpu()
+        if return_logits and not graph:
+            out_logits[f"eager_step{i}"] = step_logits.float().cpu()
         tok = step_logits.argmax(-1)
         toks.append(tok)
     torch.cuda.synchronize()
-    decode_s = time.perf_counter() - t0
+    eager_s = time.perf_counter() - t0
     cache.encode_and_attend = ea
-    attn_us = attn.total_ms() * 1e3 / (8 * L)
+    attn_us = attn.total_ms() * 1e3 / (min(8, n_eager) * L)
+    graph_s, n_graph = 0.0, new_tokens - n_eager
+    if n_graph > 0:
+        cache.use_device_lengths()
+        ids = tok.clone()
+        pos = torch.full((batch, 1), prompt_len + n_eager, device=device, dtype=torch.long)
+        logits_buf = [None]
+
+        def step():
+            lg = production_decode_step(model, ids, pos, cache)
+            logits_buf[0] = lg
+            ids.copy_(lg.argmax(-1))
+            pos.add_(1)
+
+        state = (ids.clone(), pos.clone(), cache._seq_lens.clone(), cache.seq_len)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            step()
+        ids.copy_(state[0]); pos.copy_(state[1]); cache._seq_lens.copy_(state[2])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_graph):
+            g.replay()
+            toks.append(ids.clone())
+            if return_logits and i < 3:
+                out_logits[f"graph_step{i}"] = logits_buf[0].float().cpu()
+        torch.cuda.synchronize()
+        graph_s = time.perf_counter() - t0
+        cache.seq_len = state[3] + n_graph
+    if return_logits:
+        out_logits["tokens"] = torch.cat(toks, 1).cpu()
+    decode_s = eager_s + graph_s
     out = {
         "model": model_name, "layers": L, "batch": batch, "prompt_len": prompt_len,
         "new_tokens": new_tokens, "k_bits_avg": k_bits, "v_bits": v_bits,
         "data": "random-init bf16 weights, uniform random token ids", "calibration_s": round(calib_s, 1),
         "prefill_ms": round(prefill_ms, 1), "prefill_pack_ms": round(pack_ms, 2),
-        "decode_tokens_per_s": round(batch * new_tokens / decode_s, 1),
-        "decode_ms_per_step": round(decode_s / new_tokens * 1e3, 3),
+        "decode_tokens_per_s": round(batch * (n_graph / graph_s if n_graph else new_tokens / decode_s), 1),
+        "decode_ms_per_step": round((graph_s / n_graph if n_graph else decode_s / new_tokens) * 1e3, 3),
+        "decode_mode": "HIP graph of the whole step" if n_graph else "eager",
+        "decode_tokens_per_s_eager": round(batch * n_eager / eager_s, 1),
         "attn_us_per_layer": round(attn_us, 2),
         "packed_cache_bytes": cache.cache_memory_bytes(), "fp16_cache_bytes": cache.fp16_cache_bytes(),
     }
@@ -180,9 +226,10 @@ def main():
     ap.add_argument("--v-bits", type=int, default=3)
     ap.add_argument("--layers", type=int, default=0)
     ap.add_argument("--no-fp16", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="decode eagerly instead of replaying a HIP graph")
     a = ap.parse_args()
     print(json.dumps(run(a.model, a.batch, a.prompt_len, a.new_tokens, a.k_bits, a.v_bits,
-                         n_layers=a.layers or None, fp16_baseline=not a.no_fp16)))
+                         n_layers=a.layers or None, fp16_baseline=not a.no_fp16, graph=not a.no_graph)))
 
 
 if __name__ == "__main__":

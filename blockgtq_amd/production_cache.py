@@ -36,6 +36,7 @@ class BlockGTQProductionCache:
         self.scale = 1.0 / math.sqrt(hd)
         self.seq_len = 0
         self._seq_lens = None
+        self._static_T = None          # launch bound used instead of seq_len in graph mode
         self.max_T = max_T
 
         self.max_ng = max(max(quantizers[li][hi]._n_groups
@@ -78,14 +79,26 @@ class BlockGTQProductionCache:
     _encode_graphed = _encode_batched      # single-token appends take the same path
 
     def set_seq_lens(self, seq_lens):
-        """Per-row visible lengths for a ragged batch (``None``: one shared length)."""
+        """Per-row visible lengths for a ragged batch (``None``: one shared length).
+        The cache keeps its own copy and advances it in place."""
         if seq_lens is None:
             self._seq_lens = None
+            self._static_T = None
             return
-        t = torch.as_tensor(seq_lens, dtype=torch.int32).to(self.device)
+        t = torch.as_tensor(seq_lens, dtype=torch.int32).to(self.device).clone()
         assert t.numel() == self.B
         self._seq_lens = t
         self.seq_len = int(t.max().item())
+
+    def use_device_lengths(self):
+        """Keep the lengths on the device only, so that a decode step contains no
+        host-side number that changes from step to step and can be recorded into a
+        HIP graph once and replayed: append positions and visible lengths come from
+        the device copy, launches are sized for ``max_T``.  ``seq_len`` on the host
+        then counts the steps issued, not replays."""
+        if self._seq_lens is None:
+            self._seq_lens = torch.full((self.B,), self.seq_len, dtype=torch.int32, device=self.device)
+        self._static_T = self.max_T
 
     # ---------------------------------------------------------------- decode
     @torch.no_grad()
@@ -94,7 +107,7 @@ class BlockGTQProductionCache:
         li = layer_idx
         S = k.shape[2]
         t_pos = self._seq_lens if self._seq_lens is not None else self.seq_len
-        T = self.seq_len + S
+        T = self._static_T if self._static_T is not None else self.seq_len + S
         plans = self.batched_args[li]['plans']
         B = q.shape[0]
         q3 = q.reshape(B, self.nq, self.hd)
@@ -122,7 +135,7 @@ class BlockGTQProductionCache:
     def increment_seq_len(self, by=1):
         self.seq_len += by
         if self._seq_lens is not None:
-            self._seq_lens = self._seq_lens + by
+            self._seq_lens.add_(by)
 
     # ------------------------------------------------------------ accounting
     def cache_memory_bytes(self) -> int:
