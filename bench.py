@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per attention launch from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy
 # kernel of known size (profiles/decode_mfma_kernel_<workload>_hbm_traffic.txt); valid for the
 # workload's own context, batch and default partition count only.
-MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 65.13e6}
+MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 66.06e6}
 
 
 def parse():
@@ -43,6 +43,9 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--k-row-bytes", type=int, default=0,
+                    help="force the row width of every layer's K cache (measurement knob: 64 shows the "
+                         "LDS bank collisions the default widths avoid); 0 = the manager's choice")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run a device-to-device copy of this many MiB (a kernel of known HBM "
                          "traffic, to calibrate FETCH_SIZE / WRITE_SIZE counter readings)")
@@ -61,7 +64,7 @@ def cpu_baseline(mgr, w, q_rot_layer0, seconds, packed_lens):
     cores = min(os.cpu_count() or 1, 16)
     T = max(packed_lens)
     li = 0
-    kp = mgr._k_packed[li, :, :, :T].cpu().numpy()
+    kp = mgr._k_packed[li][:, :, :T].cpu().numpy()
     kn = mgr._k_norms[li, :, :, :T].cpu().numpy()
     vp = mgr._v_packed[li, :, :, :T].cpu().numpy()
     vn = mgr._v_norms[li, :, :, :T].cpu().numpy()
@@ -115,6 +118,8 @@ def main():
 
     t_setup = time.perf_counter()
     mgr, energies = wl.build_manager(w, dev, max_T=w.context + 8, n_layers=L)
+    if args.k_row_bytes:
+        mgr.force_k_row_bytes(args.k_row_bytes)
     wl.fill_cache(mgr, w, energies, dev)
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t_setup
@@ -187,7 +192,7 @@ def main():
     def attn_only(li):
         _capi.check(lib.bgtq_decode_attn(
             _capi.ptr(plans0[li]), _capi.ptr(q_rots[li]), q_rots[li].stride(0), q_rots[li].stride(1),
-            _capi.ptr(mgr._k_packed[li]), *mgr._k_packed[li].stride()[:3], mgr._k_row,
+            _capi.ptr(mgr._k_packed[li]), *mgr._k_packed[li].stride()[:3], mgr._k_rows[li],
             _capi.ptr(mgr._k_norms[li]), *mgr._k_norms[li].stride()[:3],
             _capi.ptr(mgr._v_packed[li]), *mgr._v_packed[li].stride()[:3], mgr._vpb,
             _capi.ptr(mgr._v_norms[li]), *mgr._v_norms[li].stride()[:3],
@@ -234,7 +239,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": (MEASURED_TRAFFIC_BYTES.get(w.name)
-                                 if not (args.context or args.splits) else None),
+                                 if not (args.context or args.splits or args.k_row_bytes) else None),
                      "kernel": "decode attention",
                      "algorithmic_bytes_per_launch": int(alg_bytes),
                      "avg_launch_us": round(attn_us, 3)},

@@ -108,12 +108,17 @@ class BlockGTQKVManager:
             return
         # Rows start on a dword and keep clear of the strides that collide in LDS; the V
         # cache is a view of the first _vpb bytes of its (possibly wider) rows.
-        self._k_row = _plan.cache_row_bytes(self._max_k_packed_bytes)
+        # every layer's K cache has its own row width (the widest record of that layer)
+        self._k_rows = [_plan.cache_row_bytes(max(ba['max_tpb'], 1) if ba is not None else self._max_k_packed_bytes)
+                        for ba in self._batched_args]
+        if getattr(self, '_forced_k_row', 0):
+            self._k_rows = [self._forced_k_row] * self.n_layers
+        self._k_row = max(self._k_rows)
         self._vpb = packed_v_bytes(self.hd, self.v_bits)
         ng = max(self._max_n_groups, 1)
         shape = (self.n_layers, self.B, self.n_kv, self.max_T)
         dev = self.device
-        self._k_packed = torch.zeros(*shape, self._k_row, dtype=torch.uint8, device=dev)
+        self._k_packed = [torch.zeros(*shape[1:], w, dtype=torch.uint8, device=dev) for w in self._k_rows]
         self._k_norms = torch.zeros(*shape, ng, dtype=torch.float16, device=dev)
         self._v_row = _plan.cache_row_bytes(self._vpb)
         self._v_packed = torch.zeros(*shape, self._v_row, dtype=torch.uint8, device=dev)[..., :self._vpb]
@@ -122,6 +127,14 @@ class BlockGTQKVManager:
             bshape = (self.n_layers, self.B, self.n_kv, self.n_sink + self.window, self.hd)
             self._buf_k = torch.zeros(bshape, dtype=torch.float16, device=dev)
             self._buf_v = torch.zeros(bshape, dtype=torch.float16, device=dev)
+
+    def force_k_row_bytes(self, row_bytes: int):
+        """Use ``row_bytes`` as the K row width of every layer instead of the
+        widths ``_ensure_storage`` would choose (measurement knob; call before the
+        first append).  Must hold the widest record and be a multiple of 4."""
+        assert self._k_packed is None, "storage is already allocated"
+        assert row_bytes % 4 == 0 and row_bytes >= self._max_k_packed_bytes
+        self._forced_k_row = int(row_bytes)
 
     def set_seq_lens(self, seq_lens):
         """Per-row visible lengths (ragged batch); ``None`` returns to one shared length."""
@@ -145,7 +158,7 @@ class BlockGTQKVManager:
         if v16.stride(-1) != 1:
             v16 = v16.contiguous()
         encode_k_into(plans, k16, self._k_packed[li], self._k_norms[li], t_pos,
-                      self._k_row, self._k_norms.shape[-1], _plan.K_BITPACKED)
+                      self._k_rows[li], self._k_norms.shape[-1], _plan.K_BITPACKED)
         encode_v_into(plans, v16, self._v_packed[li], self._v_norms[li], t_pos,
                       self._vpb, _plan.V_BITPACKED)
 
@@ -219,7 +232,7 @@ class BlockGTQKVManager:
         old_v = bv[ar, :, slot].unsqueeze(2)
         q_rot = ops.decode_prepare(
             plans, old_k, old_v, q3, self._k_packed[li], self._k_norms[li],
-            self._v_packed[li], self._v_norms[li], t_flush, self._k_row,
+            self._v_packed[li], self._v_norms[li], t_flush, self._k_rows[li],
             self._k_norms.shape[-1], self._vpb, self.n_kv, _plan.K_BITPACKED, _plan.V_BITPACKED)
         bk[ar, :, slot] = k_new[:, :, 0].to(torch.float16)
         bv[ar, :, slot] = v_new[:, :, 0].to(torch.float16)
@@ -229,7 +242,7 @@ class BlockGTQKVManager:
             plans, q_rot, self._k_packed[li], self._k_norms[li],
             self._v_packed[li], self._v_norms[li], T, seq_lens=packed_len, n_splits=self.n_splits,
             k_layout=_plan.K_BITPACKED, v_layout=_plan.V_BITPACKED, scale=self.scale,
-            k_row_width=self._k_row, v_row_width=self._vpb, workspace=self._ws,
+            k_row_width=self._k_rows[li], v_row_width=self._vpb, workspace=self._ws,
             extra_out=ext_out, extra_lse=ext_lse)
         return out.unsqueeze(2)
 
@@ -260,7 +273,7 @@ class BlockGTQKVManager:
             v16 = v16 if v16.stride(-1) == 1 else v16.contiguous()
             q3 = ops.decode_prepare(
                 plans, k16, v16, q3.contiguous(), self._k_packed[li], self._k_norms[li],
-                self._v_packed[li], self._v_norms[li], t_pos, self._k_row,
+                self._v_packed[li], self._v_norms[li], t_pos, self._k_rows[li],
                 self._k_norms.shape[-1], self._vpb, self.n_kv, _plan.K_BITPACKED, _plan.V_BITPACKED)
         lens = None
         if self._seq_lens is not None:
@@ -271,7 +284,7 @@ class BlockGTQKVManager:
             plans, q3.contiguous(), self._k_packed[li], self._k_norms[li],
             self._v_packed[li], self._v_norms[li], T, seq_lens=lens, n_splits=self.n_splits,
             k_layout=_plan.K_BITPACKED, v_layout=_plan.V_BITPACKED, scale=self.scale,
-            k_row_width=self._k_row, v_row_width=self._vpb, workspace=self._ws)
+            k_row_width=self._k_rows[li], v_row_width=self._vpb, workspace=self._ws)
         return out.unsqueeze(2)
 
     def increment_seq_len(self):
@@ -291,9 +304,9 @@ class BlockGTQKVManager:
     # ------------------------------------------------------------- accounting
     def cache_memory_bytes(self) -> int:
         """Bytes the packed cache holds for the current length (padding included)."""
-        n = self.seq_len * self.n_kv * self.B * self.n_layers
         self._ensure_storage()
-        return n * (self._k_row + self._v_row + self._k_norms.shape[-1] * 2 + 2)
+        per_token = sum(self._k_rows) + self.n_layers * (self._v_row + self._k_norms.shape[-1] * 2 + 2)
+        return self.seq_len * self.n_kv * self.B * per_token
 
     def fp16_cache_bytes(self) -> int:
         return self.n_layers * self.B * self.n_kv * self.seq_len * self.hd * 2 * 2

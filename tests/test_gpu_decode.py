@@ -223,17 +223,17 @@ def test_full_size_properties_config1():
     plans = mgr._batched_args[0]['plans']
     q_rot = ops.rotate_q(plans, q, w.n_kv)
     args = (mgr._k_packed[0], mgr._k_norms[0], mgr._v_packed[0], mgr._v_norms[0])
-    base = ops.decode_attention(plans, q_rot, *args, T, n_splits=1, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+    base = ops.decode_attention(plans, q_rot, *args, T, n_splits=1, k_row_width=mgr._k_rows[0], v_row_width=mgr._vpb).float()
     for ns in (7, 64, 512):
-        o = ops.decode_attention(plans, q_rot, *args, T, n_splits=ns, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+        o = ops.decode_attention(plans, q_rot, *args, T, n_splits=ns, k_row_width=mgr._k_rows[0], v_row_width=mgr._vpb).float()
         assert (o - base).abs().max() < 1e-3
     perm = torch.randperm(T, generator=torch.Generator().manual_seed(1)).to(DEV)
     shuffled = tuple(t[:, :, :T][:, :, perm].contiguous() for t in args)
-    o = ops.decode_attention(plans, q_rot, *shuffled, T, n_splits=16, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+    o = ops.decode_attention(plans, q_rot, *shuffled, T, n_splits=16, k_row_width=mgr._k_rows[0], v_row_width=mgr._vpb).float()
     assert (o - base).abs().max() < 1e-3
     # doubling the context by repeating it leaves the output unchanged
     doubled = tuple(torch.cat([t[:, :, :T], t[:, :, :T]], dim=2).contiguous() for t in args)
-    o = ops.decode_attention(plans, q_rot, *doubled, 2 * T, n_splits=32, k_row_width=mgr._k_row, v_row_width=mgr._vpb).float()
+    o = ops.decode_attention(plans, q_rot, *doubled, 2 * T, n_splits=32, k_row_width=mgr._k_rows[0], v_row_width=mgr._vpb).float()
     assert (o - base).abs().max() < 1e-3
 
 
