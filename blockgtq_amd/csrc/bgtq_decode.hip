@@ -515,7 +515,7 @@ int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
 }
 
 size_t bgtq_plan_sizeof(void) { return sizeof(bgtq_head_plan); }
-int bgtq_abi_version(void) { return 1; }
+int bgtq_abi_version(void) { return 2; }
 
 const char* bgtq_strerror(int code) {
     switch (code) {

@@ -74,11 +74,11 @@ constexpr int QROW = 400;                      // one head: zero unit + up to 24
 constexpr int VTAB_BYTES = 8192;
 __host__ __device__ constexpr int kimg_bytes(int k_layout) { return k_layout == BGTQ_K_MIXED ? BGTQ_LUTM_V : BGTQ_LUT_V; }
 __host__ __device__ constexpr int vlut_bytes(int vbw) { return vbw == 4 ? 256 * 32 : (1 << (2 * vbw)) * 128; }
-__host__ __device__ constexpr int steptab_off(int kimg) { return VTAB_BYTES + kimg; }   // [step][lane group] x 32 B
-__host__ __device__ constexpr int qpad_off(int kimg) { return steptab_off(kimg) + MAX_STEPS * 4 * 32; }
+__host__ __device__ constexpr int steptab_off(int kimg) { return VTAB_BYTES + kimg; }   // [step][column half][lane group] x 32 B
+__host__ __device__ constexpr int qpad_off(int kimg) { return steptab_off(kimg) + MAX_STEPS * 8 * 32; }
 __host__ __device__ constexpr int waves_off(int kimg) { return qpad_off(kimg) + 16 * QROW; }
 constexpr int WAVE_NORM_BYTES = BGTQ_MAX_SEGMENTS * MT * 2 + MT * 4;   // fp16 K norms [seg][token], fp32 V norms
-constexpr int INIT_SCRATCH = MAX_STEPS * 4 * 32 + 256 + 16 * D * 2;
+constexpr int INIT_SCRATCH = MAX_STEPS * 8 * 32 + 256 + 16 * D * 2;
 
 struct TileLayout {
     int kt, vt, knr, vnr, kbuf;    // bytes of the K, V, K-norm, V-norm areas; K + both norm areas
@@ -319,24 +319,36 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     int k0_loads = 0;
     if (tile < t1) k0_loads = issue_k(tile, 0);
     TRACE(1);
-    uint32_t* st_raw = (uint32_t*)scratch;                // steptab as stored in the plan
-    int* qu_s = (int*)(scratch + MAX_STEPS * 4 * 32);     // qunit_dim[32], qunit_len[32]
-    uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 4 * 32 + 256);   // [16][128] rotated queries
-    const uint32_t* st_src = kmix ? &P.steptab_mixed[0][0][0] : &P.steptab[0][0][0];
+    // Step table per (step, column half, lane group).  Query groups of at most 8 heads use the
+    // plan's two-segment schedule (the halves differ); larger groups need all 16 columns for
+    // heads and run the one-segment schedule with both halves alike.
+    const bool dense = gqa <= 8;
+    uint32_t* st_raw = (uint32_t*)scratch;                // step table as stored in the plan
+    int* qu_s = (int*)(scratch + MAX_STEPS * 8 * 32);     // qunit_dim[32], qunit_len[32]
+    uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 8 * 32 + 256);   // [16][128] rotated queries
     const int32_t* qu_src = kmix ? P.qunit_dim_mixed : P.qunit_dim;     // qunit_len follows qunit_dim
-    for (int i = tid; i < MAX_STEPS * 4 * 8; i += nthr) st_raw[i] = st_src[i];
+    if (dense) {
+        const uint32_t* st_src = kmix ? &P.steptab_dense_mixed[0][0][0][0] : &P.steptab_dense[0][0][0][0];
+        for (int i = tid; i < MAX_STEPS * 8 * 8; i += nthr) st_raw[i] = st_src[i];
+    } else {
+        const uint32_t* st_src = kmix ? &P.steptab_mixed[0][0][0] : &P.steptab[0][0][0];
+        for (int i = tid; i < MAX_STEPS * 8 * 8; i += nthr) st_raw[i] = st_src[(i >> 6) * 32 + (i & 31)];
+    }
     for (int i = tid; i < 64; i += nthr) qu_s[i] = qu_src[i];
     for (int i = tid; i < 16 * D / 2; i += nthr) {
         int hq = i / (D / 2), d2 = i - hq * (D / 2);
+        const int src = dense ? (hq & 7) : hq;              // columns 8..15 repeat heads 0..7
         uint32_t v = 0;
-        if (hq < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + hq) * a.q_sh + d2 * 2);
+        if (src < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + src) * a.q_sh + d2 * 2);
         ((uint32_t*)q_s)[i] = v;
     }
-    const int n_steps = min(kmix ? P.n_steps_mixed : P.n_steps, MAX_STEPS);
-    const int n_packed = min(kmix ? P.n_packed_steps_mixed : P.n_packed_steps, n_steps);   // raw-byte steps come last
+    const int n_steps = min(dense ? (kmix ? P.n_steps_dense_mixed : P.n_steps_dense)
+                                  : (kmix ? P.n_steps_mixed : P.n_steps), MAX_STEPS);
+    const int n_packed = min(dense ? (kmix ? P.n_packed_steps_dense_mixed : P.n_packed_steps_dense)
+                                   : (kmix ? P.n_packed_steps_mixed : P.n_packed_steps), n_steps);   // raw-byte steps come last
     __syncthreads();
     TRACE(2);
-    for (int i = tid; i < n_steps * 4; i += nthr) {        // the row offset depends on the cache's alignment
+    for (int i = tid; i < n_steps * 8; i += nthr) {        // the row offset depends on the cache's alignment
         const uint32_t* r = st_raw + i * 8;
         const uint32_t o = kph + r[0];
         steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2] + smem_lds + VTAB_BYTES, r[3]};     // table as an absolute LDS address
@@ -367,7 +379,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const uint32_t kstride = 16u * krow;
     const uint32_t vc = vph + (uint32_t)li * VBW;
     const uint32_t vbase = smem_lds + vbuf_off + (vc & ~3u) + (uint32_t)lg * 4 * vrow, v_sh = vc & 3u;
-    const uint32_t stl = smem_lds + steptab_off(kimg) + lg * 32;         // absolute LDS addresses from here on
+    const uint32_t stl = smem_lds + steptab_off(kimg) + (li >> 3) * 128 + lg * 32;   // absolute LDS addresses from here on
     const uint32_t qrow = smem_lds + qpad_off(kimg) + li * QROW;
     const uint32_t nrm = smem_lds + norm_off + lg * 8;
     const uint32_t vnf = smem_lds + norm_off + BGTQ_MAX_SEGMENTS * MT * 2;
@@ -434,11 +446,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             half8 Q;
             half4v n4[NBLK];
             auto params = [&](int m) {
-                const uint32_t at = stl + (uint32_t)min(m, last) * 128;
+                const uint32_t at = stl + (uint32_t)min(m, last) * 256;
                 e0 = lds_at<uint4v>(at);
                 e1 = lds_at<uint4v>(at + 16);
             };
-            auto raw_offset = [&](int m) { return lds_at<uint32_t>(stl + (uint32_t)min(m, last) * 128); };
+            auto raw_offset = [&](int m) { return lds_at<uint32_t>(stl + (uint32_t)min(m, last) * 256); };
             auto raws = [&](uint32_t off) {
                 const uint32_t oa = kbase + off;
 #pragma unroll
@@ -518,7 +530,23 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                 multiply();
             }
             TRACE(8 + trace_j * 8 + 6);
-            for (int m = n_packed; m < n_steps; m++) k_raw_step(S, stl + m * 128, qrow, kbase, kstride, nrm);
+            for (int m = n_packed; m < n_steps; m++) k_raw_step(S, stl + m * 256, qrow, kbase, kstride, nrm);
+            if (dense) {
+                // the two column halves hold the partial sums of different segments: add them, so
+                // that column c and column c ^ 8 both carry the full score of head c & 7
+#pragma unroll
+                for (int k = 0; k < NBLK; k++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+{
+                        // (through a scalar: bit-casting the vector element in place makes the
+                        // compiler read element 0 of the vector for every r)
+                        const float x = S[k][r];
+                        const int rot = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x),
+                                                                    0x128 /* row_ror:8 */, 0xf, 0xf, false);
+                        S[k][r] = x + __builtin_bit_cast(float, rot);
+                    }
+            }
         }
         if (KB == 1 && more) k_loads = issue_k(tile + step_tiles, 0);   // all reads of the K buffer are done
         TRACE(8 + trace_j * 8 + 3);

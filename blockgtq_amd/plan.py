@@ -43,6 +43,9 @@ PLAN_DTYPE = np.dtype([
     ('n_steps_mixed', '<i4'), ('n_packed_steps_mixed', '<i4'), ('reserved3', '<i4', (2,)),
     ('steptab_mixed', '<u4', (MAX_STEPS, 4, 8)), ('qunit_dim_mixed', '<i4', (32,)),
     ('qunit_len_mixed', '<i4', (32,)), ('lut_image_mixed', '<u4', (43008 // 4,)),
+    ('n_steps_dense', '<i4'), ('n_packed_steps_dense', '<i4'),
+    ('n_steps_dense_mixed', '<i4'), ('n_packed_steps_dense_mixed', '<i4'),
+    ('steptab_dense', '<u4', (MAX_STEPS, 2, 4, 8)), ('steptab_dense_mixed', '<u4', (MAX_STEPS, 2, 4, 8)),
 ], align=True)
 
 # byte offsets inside lut_image (BGTQ_LUT_* of include/bgtq.h)
@@ -126,7 +129,56 @@ def fill_decode_steps(p) -> None:
         t = _pair_table(p['v_lut_f16'], vb)
         img[LUT_V // 4:LUT_V // 4 + t.size] = t
     p['lut_image'] = img
+    _fill_dense(p, '')
     _fill_mixed_tables(p)
+
+
+def _fill_dense(p, suffix: str) -> None:
+    """Two-segment schedule for query groups of at most 8 heads, derived from the
+    one-segment schedule ``steptab<suffix>``: the packed units keep their order and
+    their table entries, but a step takes the next four of them as long as they
+    belong to at most two segments; the first segment of a step owns column half
+    0, the second half 1.  Raw-byte steps follow unchanged (half 1 all zero)."""
+    tab = p['steptab' + suffix]
+    n_steps, n_packed = int(p['n_steps' + suffix]), int(p['n_packed_steps' + suffix])
+    units = []                                   # table rows of the real packed units, in order
+    for m in range(n_packed):
+        for g in range(4):
+            row = tab[m, g]
+            if int(row[7]) != 0:
+                units.append(row.copy())
+    dense = p['steptab_dense' + suffix]
+    dense[...] = 0
+    m = i = 0
+    while i < len(units):
+        step, segs = [], []
+        while i < len(units) and len(step) < 4:
+            seg = int(units[i][6])
+            if seg not in segs:
+                if len(segs) == 2:
+                    break
+                segs.append(seg)
+            step.append(units[i])
+            i += 1
+        for half in range(2):
+            own = segs[min(half, len(segs) - 1)]
+            for g in range(4):
+                row = step[min(g, len(step) - 1)].copy()
+                mine = g < len(step) and int(row[6]) == own and (half == 0 or len(segs) == 2)
+                row[7] = row[7] if mine else 0
+                row[6] = own
+                dense[m, half, g] = row
+        m += 1
+    n_dense_packed = m
+    for r in range(n_packed, n_steps):           # raw-byte steps: half 0 as it is, half 1 silent
+        if m >= MAX_STEPS:
+            raise ValueError("segment table needs more MFMA steps than the plan holds")
+        dense[m, 0] = tab[r]
+        dense[m, 1] = tab[r]
+        dense[m, 1, :, 7] = 0
+        m += 1
+    p['n_steps_dense' + suffix] = m
+    p['n_packed_steps_dense' + suffix] = n_dense_packed
 
 
 def _byte_pair_table(cb16: np.ndarray, bw: int) -> np.ndarray:
@@ -183,6 +235,7 @@ def _fill_mixed_tables(p) -> None:
     if 1 <= vb <= 4:
         img[LUTM_V // 4:LUTM_V // 4 + 2048] = _byte_pair_table(p['v_lut_f16'], vb)
     p['lut_image_mixed'] = img
+    _fill_dense(p, '_mixed')
 
 
 def build_head_plan(quantizer) -> np.ndarray:

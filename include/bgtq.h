@@ -155,6 +155,27 @@ typedef struct bgtq_head_plan {
     int32_t  qunit_dim_mixed[32];
     int32_t  qunit_len_mixed[32];
     uint32_t lut_image_mixed[BGTQ_LUTM_IMAGE_BYTES / 4];
+
+    /*
+     * Denser schedules for query groups of at most 8 heads, where half of the
+     * MFMA's 16 output columns is free: a packed step may hold units of TWO
+     * segments.  The units of the step's first segment multiply query units
+     * that are non-zero only in columns 0..7, those of its second segment only in
+     * columns 8..15, so every segment still accumulates on its own, is scaled by
+     * its own norm, and the two column halves are added once per tile.
+     * steptab_dense[m][c][g]: as steptab[m][g], for the lanes of column half c;
+     * [6] is the norm row of the segment that owns half c in step m and [7] is
+     * query unit 0 (all zero) unless unit g's segment owns half c.  Steps of one
+     * segment (all raw-byte steps among them) give half 1 nothing but zero query
+     * units.  Query unit numbers are those of qunit_dim / qunit_len (or their
+     * _mixed forms).
+     */
+    int32_t  n_steps_dense;
+    int32_t  n_packed_steps_dense;
+    int32_t  n_steps_dense_mixed;
+    int32_t  n_packed_steps_dense_mixed;
+    uint32_t steptab_dense[BGTQ_MAX_STEPS][2][4][8];
+    uint32_t steptab_dense_mixed[BGTQ_MAX_STEPS][2][4][8];
 } bgtq_head_plan;
 
 /* sizeof(bgtq_head_plan) as the library was compiled; the host mirror checks it. */

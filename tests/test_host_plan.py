@@ -11,7 +11,7 @@ import torch
 from blockgtq_amd import BlockGTQPipeline, BlockGTQQuantizer, greedy_bit_allocation
 from blockgtq_amd import codebooks, plan as P, v_packing
 from blockgtq_amd.quantizer import build_pack_meta
-from helpers import make_quantizer, stream_pack
+from helpers import make_kv, make_quantizer, stream_pack
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -290,6 +290,74 @@ def test_v_packing_matches_a_plain_bit_stream(bits):
 
 
 # ---------------------------------------------------------------- library surface
+def _emulate_steps(p, rec, norms, qrot, dense, mixed):
+    """Scores of one token record computed the way the MFMA kernel walks the plan's step
+    tables: per (step, column half, lane group) one unit of 8 codes through the pair table
+    (or the raw-byte table), times the query unit, scaled by the norm row of the half."""
+    sfx = '_mixed' if mixed else ''
+    img = (p['lut_image_mixed'] if mixed else p['lut_image']).view(np.uint8)
+    qd, ql = p['qunit_dim' + sfx], p['qunit_len' + sfx]
+    if dense:
+        tab, ns, npk = p['steptab_dense' + sfx], int(p['n_steps_dense' + sfx]), int(p['n_packed_steps_dense' + sfx])
+    else:
+        t = p['steptab' + sfx]
+        tab, ns, npk = np.stack([t, t], 1), int(p['n_steps' + sfx]), int(p['n_packed_steps' + sfx])
+    out = np.zeros((2, qrot.shape[0]))
+    recp = np.concatenate([rec, np.zeros(16, np.uint8)])
+    for m in range(ns):
+        for half in range(2):
+            acc = np.zeros(qrot.shape[0])
+            for g in range(4):
+                off, _, table, _mask, pw, tsh, nrm_off, qoff = (int(x) for x in tab[m, half, g])
+                uid = qoff // 16
+                if uid == 0:
+                    continue
+                d0, ln = int(qd[uid]), int(ql[uid])
+                if m < npk:
+                    raw = int.from_bytes(recp[off:off + 8].tobytes(), 'little')
+                    vals = []
+                    for i in range(4):
+                        a = table + (((raw >> (i * pw)) & ((1 << pw) - 1)) << tsh)
+                        vals += list(img[a:a + 4].view(np.float16))
+                else:
+                    vals = [img[table + 2 * int(recp[off + i]):][:2].view(np.float16)[0] for i in range(8)]
+                acc += qrot[:, d0:d0 + ln].astype(np.float64) @ np.array(vals[:ln], np.float64)
+            out[half] += acc * float(norms[int(tab[m, half, 0][6]) // 128])
+    return out.sum(0) if dense else out[0]
+
+
+@pytest.mark.parametrize("seed,min_bits,max_bits,budget", [(9, 1, 7, 200), (4, 0, 4, 128), (5, 1, 5, 192), (2, 2, 2, 128)])
+def test_step_tables_reproduce_the_checker_scores(oracle_lib, seed, min_bits, max_bits, budget):
+    """Both schedules (one segment per step; two segments per step in separate column
+    halves) and both record layouts, walked on the CPU, give q . dequant(k) of the checker
+    exactly; the two-segment schedule never needs more steps and its halves agree on
+    everything but query unit and norm row."""
+    q, en = make_quantizer(seed=seed, min_bits=min_bits, max_bits=max_bits, budget=budget)
+    k, _, qq = make_kv(en, 4, seed=seed)
+    plan = q.plan()
+    p = plan[0]
+    ng = int(p['n_seg'])
+    codes, raw, corr = oracle_lib.encode_k(plan, k)
+    qr = oracle_lib.rotate_q(plan, qq).astype(np.float32)
+    for mixed in (False, True):
+        sfx = '_mixed' if mixed else ''
+        assert 1 <= int(p['n_steps_dense' + sfx]) <= int(p['n_steps' + sfx])
+        d = p['steptab_dense' + sfx][:int(p['n_steps_dense' + sfx])]
+        assert np.array_equal(d[:, 0, :, :6], d[:, 1, :, :6])
+        for m in range(d.shape[0]):
+            both = (d[m, 0, :, 7] != 0) & (d[m, 1, :, 7] != 0)
+            assert not both.any()                        # a unit feeds one half only
+            assert len({int(x) for x in d[m, :, :, 6].ravel()}) <= 2
+        kp = oracle_lib.pack_k(plan, codes, int(mixed))
+        nr = (corr if mixed else raw)[:, :max(ng, 1)]
+        kn = oracle_lib.f2h(nr).view(np.float16).astype(np.float32)
+        for t in range(k.shape[0]):
+            ref = qr.astype(np.float64) @ oracle_lib.dequant_k(plan, codes[t:t + 1], oracle_lib.f2h(nr[t:t + 1]))[0].astype(np.float64)
+            for dense in (False, True):
+                got = _emulate_steps(p, kp[t], kn[t], qr, dense, mixed)
+                assert np.abs(got - ref).max() < 1e-9
+
+
 def test_cache_rows_avoid_strides_that_collide_in_lds():
     from blockgtq_amd.plan import cache_row_bytes
     for n in range(1, 129):
