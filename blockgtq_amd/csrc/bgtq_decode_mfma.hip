@@ -21,11 +21,15 @@
 // triples and yields the eight fp16 operands of one MFMA k-group.
 //
 // QK^T:  v_mfma_f32_16x16x32_f16, A = dequantised K (row = token, lane group g
-//        supplies unit 4m+g of step m; a step never mixes segments, so field
-//        width and table are the same for the whole wave), B = rotated queries
-//        stored per unit in LDS (zero on padding dims), D[token][head].  Each
-//        segment accumulates on its own and is scaled by the fp16 group norm of
-//        its token row, in fp32, when the segment ends.
+//        supplies unit g of step m; field width and table come from the step
+//        table per lane group), B = rotated queries stored per unit in LDS (zero
+//        on padding dims), D[token][head].  Every step starts from a zero
+//        accumulator and is scaled by the fp16 group norm of its token rows in
+//        fp32.  With more than 8 query heads a step holds units of one segment.
+//        With at most 8, columns 8..15 repeat heads 0..7 and a step may hold two
+//        segments: the first one's query units are non-zero only in columns 0..7,
+//        the second one's only in columns 8..15, each half is scaled by its own
+//        segment's norm and the halves are added once per tile.
 // PV:    the D layout of two 16-token blocks is exactly the A layout of a
 //        K=32 step (row = head, lane group g holds 8 tokens), so P never leaves
 //        its lane; B = dequantised V where lane (j, g) decodes unit j of its 8
