@@ -161,21 +161,17 @@ __device__ __forceinline__ void dma_region(const uint8_t* src_al, uint32_t lds_a
 
 // Waits until at most n of the loads issued so far are still in flight.
 __device__ __forceinline__ void wait_loads(int n) {
+#define BGTQ_WAIT_CASE(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
     switch (n) {
-    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
-    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
-    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
-    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
-    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
-    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-    case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
-    default: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+    BGTQ_WAIT_CASE(0) BGTQ_WAIT_CASE(1) BGTQ_WAIT_CASE(2) BGTQ_WAIT_CASE(3) BGTQ_WAIT_CASE(4) BGTQ_WAIT_CASE(5)
+    BGTQ_WAIT_CASE(6) BGTQ_WAIT_CASE(7) BGTQ_WAIT_CASE(8) BGTQ_WAIT_CASE(9) BGTQ_WAIT_CASE(10) BGTQ_WAIT_CASE(11)
+    BGTQ_WAIT_CASE(12) BGTQ_WAIT_CASE(13) BGTQ_WAIT_CASE(14) BGTQ_WAIT_CASE(15) BGTQ_WAIT_CASE(16) BGTQ_WAIT_CASE(17)
+    BGTQ_WAIT_CASE(18) BGTQ_WAIT_CASE(19) BGTQ_WAIT_CASE(20) BGTQ_WAIT_CASE(21) BGTQ_WAIT_CASE(22) BGTQ_WAIT_CASE(23)
+    BGTQ_WAIT_CASE(24) BGTQ_WAIT_CASE(25) BGTQ_WAIT_CASE(26) BGTQ_WAIT_CASE(27) BGTQ_WAIT_CASE(28) BGTQ_WAIT_CASE(29)
+    BGTQ_WAIT_CASE(30) BGTQ_WAIT_CASE(31) BGTQ_WAIT_CASE(32) BGTQ_WAIT_CASE(33) BGTQ_WAIT_CASE(34) BGTQ_WAIT_CASE(35)
+    default: asm volatile("s_waitcnt vmcnt(36)" ::: "memory"); break;
     }
+#undef BGTQ_WAIT_CASE
 }
 
 // One step of raw byte codes (bw 5..8): one table read per code.
@@ -300,9 +296,49 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     int tile = t0 + wave * MT;
     int v_loads = 0;                 // loads of the V tile issued after the current K tile
 
-    // ---- init: tables, step parameters, query units -------------------------------------
-    // The pair tables come ready-made from the plan and are copied into LDS by DMA, each
-    // wave taking every nw-th KB; the first K tile follows right behind them.
+    // ---- init: step parameters, query units, tables --------------------------------------
+    // Everything a work-group needs comes in by DMA, in the order in which it is needed: first
+    // the small things the set-up code reads (step table, query-unit map, rotated queries) into
+    // a scratch area, then the pair tables, then the first K and V tiles.  Loads of one wave
+    // land in issue order, so the set-up can run on the small things while the table image and
+    // the first tiles are still on their way.
+    //
+    // Step table per (step, column half, lane group).  Query groups of at most 8 heads use the
+    // plan's two-segment schedule (the halves differ); larger groups need all 16 columns for
+    // heads and run the one-segment schedule with both halves alike.
+    const bool dense = gqa <= 8;
+    uint32_t* st_raw = (uint32_t*)scratch;                // step table as stored in the plan
+    int* qu_s = (int*)(scratch + MAX_STEPS * 8 * 32);     // qunit_dim[32], qunit_len[32]
+    uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 8 * 32 + 256);   // [16][128] rotated queries
+    const uint32_t scratch_lds = smem_lds + (uint32_t)(scratch - smem);
+    const uint8_t* st_src = dense ? (const uint8_t*)(kmix ? &P.steptab_dense_mixed[0][0][0][0] : &P.steptab_dense[0][0][0][0])
+                                  : (const uint8_t*)(kmix ? &P.steptab_mixed[0][0][0] : &P.steptab[0][0][0]);
+    const uint8_t* qu_src = (const uint8_t*)(kmix ? P.qunit_dim_mixed : P.qunit_dim);   // qunit_len follows qunit_dim
+    const uint8_t* q_src = (const uint8_t*)(a.q + b * a.q_sb + (int64_t)h * gqa * a.q_sh);
+    const bool q_dma = ((((uintptr_t)q_src) | (uintptr_t)(a.q_sh * 2)) & 15) == 0;   // rows on 16-byte boundaries
+    int n_small = 0;                                      // small loads of this wave, first in its queue
+    for (int j = wave; j < 8; j += nw) {                  // 3 KB step table, 256 B unit map, 4 x 4 query rows
+        if (j < 3) {
+            const uint32_t i = (uint32_t)j * 64 + lane;                          // 16-byte piece of the LDS copy
+            const uint32_t m = i >> 4, g = (i >> 1) & 3, part = i & 1;           // piece = (step, half, group, part)
+            dma16(dense ? i * 16 : ((m * 4 + g) * 2 + part) * 16, st_src, scratch_lds + j * 1024, ~0ull);
+            n_small++;
+        } else if (j == 3) {
+            dma16(voff, qu_src, scratch_lds + MAX_STEPS * 8 * 32, 0xFFFFull);
+            n_small++;
+        } else if (q_dma) {
+            const int row = (j - 4) * 4 + (lane >> 4);
+            const int src = dense ? (row & 7) : row;                             // columns 8..15 repeat heads 0..7
+            const uint64_t ok = __builtin_amdgcn_ballot_w64(src < gqa);
+            if (src >= gqa) ((uint4*)q_s)[row * 16 + (lane & 15)] = uint4{0, 0, 0, 0};
+            if (ok) {
+                dma16((uint32_t)(src * (int)a.q_sh * 2 + (lane & 15) * 16), q_src,
+                      scratch_lds + MAX_STEPS * 8 * 32 + 256 + (j - 4) * 1024, ok);
+                n_small++;
+            }
+        }
+    }
+    int n_later = 0;                                      // loads issued behind the small ones
     {
         // V table of the value layout in use at LDS offset 0, K tables of the record layout
         // in use behind it; the chunks of both are dealt round-robin to the waves
@@ -318,38 +354,30 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             dma16(voff, (isv ? vimg : kimg_src) + o,
                   __builtin_amdgcn_readfirstlane(smem_lds + (isv ? 0 : VTAB_BYTES) + o),
                   __builtin_amdgcn_ballot_w64((int)voff < left));
+            n_later++;
         }
     }
+    // first tiles; the V tile only if its buffer does not lie under the scratch area
+    const bool v_early = KB == 2 && (size_t)nw * tl.kbuf >= (size_t)INIT_SCRATCH;
     int k0_loads = 0;
-    if (tile < t1) k0_loads = issue_k(tile, 0);
+    if (tile < t1) {
+        k0_loads = issue_k(tile, 0);
+        if (v_early) v_loads = issue_v(tile);
+    }
     TRACE(1);
-    // Step table per (step, column half, lane group).  Query groups of at most 8 heads use the
-    // plan's two-segment schedule (the halves differ); larger groups need all 16 columns for
-    // heads and run the one-segment schedule with both halves alike.
-    const bool dense = gqa <= 8;
-    uint32_t* st_raw = (uint32_t*)scratch;                // step table as stored in the plan
-    int* qu_s = (int*)(scratch + MAX_STEPS * 8 * 32);     // qunit_dim[32], qunit_len[32]
-    uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 8 * 32 + 256);   // [16][128] rotated queries
-    const int32_t* qu_src = kmix ? P.qunit_dim_mixed : P.qunit_dim;     // qunit_len follows qunit_dim
-    if (dense) {
-        const uint32_t* st_src = kmix ? &P.steptab_dense_mixed[0][0][0][0] : &P.steptab_dense[0][0][0][0];
-        for (int i = tid; i < MAX_STEPS * 8 * 8; i += nthr) st_raw[i] = st_src[i];
-    } else {
-        const uint32_t* st_src = kmix ? &P.steptab_mixed[0][0][0] : &P.steptab[0][0][0];
-        for (int i = tid; i < MAX_STEPS * 8 * 8; i += nthr) st_raw[i] = st_src[(i >> 6) * 32 + (i & 31)];
-    }
-    for (int i = tid; i < 64; i += nthr) qu_s[i] = qu_src[i];
-    for (int i = tid; i < 16 * D / 2; i += nthr) {
-        int hq = i / (D / 2), d2 = i - hq * (D / 2);
-        const int src = dense ? (hq & 7) : hq;              // columns 8..15 repeat heads 0..7
-        uint32_t v = 0;
-        if (src < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + src) * a.q_sh + d2 * 2);
-        ((uint32_t*)q_s)[i] = v;
-    }
+    if (!q_dma)                                           // odd query strides: through registers
+        for (int i = tid; i < 16 * D / 2; i += nthr) {
+            int hq = i / (D / 2), d2 = i - hq * (D / 2);
+            const int src = dense ? (hq & 7) : hq;
+            uint32_t v = 0;
+            if (src < gqa) v = *(const uint32_t*)(a.q + b * a.q_sb + (h * gqa + src) * a.q_sh + d2 * 2);
+            ((uint32_t*)q_s)[i] = v;
+        }
     const int n_steps = min(dense ? (kmix ? P.n_steps_dense_mixed : P.n_steps_dense)
                                   : (kmix ? P.n_steps_mixed : P.n_steps), MAX_STEPS);
     const int n_packed = min(dense ? (kmix ? P.n_packed_steps_dense_mixed : P.n_packed_steps_dense)
                                    : (kmix ? P.n_packed_steps_mixed : P.n_packed_steps), n_steps);   // raw-byte steps come last
+    wait_loads(n_later + k0_loads + v_loads);              // this wave's small loads have landed
     __syncthreads();
     TRACE(2);
     for (int i = tid; i < n_steps * 8; i += nthr) {        // the row offset depends on the cache's alignment
@@ -365,9 +393,9 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         const uint32_t lo = 2 * pp < len ? row[d0] : 0, hi = 2 * pp + 1 < len ? row[d0 + 1] : 0;
         ((uint32_t*)qpad)[i] = lo | (hi << 16);
     }
-    wait_loads(k0_loads);                                   // this wave's share of the tables has landed
+    wait_loads(k0_loads + v_loads);                         // this wave's share of the tables has landed
     __syncthreads();                                        // scratch is dead from here
-    if (tile < t1) v_loads = issue_v(tile);
+    if (tile < t1 && !v_early) v_loads = issue_v(tile);
     TRACE(4);
 #ifdef BGTQ_TRACE
     int trace_j = 0;
