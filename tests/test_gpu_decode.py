@@ -237,6 +237,51 @@ def test_full_size_properties_config1():
     assert (o - base).abs().max() < 1e-3
 
 
+@pytest.mark.parametrize("name", ["qwen3b_b8_32k_k3v3", "llama8b_128k_k2v2"])
+def test_full_size_properties_long_contexts(name):
+    """The 32k-token batch-8 workload and the 131072-token K2V2 workload (0-bit blocks,
+    heavy-tailed data), one layer at full size: invariance to the partition count and to
+    the order of the context, equality of the two decode kernels, and the LSE of a context
+    repeated twice (+ln 2)."""
+    from blockgtq_amd import _capi
+    lib = _capi.lib()
+    w = wl.WORKLOADS[name]
+    mgr, energies = wl.build_manager(w, DEV, n_layers=1)
+    wl.fill_cache(mgr, w, energies, DEV)
+    T = mgr.seq_len
+    assert T == w.context
+    q = wl.draw_q(w, 0, DEV, T)[:, :, 0].contiguous()
+    plans = mgr._batched_args[0]['plans']
+    q_rot = ops.rotate_q(plans, q, w.n_kv)
+    args = (mgr._k_packed[0], mgr._k_norms[0], mgr._v_packed[0], mgr._v_norms[0])
+    kw = dict(k_row_width=mgr._k_rows[0], v_row_width=mgr._vpb, return_lse=True)
+    base, base_lse = ops.decode_attention(plans, q_rot, *args, T, n_splits=0, **kw)
+    base = base.float()
+    assert torch.isfinite(base).all() and torch.isfinite(base_lse).all()
+    tol = 2e-3 * max(1.0, float(base.abs().max()))
+    for ns in (1, 37, 512):
+        o, l = ops.decode_attention(plans, q_rot, *args, T, n_splits=ns, **kw)
+        assert (o.float() - base).abs().max() < tol and (l - base_lse).abs().max() < LSE_TOL
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(3)).to(DEV)
+    shuffled = tuple(t[:, :, :T][:, :, perm].contiguous() for t in args)
+    o, l = ops.decode_attention(plans, q_rot, *shuffled, T, n_splits=64, **kw)
+    assert (o.float() - base).abs().max() < tol and (l - base_lse).abs().max() < LSE_TOL
+    del shuffled
+    if w.batch * T <= 1 << 18:                    # the layout-agnostic kernel is slow: long single rows only
+        assert lib.bgtq_set_decode_path(1) == 0
+        try:
+            o, l = ops.decode_attention(plans, q_rot, *args, T, n_splits=128, **kw)
+        finally:
+            lib.bgtq_set_decode_path(0)
+        assert (o.float() - base).abs().max() < tol and (l - base_lse).abs().max() < LSE_TOL
+    half = T // 2                                  # first half repeated twice: same output, LSE + ln 2
+    o1, l1 = ops.decode_attention(plans, q_rot, *args, half, n_splits=0, **kw)
+    twice = tuple(torch.cat([t[:, :, :half], t[:, :, :half]], dim=2).contiguous() for t in args)
+    o2, l2 = ops.decode_attention(plans, q_rot, *twice, 2 * half, n_splits=0, **kw)
+    assert (o2.float() - o1.float()).abs().max() < tol
+    assert (l2 - l1 - float(np.log(2.0))).abs().max() < LSE_TOL
+
+
 def test_window_partial_merges_like_one_softmax(oracle_lib):
     """Closed form: softmax over [window ++ packed] == lse-merge of the two partials."""
     from blockgtq_amd import _capi
