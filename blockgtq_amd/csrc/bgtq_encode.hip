@@ -427,24 +427,30 @@ __device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t ro
     __shared__ float xs[D];
     const int j = threadIdx.x;
     const bgtq_head_plan& P = a.plans[hq / a.gqa];
-    xs[j] = bgtq_h2f(a.q[row * a.q_sr + hq * a.q_sh + P.head_perm[j]]);
-    __syncthreads();
+    // One round of independent loads: the thread's whole column of the rotation, its source
+    // dim and its group; the group's range comes from the (wave-uniform) segment table.
+    float rcol[D];
+#pragma unroll
+    for (int i = 0; i < D; i++) rcol[i] = P.k_rot_T[i * D + j];
+    const int src = P.head_perm[j];
     const int g = P.group_of[j];
+    int s = 0, e = 0, ident = 0;
+#pragma unroll
+    for (int k = 0; k < BGTQ_MAX_SEGMENTS; k++) {
+        const int ks = P.seg_start[k], kl = P.seg_len[k], ki = P.seg_identity[k];
+        if (k == g) { s = ks; e = ks + kl; ident = ki; }
+    }
+    xs[j] = bgtq_h2f(a.q[row * a.q_sr + hq * a.q_sh + src]);
+    __syncthreads();
     float acc = 0.f;
     if (g >= 0) {
-        if (P.seg_identity[g]) {
+        if (ident) {
             acc = xs[j];
         } else {
-            const int s = P.seg_start[g], e = s + P.seg_len[g];
-            constexpr int RB = 16;
-            for (int k0 = s; k0 < e; k0 += RB) {
-                float rt[RB];
+            // the same chain as over the group's own range: entries outside it are skipped
 #pragma unroll
-                for (int i = 0; i < RB; i++) rt[i] = P.k_rot_T[min(k0 + i, e - 1) * D + j];
-#pragma unroll
-                for (int i = 0; i < RB; i++)
-                    if (k0 + i < e) acc = __builtin_fmaf(xs[k0 + i], rt[i], acc);
-            }
+            for (int i = 0; i < D; i++)
+                if (i >= s && i < e) acc = __builtin_fmaf(xs[i], rcol[i], acc);
         }
     }
     a.q_rot[row * a.qr_sr + hq * a.qr_sh + j] = bgtq_f2h(acc);
