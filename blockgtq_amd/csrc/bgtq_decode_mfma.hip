@@ -204,7 +204,7 @@ __device__ __forceinline__ void k_raw_step(float4v (&S)[NBLK], uint32_t st, uint
 __device__ unsigned long long* g_trace;
 #define TRACE(slot)                                                                              \
     do {                                                                                         \
-        if (lane == 0 && (slot) < 64)                                                            \
+        if (lane == 0 && (slot) < 64 && g_trace)                                                 \
             g_trace[(((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + wave) * 64 + (slot)] = \
                 __builtin_readcyclecounter();                                                    \
     } while (0)
@@ -214,7 +214,7 @@ __device__ unsigned long long* g_trace;
 #ifdef BGTQ_TRACE
 #define TRACE_WALL(slot)                                                                         \
     do {                                                                                         \
-        if (lane == 0)                                                                           \
+        if (lane == 0 && g_trace)                                                                \
             g_trace[(((size_t)(blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + wave) * 64 + (slot)] = \
                 __builtin_amdgcn_s_memrealtime();                                                \
     } while (0)

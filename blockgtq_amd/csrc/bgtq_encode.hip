@@ -66,6 +66,14 @@ __device__ inline unsigned stream_byte(const uint8_t* codes, StreamSlot s, int b
     return (w >> s.skip) & 0xFFu;
 }
 
+// Row n of the [B][S] input is (batch b, step s).  The row count fits 32 bits (the launchers
+// check), so this is one 32-bit division instead of the 64-bit software routine.
+__device__ inline void split_row(int64_t n, int S, int& b, int& s) {
+    const unsigned q = (unsigned)n / (unsigned)S;
+    b = (int)q;
+    s = (int)((unsigned)n - q * (unsigned)S);
+}
+
 // Plan tables a work-group needs, copied to LDS with one burst of independent loads:
 // every later table access is an LDS read instead of one more dependent trip to memory.
 struct StagedK {
@@ -121,16 +129,21 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
     uint16_t xr[ROWS];                 // raw rows of the tile about to be processed
+    int tp[ROWS == 2 ? 2 : 1];         // decode append: their cache positions, fetched with them
     auto fetch_rows = [&](int64_t tile) {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
             int64_t n = tile * ROWS + r;
             uint16_t v = 0;
+            int t = 0;
             if (n < N) {
-                int64_t b = n / a.S, s = n - b * a.S;
+                int b, s;
+                split_row(n, a.S, b, s);
                 v = a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + j];
+                if (ROWS == 2) t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             }
             xr[r] = v;
+            if (ROWS == 2) tp[r] = t;
         }
     };
     fetch_rows(bx);
@@ -184,6 +197,8 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
 
     for (int64_t tile = bx; tile < n_tiles; tile += tile_stride) {
     const int64_t row0 = tile * ROWS;
+    int tcur[2] = {0, 0};              // this tile's positions (the prefetch below overwrites tp)
+    if (ROWS == 2) { tcur[0] = tp[0]; tcur[1] = tp[ROWS == 2 ? 1 : 0]; }
     // ---- 1. rows to LDS, next tile's rows on their way, gather by head_perm (K) -------------
 #pragma unroll
     for (int r = 0; r < ROWS; r++) xraw[r][j] = xr[r];
@@ -364,8 +379,9 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         int64_t n = row0 + r;
         int width = IS_V ? 1 : a.norm_width;
         if (n < N && gg < width) {
-            int64_t b = n / a.S, s = n - b * a.S;
-            int64_t t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            int b, s;
+            split_row(n, a.S, b, s);
+            int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             a.norms[b * a.n_sb + h * a.n_sh + t * a.n_st + gg] = bgtq_f2h(nrm_out[r][gg]);
         }
     }
@@ -376,8 +392,9 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         for (int r = 0; r < ROWS; r++) {
             int64_t n = row0 + r;
             if (n >= N) break;
-            int64_t b = n / a.S, s = n - b * a.S;
-            int64_t t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            int b, s;
+            split_row(n, a.S, b, s);
+            int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             unsigned v = 0;
             if (mode == 1)      v = stream_byte(&cds[r][c0], slot, bw);
             else if (mode == 2) v = cds[r][c0];
@@ -398,6 +415,7 @@ template <bool IS_V>
 int launch_encode(const EncodeArgs& a, hipStream_t st) {
     int64_t N = (int64_t)a.B * a.S;
     if (N == 0 || a.n_kv == 0) return BGTQ_OK;
+    if (N > INT32_MAX) return BGTQ_EINVAL;        // the kernels index rows with 32 bits
     // Few rows (decode append): small tiles so every row gets its own work-group
     // and the step stays latency-bound; many rows (prefill): 16-row tiles so the
     // rotation matrix is amortised.
