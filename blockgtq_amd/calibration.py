@@ -5,6 +5,7 @@ activation tensors) into the ``(quantizers, batched_args, kernel_args)`` triple
 ``BlockGTQProductionCache`` takes.  Reference behaviour:
 blockgtq/calibration.py:35-181.
 """
+import numpy as np
 import torch
 
 from .quantizer import BlockGTQQuantizer, build_batched_encode_args
@@ -98,4 +99,62 @@ def bake_q_rotations(model, quantizers, n_layers, nkv, nq):
                 q_proj_bias=getattr(attn.q_proj, 'bias', None))
 
 
-__all__ = ["collect_qk_activations", "build_quantizers", "bake_q_rotations"]
+_CALIB_FORMAT = 1
+
+
+def save_calibration(path, quantizers) -> None:
+    """Write the calibration result of ``quantizers[li][hi]`` to ``path`` (``.npz``).
+
+    Everything a head's tables hold follows from its per-block bit allocation and the
+    constructor arguments (rotations and codebooks are seeded), so that is all the file
+    keeps: a few hundred bytes a head instead of the activations the reference stores
+    and recalibrates from on every run (examples/build_calib_cache.py:238-298)."""
+    n_layers, nkv = len(quantizers), len(quantizers[0])
+    q0 = quantizers[0][0]
+    alloc = np.zeros((n_layers, nkv, q0.head_dim // 2), dtype=np.int16)
+    v_seed = np.zeros((n_layers, nkv), dtype=np.int64)
+    params = np.zeros((n_layers, nkv, 6), dtype=np.float64)
+    for li in range(n_layers):
+        for hi in range(nkv):
+            q8 = quantizers[li][hi]
+            assert q8._calibrated and hasattr(q8, '_v_bits'), \
+                f"layer {li} head {hi}: calibrate() and init_v_quantizer() first"
+            assert q8.head_dim == q0.head_dim and q8.v_bits == q0.v_bits
+            alloc[li, hi] = q8.bit_allocation.cpu().numpy()
+            v_seed[li, hi] = q8._v_seed
+            params[li, hi] = (q8.avg_bits, q8.rotation_threshold, q8.min_bits, q8.max_bits,
+                              q8.rope_base, q8.n_bins)
+    np.savez(path, format=np.int64(_CALIB_FORMAT), head_dim=np.int64(q0.head_dim),
+             v_bits=np.int64(q0.v_bits), bit_allocation=alloc, v_seed=v_seed, params=params)
+
+
+def load_calibration(path, device='cuda'):
+    """``(quantizers, batched_args, kernel_args)`` as ``build_quantizers`` returns them,
+    rebuilt from a file written by ``save_calibration``; the device plans come out
+    byte-identical to those of the quantizers that were saved."""
+    with np.load(path, allow_pickle=False) as f:
+        if int(f['format']) != _CALIB_FORMAT:
+            raise ValueError(f"{path}: calibration format {int(f['format'])}, "
+                             f"this build reads {_CALIB_FORMAT}")
+        hd, v_bits = int(f['head_dim']), int(f['v_bits'])
+        alloc, v_seed, params = f['bit_allocation'], f['v_seed'], f['params']
+    n_layers, nkv = alloc.shape[:2]
+    quantizers = [[None] * nkv for _ in range(n_layers)]
+    kernel_args = [[None] * nkv for _ in range(n_layers)]
+    batched_args = [None] * n_layers
+    for li in range(n_layers):
+        for hi in range(nkv):
+            avg, thr, lo, hi_bits, base, bins = params[li, hi]
+            q8 = BlockGTQQuantizer(head_dim=hd, avg_bits=float(avg), device=device,
+                                   rotation_threshold=int(thr), min_bits=int(lo),
+                                   max_bits=int(hi_bits), rope_base=float(base), n_bins=int(bins))
+            q8.calibrate_from_allocation(torch.from_numpy(alloc[li, hi].astype(np.int64)))
+            q8.init_v_quantizer(v_bits=v_bits, seed=int(v_seed[li, hi]))
+            quantizers[li][hi] = q8
+            kernel_args[li][hi] = q8.build_kernel_args()
+        batched_args[li] = build_batched_encode_args(quantizers[li], device=device)
+    return quantizers, batched_args, kernel_args
+
+
+__all__ = ["collect_qk_activations", "build_quantizers", "bake_q_rotations",
+           "save_calibration", "load_calibration"]

@@ -314,6 +314,7 @@ class BlockGTQQuantizer:
         self._v_quantizer = PolarQuantGPU(d=self.head_dim, bit_width=v_bits, seed=seed,
                                           device=self.device)
         self._v_bits = v_bits
+        self._v_seed = seed
         self._v_rot_T = self._v_quantizer.rotation.T.contiguous()
         self._v_rot = self._v_quantizer.rotation.contiguous()
         self._v_boundaries = self._v_quantizer.boundaries.contiguous()

@@ -396,3 +396,30 @@ def test_device_paths_refuse_cpu_tensors():
     q, _ = make_quantizer(seed=1)
     with pytest.raises(_capi.BgtqError):
         q.compress(torch.zeros(4, 128, dtype=torch.float16))
+
+
+def test_saved_calibration_rebuilds_identical_plans(tmp_path):
+    from blockgtq_amd import calibration
+    quantizers = [[make_quantizer(seed=10 * li + hi, head=hi, budget=192 - 32 * li,
+                                  min_bits=li, max_bits=5 - li)[0] for hi in range(2)]
+                  for li in range(2)]
+    path = tmp_path / "calib.npz"
+    calibration.save_calibration(path, quantizers)
+    assert path.stat().st_size < 16384                 # allocations, not activations
+    loaded, batched_args, kernel_args = calibration.load_calibration(path, device='cpu')
+    assert len(loaded) == 2 and len(loaded[0]) == 2 and len(batched_args) == 2
+    for li in range(2):
+        for hi in range(2):
+            a, b = quantizers[li][hi], loaded[li][hi]
+            assert torch.equal(a.bit_allocation, b.bit_allocation)
+            assert a.plan().tobytes() == b.plan().tobytes()
+            assert kernel_args[li][hi]['segments_b'] == a.build_kernel_args()['segments_b']
+        stacked = P.stack_plans(quantizers[li])
+        assert batched_args[li]['plans'].numpy().tobytes() == stacked.tobytes()
+    # a file of another format version is refused, not misread
+    with np.load(path) as f:
+        fields = {k: f[k] for k in f.files}
+    fields['format'] = np.int64(99)
+    np.savez(tmp_path / "other.npz", **fields)
+    with pytest.raises(ValueError):
+        calibration.load_calibration(tmp_path / "other.npz", device='cpu')
