@@ -262,35 +262,40 @@ int launch_generic(const DecodeArgs& a, hipStream_t st) {
 }
 
 // ---- partition merge + V un-rotation ------------------------------------------
-// One work-group per (batch row, query head).  Thread j first takes part in
-// finding the global maximum and the weight of every partition (partitions are
-// spread over the threads, weights parked in LDS), then owns output dim j.
-// Every global load that does not depend on a computed value (the first batch of
-// partial vectors, this thread's column of the un-rotation) is issued up front,
-// so the kernel pays for about one memory round trip.
+// One work-group per (batch row, query head).  Its loads are 16 bytes a lane and
+// contiguous across the wave: thread t holds columns 4(t & 31) .. +3 of the rows
+// r = t >> 5 (mod 4) of the partial vectors and of the un-rotation, sums over its own
+// rows, and the four row classes are added through LDS (in a fixed order, so the result
+// does not depend on timing).  Every load that does not depend on a computed value
+// (the first 16 partial vectors, the whole un-rotation) is issued up front, so the
+// kernel pays for about one memory round trip of 36 wide loads a thread.
+static_assert(offsetof(bgtq_head_plan, v_rot) % 16 == 0 && sizeof(bgtq_head_plan) % 16 == 0,
+              "the un-rotation is read 16 bytes at a time");
 __global__ __launch_bounds__(D) void lse_reduce_kernel(
     const bgtq_head_plan* plans, const float* part_out, const float* part_lse, int n_splits,
     const float* extra_out, const float* extra_lse, int n_extra,
     int n_q, int gqa, int unrotate, uint16_t* out, int64_t o_sb, int64_t o_sh, float* lse_out) {
+    __shared__ __align__(16) float cls_sum[4][D];
     __shared__ float vec[D];
     __shared__ float wgt[BGTQ_MAX_SPLITS];
     __shared__ float red[4];
     const int j = threadIdx.x;
+    const int cls = j >> 5, c4 = (j & 31) * 4;
     const int hq = blockIdx.x, b = blockIdx.y;
     const size_t row = (size_t)b * n_q + hq;
     const float* pl = part_lse + row * n_splits;
     const float* el = extra_lse ? extra_lse + row * n_extra : nullptr;
     const float* R = plans[hq / gqa].v_rot;
-    const float* po = part_out + row * n_splits * D + j;
+    const float* po = part_out + row * n_splits * D + c4;
 
-    constexpr int NB = 16;                     // partial vectors fetched before anything else
-    float pv[NB];
+    constexpr int NB = 4;                      // rounds of 4 partial vectors fetched before anything else
+    float4 pv[NB];
 #pragma unroll
-    for (int i = 0; i < NB; i++) pv[i] = po[(size_t)min(i, n_splits - 1) * D];
-    float rcol[D];                             // this thread's column of the un-rotation
+    for (int i = 0; i < NB; i++) pv[i] = *(const float4*)(po + (size_t)min(4 * i + cls, n_splits - 1) * D);
+    float4 rv[D / 4];                          // rows 4i + cls of the un-rotation, this thread's four columns
     if (unrotate) {
 #pragma unroll
-        for (int k = 0; k < D; k++) rcol[k] = R[k * D + j];
+        for (int i = 0; i < D / 4; i++) rv[i] = *(const float4*)(R + (4 * i + cls) * D + c4);
     }
 
     float m = -INFINITY;
@@ -308,32 +313,19 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     // weights: exp(lse - m), 0 for empty partitions (their vectors are undefined)
     for (int c = j; c < n_splits; c += D) { float l = wgt[c]; wgt[c] = (l == -INFINITY) ? 0.f : __expf(l - m); }
     __syncthreads();
-    float den = 0.f, accp = 0.f, acce = 0.f;
+    float dcl = 0.f;                           // weight sum of this thread's row class
+    float4 a4 = {0.f, 0.f, 0.f, 0.f};
+    auto add = [&](float w, const float4& v) {
+        dcl += w;
+        if (w != 0.f) { a4.x += w * v.x; a4.y += w * v.y; a4.z += w * v.z; a4.w += w * v.w; }
+    };
 #pragma unroll
-    for (int i = 0; i < NB; i++) {
-        if (i < n_splits) {
-            const float w = wgt[i];
-            den += w;
-            if (w != 0.f) accp += w * pv[i];
-        }
-    }
-    int c = NB;
-    for (; c + 8 <= n_splits; c += 8) {
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = po[(size_t)(c + i) * D];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float w = wgt[c + i];
-            den += w;
-            if (w != 0.f) accp += w * v[i];
-        }
-    }
-    for (; c < n_splits; c++) {
-        const float w = wgt[c];
-        den += w;
-        if (w != 0.f) accp += w * po[(size_t)c * D];
-    }
+    for (int i = 0; i < NB; i++)
+        if (4 * i + cls < n_splits) add(wgt[4 * i + cls], pv[i]);
+    for (int c = 4 * NB + cls; c < n_splits; c += 4) add(wgt[c], *(const float4*)(po + (size_t)c * D));
+    *(float4*)&cls_sum[cls][c4] = a4;
+    if ((j & 31) == 0) red[cls] = dcl;         // (the maxima in red were read before the last barrier)
+    float acce = 0.f, den = 0.f;
     for (int e = 0; e < n_extra; e++) {
         float l = el[e];
         if (l == -INFINITY) continue;
@@ -341,14 +333,21 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
         den += w;
         acce += w * extra_out[(row * n_extra + e) * D + j];
     }
-    float res = accp;
+    __syncthreads();
+    den += (red[0] + red[1]) + (red[2] + red[3]);
+    float res = (cls_sum[0][j] + cls_sum[1][j]) + (cls_sum[2][j] + cls_sum[3][j]);
     if (unrotate) {
-        vec[j] = accp;
-        __syncthreads();
-        float r = 0.f;
+        vec[j] = res;
+        __syncthreads();                       // also: every read of cls_sum above is done
+        float4 r4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int k = 0; k < D; k++) r += vec[k] * rcol[k];
-        res = r;
+        for (int i = 0; i < D / 4; i++) {
+            const float x = vec[4 * i + cls];
+            r4.x += x * rv[i].x; r4.y += x * rv[i].y; r4.z += x * rv[i].z; r4.w += x * rv[i].w;
+        }
+        *(float4*)&cls_sum[cls][c4] = r4;
+        __syncthreads();
+        res = (cls_sum[0][j] + cls_sum[1][j]) + (cls_sum[2][j] + cls_sum[3][j]);
     }
     out[b * o_sb + hq * o_sh + j] = bgtq_f2h((res + acce) / den);
     if (lse_out && j == 0) lse_out[row] = m + __logf(den);
@@ -487,6 +486,9 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
     BGTQ_CHECK_ARG(plans && partial_out && partial_lse && out);
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && gqa >= 1 && n_splits >= 1 && n_extra >= 0);
     BGTQ_CHECK_ARG(n_extra == 0 || (extra_out && extra_lse));
+    // the kernel reads the partial vectors and the plan 16 bytes at a time
+    BGTQ_CHECK_ARG(((uintptr_t)partial_out & 15) == 0 && ((uintptr_t)plans & 15) == 0);
+    if (n_splits > BGTQ_MAX_SPLITS) return BGTQ_ELIMIT;
     if (B == 0 || n_kv == 0) return BGTQ_OK;
     dim3 grid((unsigned)(n_kv * gqa), (unsigned)B);
     hipLaunchKernelGGL(lse_reduce_kernel, grid, dim3(D), 0, (hipStream_t)stream,

@@ -331,6 +331,8 @@ int bgtq_decode_attn(const bgtq_head_plan* plans,
  * the per-partition `partial_out @ R` of :875-882 and the return_lse
  * logsumexp of :1856-1860.  Partitions whose lse is -inf are skipped.
  *
+ *   partial_out, plans  16-byte aligned (read 16 bytes at a time; BGTQ_EINVAL otherwise);
+ *              n_splits <= BGTQ_MAX_SPLITS (BGTQ_ELIMIT otherwise)
  *   extra_out  fp32 [B][n_q][n_extra][128] or NULL, in the ORIGINAL value space:
  *              added after the packed sum has been un-rotated (needs unrotate != 0)
  *   extra_lse  fp32 [B][n_q][n_extra] or NULL
