@@ -410,6 +410,13 @@ __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
     const int64_t N = (int64_t)a.B * a.S;
     encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y, (N + ROWS - 1) / ROWS, gridDim.x);
 }
+// The prefill-sized encoder is throughput bound: at least 4 waves per SIMD (128 registers a
+// lane), which the register allocator does not aim for by itself.
+template <bool IS_V>
+__global__ __launch_bounds__(NT, 4) void encode_kernel16(EncodeArgs a) {
+    const int64_t N = (int64_t)a.B * a.S;
+    encode_rows<16, IS_V>(a, blockIdx.x, blockIdx.y, (N + 15) / 16, gridDim.x);
+}
 
 template <bool IS_V>
 int launch_encode(const EncodeArgs& a, hipStream_t st) {
@@ -428,7 +435,7 @@ int launch_encode(const EncodeArgs& a, hipStream_t st) {
         int64_t tiles = (N + 15) / 16;
         int64_t want = (256 * 10 + a.n_kv - 1) / a.n_kv;
         dim3 grid((unsigned)(tiles < want ? tiles : want), (unsigned)a.n_kv);
-        hipLaunchKernelGGL((encode_kernel<16, IS_V>), grid, dim3(NT), 0, st, a);
+        hipLaunchKernelGGL((encode_kernel16<IS_V>), grid, dim3(NT), 0, st, a);
     }
     return bgtq_launch_status();
 }
