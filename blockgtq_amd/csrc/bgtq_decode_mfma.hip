@@ -56,10 +56,10 @@ constexpr int D = BGTQ_D;
 #define BGTQ_MT 64
 #endif
 #ifndef BGTQ_MAX_WAVES
-#define BGTQ_MAX_WAVES 8
+#define BGTQ_MAX_WAVES 12
 #endif
 #ifndef BGTQ_KB
-#define BGTQ_KB 2
+#define BGTQ_KB 1
 #endif
 constexpr int MT = BGTQ_MT;        // tokens per wave tile = MT / 16 MFMA row blocks
 constexpr int NBLK = MT / 16;
