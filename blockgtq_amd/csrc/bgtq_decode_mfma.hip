@@ -1,13 +1,16 @@
 // MFMA decode attention over bit-packed K and V records (gfx950).
 //
-// One work-group of up to 8 waves owns one partition of one (batch row, KV
-// head); every wave walks its own 64-token tiles with a private online softmax
-// and the results are merged through LDS at the end.
+// One work-group of up to 12 waves (3 per SIMD, as many as the tile buffers leave
+// room for in LDS) owns one partition of one (batch row, KV head); every wave
+// walks its own 64-token tiles with a private online softmax and the results
+// are merged through LDS at the end.
 //
 // Data movement.  A tile of packed records is one contiguous byte range of the
 // cache.  It goes from HBM straight into LDS with global_load_lds_dwordx4
-// (aligned 16-byte pieces, the 16-byte phase of the source is kept), into one of
-// two buffers per wave, one tile ahead of the tile being processed.  The raw
+// (aligned 16-byte pieces, the 16-byte phase of the source is kept), into the
+// wave's K buffer as soon as QK^T of the previous tile has read it (BGTQ_KB = 2
+// keeps two buffers and fetches a whole tile ahead: not faster, and the LDS is
+// better spent on a third wave per SIMD), V likewise after PV.  The raw
 // fp16 norms of the tile travel the same way.  Nothing on the streaming path
 // passes through vector registers.
 //
