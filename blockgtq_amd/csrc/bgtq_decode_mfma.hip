@@ -255,6 +255,25 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     uint4* steptab = (uint4*)(smem + steptab_off(kimg));
     uint8_t* qpad = smem + qpad_off(kimg);
     const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+    // ---- pair tables first: their addresses need nothing but the plan, and they are the last
+    // thing the set-up waits for.  V table of the value layout in use at LDS offset 0, K tables
+    // of the record layout in use behind it; the chunks of both are dealt round-robin to the waves.
+    {
+        const uint32_t voff0 = (uint32_t)lane * 16;
+        const uint8_t* vimg = vnib ? (const uint8_t*)P.lut_image_mixed + BGTQ_LUTM_V
+                                   : (const uint8_t*)P.lut_image + BGTQ_LUT_V;
+        const uint8_t* kimg_src = (const uint8_t*)(kmix ? P.lut_image_mixed : P.lut_image);
+        constexpr int vch = (vlut_bytes(VBW) + 1023) >> 10;
+        const int kch = (kimg + 1023) >> 10;
+        for (int cc = wave; cc < vch + kch; cc += nw) {
+            const bool isv = cc < vch;
+            const int o = (isv ? cc : cc - vch) * 1024;
+            const int left = (isv ? vlut_bytes(VBW) : kimg) - o;
+            dma16(voff0, (isv ? vimg : kimg_src) + o,
+                  __builtin_amdgcn_readfirstlane(smem_lds + (isv ? 0 : VTAB_BYTES) + o),
+                  __builtin_amdgcn_ballot_w64((int)voff0 < left));
+        }
+    }
     const uint32_t kbufs_off = waves_off(kimg);                                   // [KB][nw] K + norm buffers
     const uint32_t vbuf_off = kbufs_off + KB * nw * tl.kbuf + wave * tl.vt;        // [nw] V buffers
     const uint32_t norm_off = kbufs_off + nw * (KB * tl.kbuf + tl.vt) + wave * WAVE_NORM_BYTES;
@@ -300,11 +319,10 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     int v_loads = 0;                 // loads of the V tile issued after the current K tile
 
     // ---- init: step parameters, query units, tables --------------------------------------
-    // Everything a work-group needs comes in by DMA, in the order in which it is needed: first
-    // the small things the set-up code reads (step table, query-unit map, rotated queries) into
-    // a scratch area, then the pair tables, then the first K and V tiles.  Loads of one wave
-    // land in issue order, so the set-up can run on the small things while the table image and
-    // the first tiles are still on their way.
+    // Everything a work-group needs comes in by DMA.  The pair tables were requested at the top of
+    // the kernel; here follow the small things the set-up code reads (step table, query-unit map,
+    // rotated queries) into a scratch area and then the first K and V tiles.  Loads of one wave
+    // land in issue order, so the set-up can run while the first tiles are still on their way.
     //
     // Step table per (step, column half, lane group).  Query groups of at most 8 heads use the
     // plan's two-segment schedule (the halves differ); larger groups need all 16 columns for
@@ -319,16 +337,13 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const uint8_t* qu_src = (const uint8_t*)(kmix ? P.qunit_dim_mixed : P.qunit_dim);   // qunit_len follows qunit_dim
     const uint8_t* q_src = (const uint8_t*)(a.q + b * a.q_sb + (int64_t)h * gqa * a.q_sh);
     const bool q_dma = ((((uintptr_t)q_src) | (uintptr_t)(a.q_sh * 2)) & 15) == 0;   // rows on 16-byte boundaries
-    int n_small = 0;                                      // small loads of this wave, first in its queue
     for (int j = wave; j < 8; j += nw) {                  // 3 KB step table, 256 B unit map, 4 x 4 query rows
         if (j < 3) {
             const uint32_t i = (uint32_t)j * 64 + lane;                          // 16-byte piece of the LDS copy
             const uint32_t m = i >> 4, g = (i >> 1) & 3, part = i & 1;           // piece = (step, half, group, part)
             dma16(dense ? i * 16 : ((m * 4 + g) * 2 + part) * 16, st_src, scratch_lds + j * 1024, ~0ull);
-            n_small++;
         } else if (j == 3) {
             dma16(voff, qu_src, scratch_lds + MAX_STEPS * 8 * 32, 0xFFFFull);
-            n_small++;
         } else if (q_dma) {
             const int row = (j - 4) * 4 + (lane >> 4);
             const int src = dense ? (row & 7) : row;                             // columns 8..15 repeat heads 0..7
@@ -337,27 +352,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             if (ok) {
                 dma16((uint32_t)(src * (int)a.q_sh * 2 + (lane & 15) * 16), q_src,
                       scratch_lds + MAX_STEPS * 8 * 32 + 256 + (j - 4) * 1024, ok);
-                n_small++;
             }
-        }
-    }
-    int n_later = 0;                                      // loads issued behind the small ones
-    {
-        // V table of the value layout in use at LDS offset 0, K tables of the record layout
-        // in use behind it; the chunks of both are dealt round-robin to the waves
-        const uint8_t* vimg = vnib ? (const uint8_t*)P.lut_image_mixed + BGTQ_LUTM_V
-                                   : (const uint8_t*)P.lut_image + BGTQ_LUT_V;
-        const uint8_t* kimg_src = (const uint8_t*)(kmix ? P.lut_image_mixed : P.lut_image);
-        constexpr int vch = (vlut_bytes(VBW) + 1023) >> 10;
-        const int kch = (kimg + 1023) >> 10;
-        for (int cc = wave; cc < vch + kch; cc += nw) {
-            const bool isv = cc < vch;
-            const int o = (isv ? cc : cc - vch) * 1024;
-            const int left = (isv ? vlut_bytes(VBW) : kimg) - o;
-            dma16(voff, (isv ? vimg : kimg_src) + o,
-                  __builtin_amdgcn_readfirstlane(smem_lds + (isv ? 0 : VTAB_BYTES) + o),
-                  __builtin_amdgcn_ballot_w64((int)voff < left));
-            n_later++;
         }
     }
     // first tiles; the V tile only if its buffer does not lie under the scratch area
@@ -380,7 +375,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                                   : (kmix ? P.n_steps_mixed : P.n_steps), MAX_STEPS);
     const int n_packed = min(dense ? (kmix ? P.n_packed_steps_dense_mixed : P.n_packed_steps_dense)
                                    : (kmix ? P.n_packed_steps_mixed : P.n_packed_steps), n_steps);   // raw-byte steps come last
-    wait_loads(n_later + k0_loads + v_loads);              // this wave's small loads have landed
+    wait_loads(k0_loads + v_loads);                        // this wave's table chunks and small loads have landed
     __syncthreads();
     TRACE(2);
     for (int i = tid; i < n_steps * 8; i += nthr) {        // the row offset depends on the cache's alignment
@@ -396,7 +391,6 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         const uint32_t lo = 2 * pp < len ? row[d0] : 0, hi = 2 * pp + 1 < len ? row[d0 + 1] : 0;
         ((uint32_t*)qpad)[i] = lo | (hi << 16);
     }
-    wait_loads(k0_loads + v_loads);                         // this wave's share of the tables has landed
     __syncthreads();                                        // scratch is dead from here
     if (tile < t1 && !v_early) v_loads = issue_v(tile);
     TRACE(4);
