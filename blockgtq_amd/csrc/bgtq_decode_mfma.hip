@@ -71,6 +71,7 @@ constexpr int MAX_WAVES = BGTQ_MAX_WAVES;
 constexpr int KB = BGTQ_KB;         // K tile buffers per wave: 2 = fetched a whole tile ahead, 1 = refilled right after QK^T
 constexpr int MAX_KN = 8;          // norm columns per token row the staging area can hold
 constexpr int LDS_LIMIT = 160 * 1024;
+constexpr int MERGE_STRIDE = BGTQ_D + 4;   // floats from one row of a wave's result to the next in the merge area
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
@@ -698,27 +699,44 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     l_tot += __shfl_xor(l_tot, 32, 64);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                         // tables and tile buffers are dead from here
+    // Row stride MS = D + 4 and the column order e * 16 + li put the 64 lanes of every store on
+    // 64 different banks (rows 4 apart are 16 banks apart); dim d sits at (d & 7) * 16 + (d >> 3).
     float* mg_m = (float*)smem;              // [nw][16]
     float* mg_l = mg_m + nw * 16;            // [nw][16]
-    float* mg_o = mg_l + nw * 16;            // [nw][16][D]
+    float* mg_o = mg_l + nw * 16;            // [nw][16][MS]
     if (lane < 16) { mg_m[wave * 16 + lane] = m_ref; mg_l[wave * 16 + lane] = l_tot; }
+    if (!dense || lg < 2) {                  // rows 8..15 repeat heads 0..7 in the two-segment schedule
 #pragma unroll
-    for (int e = 0; e < 8; e++)
+        for (int e = 0; e < 8; e++)
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-            mg_o[(wave * 16 + lg * 4 + r) * D + li * 8 + e] = acc[e][r];
+            for (int r = 0; r < 4; r++)
+                mg_o[(wave * 16 + lg * 4 + r) * MERGE_STRIDE + e * 16 + li] = acc[e][r];
+    }
     __syncthreads();
     TRACE(61);
     for (int i = tid; i < gqa * D; i += nthr) {
-        int hq = i / D, d = i - hq * D;
+        const int hq = i / D, d = i - hq * D;
+        const int col = (d & 7) * 16 + (d >> 3);
+        // all reads of a batch go out before the first is used (one LDS round trip per batch)
+        float mw[MAX_WAVES], lw[MAX_WAVES], ow[MAX_WAVES];
+#pragma unroll
+        for (int w = 0; w < MAX_WAVES; w++) {
+            const int ww = min(w, nw - 1);
+            mw[w] = mg_m[ww * 16 + hq];
+            lw[w] = mg_l[ww * 16 + hq];
+            ow[w] = mg_o[(ww * 16 + hq) * MERGE_STRIDE + col];
+        }
         float m = -INFINITY;
-        for (int w = 0; w < nw; w++) m = fmaxf(m, mg_m[w * 16 + hq]);
+#pragma unroll
+        for (int w = 0; w < MAX_WAVES; w++) if (w < nw) m = fmaxf(m, mw[w]);
         float den = 0.f, num = 0.f;
-        for (int w = 0; w < nw; w++) {
-            float mw = mg_m[w * 16 + hq];
-            float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
-            den += f * mg_l[w * 16 + hq];
-            num += f * mg_o[(w * 16 + hq) * D + d];
+#pragma unroll
+        for (int w = 0; w < MAX_WAVES; w++) {
+            if (w < nw) {
+                const float f = (mw[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw[w] - m);
+                den += f * lw[w];
+                num += f * ow[w];
+            }
         }
         size_t row = ((size_t)b * a.n_kv * gqa + (size_t)h * gqa + hq) * a.n_splits + c;
         a.part_out[row * D + d] = (t1 > t0) ? num / den : 0.f;
@@ -734,7 +752,7 @@ size_t mfma_smem_bytes(int k_layout, int krow, int vrow, int kn_st, int nw) {
     const TileLayout tl = tile_layout(krow, vrow, kn_st);
     size_t need = (size_t)woff + (size_t)nw * (KB * tl.kbuf + tl.vt + WAVE_NORM_BYTES);
     size_t scratch = (size_t)woff + (size_t)nw * tl.kbuf + INIT_SCRATCH;
-    size_t merge = (size_t)nw * (32 + 16 * D) * 4;
+    size_t merge = (size_t)nw * (32 + 16 * MERGE_STRIDE) * 4;
     size_t s = need > scratch ? need : scratch;
     return s > merge ? s : merge;
 }
