@@ -71,7 +71,7 @@ constexpr int MAX_WAVES = BGTQ_MAX_WAVES;
 constexpr int KB = BGTQ_KB;         // K tile buffers per wave: 2 = fetched a whole tile ahead, 1 = refilled right after QK^T
 constexpr int MAX_KN = 8;          // norm columns per token row the staging area can hold
 constexpr int LDS_LIMIT = 160 * 1024;
-constexpr int MERGE_STRIDE = BGTQ_D + 4;   // floats from one row of a wave's result to the next in the merge area
+constexpr int MERGE_STRIDE = BGTQ_D + 8;   // most floats from one row of a wave's result to the next in the merge area
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
@@ -228,7 +228,9 @@ __device__ unsigned long long* g_trace;
 
 // VBW: bits per V code; VST: bytes from one V record to the next (the record itself is
 // 16 * VBW bytes; a padded stride keeps the rows of a tile on different LDS banks)
-template <int VBW, int VST>
+// DENSE: at most 8 query heads per KV head (the two-segment step schedule, and a PV product
+// that uses the eight spare head rows of the MFMA instead of transposing V)
+template <int VBW, int VST, bool DENSE>
 __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -328,7 +330,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     // Step table per (step, column half, lane group).  Query groups of at most 8 heads use the
     // plan's two-segment schedule (the halves differ); larger groups need all 16 columns for
     // heads and run the one-segment schedule with both halves alike.
-    const bool dense = gqa <= 8;
+    constexpr bool dense = DENSE;
     uint32_t* st_raw = (uint32_t*)scratch;                // step table as stored in the plan
     int* qu_s = (int*)(scratch + MAX_STEPS * 8 * 32);     // qunit_dim[32], qunit_len[32]
     uint16_t* q_s = (uint16_t*)(scratch + MAX_STEPS * 8 * 32 + 256);   // [16][128] rotated queries
@@ -416,9 +418,10 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 
     float m_ref = -INFINITY;        // reference of head li, in exp2 units; never below a score seen
     float l_part = 0.f;             // this lane's share of the softmax denominator
-    float4v acc[8];
+    constexpr int NACC = DENSE ? 4 : 8;         // output accumulators (16 x 16 each)
+    float4v acc[NACC];
 #pragma unroll
-    for (int e = 0; e < 8; e++) acc[e] = (float4v){0, 0, 0, 0};
+    for (int e = 0; e < NACC; e++) acc[e] = (float4v){0, 0, 0, 0};
 
     int which = 0;
     for (; tile < t1; tile += step_tiles, which ^= 1) {
@@ -603,7 +606,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 #pragma unroll
             for (int r = 0; r < 4; r++) al[r] = __shfl(alpha, lg * 4 + r, 64);
 #pragma unroll
-            for (int e = 0; e < 8; e++)
+            for (int e = 0; e < NACC; e++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[e][r] *= al[r];
             l_part *= alpha;
@@ -613,75 +616,134 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         wait_loads(k_loads);                                 // the V records of this tile are in LDS
         __builtin_amdgcn_wave_barrier();
 
-        // values: lane (j = li, group lg) decodes unit j of its 8 tokens per half tile.  Raw
-        // codes are fetched one half ahead; the exponentials run while the table reads fly.
-        uint32_t vlo[8], vhi[8];
+        if constexpr (DENSE) {
+            // values, at most 8 heads.  The product runs over (token, dim parity) pairs: A row
+            // (head h, parity e') holds P[h][t] in slot (t, e') and zero in slot (t, 1 - e'), B
+            // column c of accumulator jb holds the table word of token t = dims (8c + 2jb, + 1) in
+            // slots (t, 0), (t, 1).  D[(h, e')][c] is then out[h][8c + 2jb + e'], a table word
+            // is an MFMA operand as it comes, and the 8 head rows that would repeat rows 0..7
+            // carry the odd dims instead.  Lane (c = li, lg) decodes unit c of tokens 4lg .. 4lg+3
+            // of every 16-token block; raw codes are fetched one block ahead.
+            const uint32_t pmask = (li & 8) ? 0xFFFF0000u : 0x0000FFFFu;
+            uint32_t vlo[4], vhi[4];
 #pragma unroll
-        for (int r = 0; r < 8; r++) {
-            const int tk = (r >> 2) * 16 + (r & 3);                       // + 4lg, folded into vbase
-            vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
-            vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
-        }
+            for (int i = 0; i < 4; i++) {
+                vlo[i] = lds_at<uint32_t>(vbase + (uint32_t)i * vrow);
+                vhi[i] = lds_at<uint32_t>(vbase + (uint32_t)i * vrow + 4);
+            }
 #pragma unroll
-        for (int half = 0; half < NBLK / 2; half++) {
-            const float4v vn_lo = lds_at<float4v>(vnf + (half * 32 + lg * 4) * 4);        // tokens 4lg .. 4lg+3
-            const float4v vn_hi = lds_at<float4v>(vnf + (half * 32 + 16 + lg * 4) * 4);   // tokens 16+4lg ..
-            uint32_t W[8][4];
+            for (int k = 0; k < NBLK; k++) {
+                const float4v vn4 = lds_at<float4v>(vnf + (k * 16 + lg * 4) * 4);
+                uint4v W[4];                                  // [pair of the unit][token]
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t raw = __builtin_amdgcn_alignbyte(vhi[i], vlo[i], v_sh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
+                        const int fp = e * 2 * VBW;
+                        const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
+                        W[e][i] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (k + 1 < NBLK) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int tk = (k + 1) * 16 + i;
+                        vlo[i] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
+                        vhi[i] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
+                    }
+                }
+                // P * v_norm is formed in fp32, rounded to fp16 once and kept in the half of
+                // the word that belongs to this lane's parity
+                uint4v Pa;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float pe = __builtin_amdgcn_exp2f(fmaf(S[k][i], c2, -m_ref));
+                    l_part += pe;
+                    const float x = pe * vn4[i];
+                    const float2v xx = {x, x};
+                    Pa[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(xx, half2v)) & pmask;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int jb = 0; jb < 4; jb++)
+                    acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, Pa),
+                                                                     __builtin_bit_cast(half8, W[jb]), acc[jb], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            // values: lane (j = li, group lg) decodes unit j of its 8 tokens per half tile.  Raw
+            // codes are fetched one half ahead; the exponentials run while the table reads fly.
+            uint32_t vlo[8], vhi[8];
 #pragma unroll
             for (int r = 0; r < 8; r++) {
-                const uint32_t raw = __builtin_amdgcn_alignbyte(vhi[r], vlo[r], v_sh);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    // shift the pair field to its place in the table address, then one and-or
-                    // merges the bank replica (the compiler would spend an and plus an add)
-                    constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
-                    const int fp = e * 2 * VBW;
-                    const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
-#ifdef BGTQ_EXPERIMENT_NOVLUT
-                    W[r][e] = and_or(sh, fmask, vbank);
-#else
-                    W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
-#endif
-                }
+                const int tk = (r >> 2) * 16 + (r & 3);                       // + 4lg, folded into vbase
+                vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
+                vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            if (half + 1 < NBLK / 2) {
+#pragma unroll
+            for (int half = 0; half < NBLK / 2; half++) {
+                const float4v vn_lo = lds_at<float4v>(vnf + (half * 32 + lg * 4) * 4);        // tokens 4lg .. 4lg+3
+                const float4v vn_hi = lds_at<float4v>(vnf + (half * 32 + 16 + lg * 4) * 4);   // tokens 16+4lg ..
+                uint32_t W[8][4];
 #pragma unroll
                 for (int r = 0; r < 8; r++) {
-                    const int tk = (half + 1) * 32 + (r >> 2) * 16 + (r & 3);
-                    vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
-                    vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
+                    const uint32_t raw = __builtin_amdgcn_alignbyte(vhi[r], vlo[r], v_sh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        // shift the pair field to its place in the table address, then one and-or
+                        // merges the bank replica (the compiler would spend an and plus an add)
+                        constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
+                        const int fp = e * 2 * VBW;
+                        const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
+#ifdef BGTQ_EXPERIMENT_NOVLUT
+                        W[r][e] = and_or(sh, fmask, vbank);
+#else
+                        W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
+#endif
+                    }
                 }
-            }
-            // P * v_norm is formed in fp32 and rounded to fp16 once
-            half8 Pm;
+                __builtin_amdgcn_sched_barrier(0);
+                if (half + 1 < NBLK / 2) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int k = half * 2 + (e >> 1), r = (e & 1) * 2;
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(S[k][r], c2, -m_ref));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(S[k][r + 1], c2, -m_ref));
-                l_part += p0 + p1;
-                const float4v vn4 = (e >> 1) ? vn_hi : vn_lo;
-                const float2v pv = {p0 * vn4[r], p1 * vn4[r + 1]};
-                const half2v ph = __builtin_convertvector(pv, half2v);
-                Pm[2 * e] = ph[0];
-                Pm[2 * e + 1] = ph[1];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                half8 Bv;
-                const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;   // high or low halves
-#pragma unroll
-                for (int p = 0; p < 4; p++) {
-                    uint32_t x = __builtin_amdgcn_perm(W[2 * p + 1][e >> 1], W[2 * p][e >> 1], sel);
-                    half2v hv = __builtin_bit_cast(half2v, x);
-                    Bv[2 * p] = hv[0];
-                    Bv[2 * p + 1] = hv[1];
+                    for (int r = 0; r < 8; r++) {
+                        const int tk = (half + 1) * 32 + (r >> 2) * 16 + (r & 3);
+                        vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
+                        vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
+                    }
                 }
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Pm, Bv, acc[e], 0, 0, 0);
+                // P * v_norm is formed in fp32 and rounded to fp16 once
+                half8 Pm;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int k = half * 2 + (e >> 1), r = (e & 1) * 2;
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(S[k][r], c2, -m_ref));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(S[k][r + 1], c2, -m_ref));
+                    l_part += p0 + p1;
+                    const float4v vn4 = (e >> 1) ? vn_hi : vn_lo;
+                    const float2v pv = {p0 * vn4[r], p1 * vn4[r + 1]};
+                    const half2v ph = __builtin_convertvector(pv, half2v);
+                    Pm[2 * e] = ph[0];
+                    Pm[2 * e + 1] = ph[1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    half8 Bv;
+                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;   // high or low halves
+#pragma unroll
+                    for (int p = 0; p < 4; p++) {
+                        uint32_t x = __builtin_amdgcn_perm(W[2 * p + 1][e >> 1], W[2 * p][e >> 1], sel);
+                        half2v hv = __builtin_bit_cast(half2v, x);
+                        Bv[2 * p] = hv[0];
+                        Bv[2 * p + 1] = hv[1];
+                    }
+                    acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Pm, Bv, acc[e], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();     // V buffer and norm areas are rewritten from here on
@@ -699,18 +761,25 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     l_tot += __shfl_xor(l_tot, 32, 64);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                         // tables and tile buffers are dead from here
-    // Row stride MS = D + 4 and the column order e * 16 + li put the 64 lanes of every store on
-    // 64 different banks (rows 4 apart are 16 banks apart); dim d sits at (d & 7) * 16 + (d >> 3).
+    // Dim d of a row sits at (d & 7) * 16 + (d >> 3); with that column order and a row stride of
+    // MS floats the 64 lanes of every store below fall on 64 different banks.
+    constexpr int MS = DENSE ? MERGE_STRIDE : MERGE_STRIDE - 4;
     float* mg_m = (float*)smem;              // [nw][16]
     float* mg_l = mg_m + nw * 16;            // [nw][16]
     float* mg_o = mg_l + nw * 16;            // [nw][16][MS]
     if (lane < 16) { mg_m[wave * 16 + lane] = m_ref; mg_l[wave * 16 + lane] = l_tot; }
-    if (!dense || lg < 2) {                  // rows 8..15 repeat heads 0..7 in the two-segment schedule
+    if constexpr (DENSE) {                   // acc[jb][r] = out[head 4(lg & 1) + r][dim 8li + 2jb + (lg >> 1)]
+#pragma unroll
+        for (int jb = 0; jb < 4; jb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                mg_o[(wave * 16 + (lg & 1) * 4 + r) * MS + (2 * jb + (lg >> 1)) * 16 + li] = acc[jb][r];
+    } else {                                 // acc[e][r] = out[head 4lg + r][dim 8li + e]
 #pragma unroll
         for (int e = 0; e < 8; e++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                mg_o[(wave * 16 + lg * 4 + r) * MERGE_STRIDE + e * 16 + li] = acc[e][r];
+                mg_o[(wave * 16 + lg * 4 + r) * MS + e * 16 + li] = acc[e][r];
     }
     __syncthreads();
     TRACE(61);
@@ -724,7 +793,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             const int ww = min(w, nw - 1);
             mw[w] = mg_m[ww * 16 + hq];
             lw[w] = mg_l[ww * 16 + hq];
-            ow[w] = mg_o[(ww * 16 + hq) * MERGE_STRIDE + col];
+            ow[w] = mg_o[(ww * 16 + hq) * MS + col];
         }
         float m = -INFINITY;
 #pragma unroll
@@ -757,8 +826,8 @@ size_t mfma_smem_bytes(int k_layout, int krow, int vrow, int kn_st, int nw) {
     return s > merge ? s : merge;
 }
 
-template <int VBW, int VST>
-int launch(const DecodeArgs& a, hipStream_t st) {
+template <int VBW, int VST, bool DENSE>
+int launch_kernel(const DecodeArgs& a, hipStream_t st) {
     // no more waves than the longest partition has tiles
     const int part = (a.T + a.n_splits - 1) / a.n_splits;
     int nw = (part + MT - 1) / MT;
@@ -766,7 +835,7 @@ int launch(const DecodeArgs& a, hipStream_t st) {
     while (nw > 1 && mfma_smem_bytes(a.k_layout, a.k_row_width, VST, (int)a.kn_st, nw) > (size_t)LDS_LIMIT) nw--;
     const size_t smem = mfma_smem_bytes(a.k_layout, a.k_row_width, VST, (int)a.kn_st, nw);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
-    auto kern = decode_mfma_kernel<VBW, VST>;
+    auto kern = decode_mfma_kernel<VBW, VST, DENSE>;
     static int ready = 0;                    // 1: usable, -1: not usable
     if (ready == 0) {
         // the kernel addresses its V table as "LDS offset 0": that holds only while it has
@@ -782,6 +851,11 @@ int launch(const DecodeArgs& a, hipStream_t st) {
     dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)a.B);
     hipLaunchKernelGGL(kern, grid, dim3(nw * 64), smem, st, a);
     return bgtq_launch_status();
+}
+
+template <int VBW, int VST>
+int launch(const DecodeArgs& a, hipStream_t st) {
+    return a.gqa <= 8 ? launch_kernel<VBW, VST, true>(a, st) : launch_kernel<VBW, VST, false>(a, st);
 }
 
 }  // namespace
