@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per attention launch from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy
 # kernel of known size (profiles/decode_mfma_kernel_<workload>_hbm_traffic.txt); valid for the
 # workload's own context, batch and default partition count only.
-MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 66.06e6}
+MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 66.12e6}
 
 
 def parse():
