@@ -340,7 +340,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const uint8_t* qu_src = (const uint8_t*)(kmix ? P.qunit_dim_mixed : P.qunit_dim);   // qunit_len follows qunit_dim
     const uint8_t* q_src = (const uint8_t*)(a.q + b * a.q_sb + (int64_t)h * gqa * a.q_sh);
     const bool q_dma = ((((uintptr_t)q_src) | (uintptr_t)(a.q_sh * 2)) & 15) == 0;   // rows on 16-byte boundaries
-    for (int j = wave; j < 8; j += nw) {                  // 3 KB step table, 256 B unit map, 4 x 4 query rows
+    for (int j = nw - 1 - wave; j < 8; j += nw) {         // 3 KB step table, 256 B unit map, 4 x 4 query rows (dealt from the last wave down: the first waves carry one table chunk more)
         if (j < 3) {
             const uint32_t i = (uint32_t)j * 64 + lane;                          // 16-byte piece of the LDS copy
             const uint32_t m = i >> 4, g = (i >> 1) & 3, part = i & 1;           // piece = (step, half, group, part)
