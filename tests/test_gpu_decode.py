@@ -523,3 +523,27 @@ def test_prompt_attention_rows_equal_decode_steps():
                                    cache.v_norms[0], s + 1, k_layout=cache._k_layout, v_layout=cache._v_layout,
                                    k_row_width=cache.k_bytes_per_tok, v_row_width=cache.vpb)
         assert (full[:, :, s].float() - dec.float()).abs().max() < TOL
+
+
+def test_merge_entry_point_refuses_what_its_kernel_cannot_take():
+    """Misaligned partial vectors and more partitions than the kernel's table holds come back
+    as error codes from the C-ABI, before anything is launched."""
+    from blockgtq_amd import _capi
+    L = _capi.lib()
+    q, _ = make_quantizer(seed=3, device=DEV)
+    plans = q.device_plan()
+    part = torch.zeros(4 * 128 + 4, dtype=torch.float32, device=DEV)
+    lse = torch.zeros(4, dtype=torch.float32, device=DEV)
+    out = torch.zeros(1, 1, 128, dtype=torch.float16, device=DEV)
+    st = _capi.stream_ptr(torch.device(DEV))
+
+    def call(part_ptr, n_splits):
+        return L.bgtq_lse_reduce(_capi.ptr(plans), part_ptr, _capi.ptr(lse), n_splits, None, None, 0,
+                                 1, 1, 1, 1, _capi.ptr(out), out.stride(0), out.stride(1), None, st)
+
+    assert call(_capi.ptr(part), 4) == 0
+    assert call(_capi.ptr(part[1:]), 4) != 0                   # 4 bytes off a 16-byte boundary
+    assert call(_capi.ptr(part), 513) != 0                     # BGTQ_MAX_SPLITS is 512
+    torch.cuda.synchronize()
+    with pytest.raises(_capi.BgtqError):
+        _capi.check(call(_capi.ptr(part[1:]), 4), "bgtq_lse_reduce")
