@@ -82,6 +82,9 @@ CASES = [  # budget mn mx vb n_kv gqa B T k_layout v_layout
     (300, 2, 8, 4, 1, 16, 1, 300, 1, 0),
     (64, 1, 1, 1, 1, 1, 3, 64, 0, 1),
     (192, 3, 3, 3, 3, 2, 1, 513, 0, 0),
+    (192, 1, 5, 3, 2, 7, 1, 400, 0, 0),       # odd head groups on either side of the 8-head schedule
+    (192, 1, 5, 3, 1, 12, 2, 333, 0, 0),
+    (160, 1, 6, 4, 2, 3, 2, 200, 1, 1),
 ]
 
 
