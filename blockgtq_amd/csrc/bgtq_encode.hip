@@ -22,6 +22,13 @@ namespace {
 constexpr int D = BGTQ_D;
 constexpr int NT = 128;  // threads per work-group
 
+#ifdef BGTQ_TRACE
+__device__ unsigned long long* g_etrace;
+#define ET(slot) do { if (threadIdx.x == 0 && g_etrace) g_etrace[(size_t)blockIdx.x * 16 + (slot)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define ET(slot) do {} while (0)
+#endif
+
 struct EncodeArgs {
     const bgtq_head_plan* plans;
     const uint16_t* x;          // fp16 [B][n_kv][S][128]
@@ -65,6 +72,18 @@ __device__ inline unsigned stream_byte(const uint8_t* codes, StreamSlot s, int b
     for (int i = 0; i < s.n; i++) w |= (unsigned)codes[s.first + i] << (i * bw);
     return (w >> s.skip) & 0xFFu;
 }
+// The same byte with all (at most 8) code reads issued at once: for the latency-bound append of
+// a few rows, where one LDS round trip per code is what the loop above would cost.
+__device__ inline unsigned stream_byte_batched(const uint8_t* codes, StreamSlot s, int bw) {
+    unsigned c[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) c[i] = codes[s.first + min(i, s.n - 1)];
+    unsigned w = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        if (i < s.n) w |= c[i] << (i * bw);
+    return (w >> s.skip) & 0xFFu;
+}
 
 // Row n of the [B][S] input is (batch b, step s).  The row count fits 32 bits (the launchers
 // check), so this is one 32-bit division instead of the 64-bit software routine.
@@ -93,9 +112,43 @@ struct StagedV {
 constexpr int H_NSEG = 0, H_NZERO = 1, H_NOPACK_START = 4, H_NOPACK_LEN = 5, H_VBITS = 6;
 constexpr int H_BW = 8, H_START = 16, H_LEN = 24, H_PACK_OFF = 32, H_IDENT = 48;
 
+// The 128 x 128 fp32 rotation as 4096 pieces of 16 bytes: thread j fetches pieces j, j + 128, ...
+// (a wave reads 1 KB of consecutive addresses per instruction) and later parks them at the same
+// offsets in LDS, where thread j reads column j (consecutive lanes, consecutive banks).
+static_assert(offsetof(bgtq_head_plan, k_rot_T) % 16 == 0 && offsetof(bgtq_head_plan, v_rot_T) % 16 == 0 &&
+              sizeof(bgtq_head_plan) % 16 == 0, "rotations are read 16 bytes at a time");
+typedef float rot_piece __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void fetch_rotation(const float* M, const int j, rot_piece (&st)[D / 4]) {
+#pragma unroll
+    for (int i = 0; i < D / 4; i++) st[i] = ((const rot_piece*)M)[i * NT + j];
+}
+__device__ __forceinline__ void park_rotation(float* rot_s, const int j, const rot_piece (&st)[D / 4]) {
+#pragma unroll
+    for (int i = 0; i < D / 4; i++) ((rot_piece*)rot_s)[i * NT + j] = st[i];
+}
+
+// sum of x[k]^2 over [s, e) in LDS as ONE fmaf chain in increasing k.  The reads of a batch are all
+// issued before its first fmaf (left to itself the compiler waits for every few reads in turn, and
+// the chain then costs an LDS round trip per step instead of per batch).
+__device__ __forceinline__ float chain_sumsq(const float* x, const int s, const int e) {
+    constexpr int CB = 32;
+    float ss = 0.f;
+    for (int k0 = s; k0 < e; k0 += CB) {
+        float v[CB];
+#pragma unroll
+        for (int i = 0; i < CB; i++) v[i] = x[min(k0 + i, e - 1)];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < CB; i++)
+            if (k0 + i < e) ss = __builtin_fmaf(v[i], v[i], ss);
+    }
+    return ss;
+}
+
 template <int ROWS, bool IS_V>
 __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, const int h,
-                                            const int64_t n_tiles, const int tile_stride) {
+                                            const int64_t n_tiles, const int tile_stride,
+                                            float* rot_s) {
     __shared__ __align__(16) float xs[ROWS][D];
     __shared__ float nrm[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ float nrm_out[ROWS][BGTQ_MAX_SEGMENTS];
@@ -104,6 +157,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     __shared__ typename std::conditional<IS_V, StagedV, StagedK>::type sp;
 
     const int j = threadIdx.x;
+    ET(0);
     const bgtq_head_plan& P = a.plans[h];
     const int64_t N = (int64_t)a.B * a.S;
     const float* RT = IS_V ? P.v_rot_T : P.k_rot_T;
@@ -147,18 +201,25 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     };
     fetch_rows(bx);
-    // Decode append (2-row tiles) is latency bound: this thread's column of the rotation is
-    // requested before anything else is known, V's whole dense column right away, the first 32
-    // entries of K's group range once the plan is in LDS.  16-row tiles fetch per tile instead
-    // (unrolled prefetched entries would run masked for every row of every tile).
-    constexpr int PF = ROWS == 2 ? (IS_V ? D : 32) : 0;
+    // Decode append (2-row tiles) is latency bound.  K: the whole rotation matrix is requested now,
+    // before anything else is known (which rows a thread needs is only known once the plan is in
+    // LDS), 16 bytes a lane and contiguous across the wave (32 loads a thread), and parked in LDS
+    // (rot_s) ahead of the rotation, which then reads its column from there.  16-row tiles fetch
+    // their column slices per tile instead.
+    // V's rotation is dense and is needed later than its rows: its column comes straight into
+    // registers, one 4-byte load per matrix row (the wide loads of the whole matrix land later).
+    constexpr bool STAGED = ROWS == 2 && !IS_V;
+    constexpr int PF = (ROWS == 2 && IS_V) ? D : 0;
+    rot_piece rst[STAGED ? D / 4 : 1];
     float rpre[PF > 0 ? PF : 1];
-    if constexpr (IS_V && PF > 0) {
+    if constexpr (STAGED) fetch_rotation(RT, j, rst);
+    if constexpr (PF > 0) {
 #pragma unroll
         for (int i = 0; i < PF; i++) rpre[i] = RT[i * D + j];
     }
     __syncthreads();
 
+    ET(1);
     // ---- per-thread static data -------------------------------------------
     int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
     if constexpr (!IS_V) {
@@ -167,10 +228,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         src_dim = sp.head_perm[j];
         if (g >= 0) { gs = sp.hdr[H_START + g]; ge = gs + sp.hdr[H_LEN + g]; ident = sp.hdr[H_IDENT + g]; }
         else        { gs = 0; ge = 0; }
-        if (PF > 0 && !(ident || g < 0)) {
-#pragma unroll
-            for (int i = 0; i < PF; i++) rpre[i] = RT[min(gs + i, ge - 1) * D + j];
-        }
     }
 
     // ---- pack geometry of output byte j (row independent) ------------------------
@@ -185,11 +242,20 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         if (j < nib)                             { mode = 1; bw = 4; c0 = z; clen = nps - z; idx = j; }
         else if (j < nib + sp.hdr[H_NOPACK_LEN]) { mode = 2; c0 = nps + (j - nib); }
     } else {
-        for (int s = 0; s < n_seg; s++) {
-            int off = sp.hdr[H_PACK_OFF + s], sb = sp.hdr[H_BW + s], sl = sp.hdr[H_LEN + s];
-            if (j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
-                if (sb >= 5) { mode = 2; c0 = sp.hdr[H_START + s] + (j - off); }
-                else         { mode = 1; bw = sb; c0 = sp.hdr[H_START + s]; clen = sl; idx = j - off; }
+        // all table reads of the walk go out together (read one segment at a time, every
+        // iteration waits for its own LDS round trip)
+        int offs[BGTQ_MAX_SEGMENTS], sbs[BGTQ_MAX_SEGMENTS], sls[BGTQ_MAX_SEGMENTS], sts[BGTQ_MAX_SEGMENTS];
+#pragma unroll
+        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) {
+            offs[s] = sp.hdr[H_PACK_OFF + s]; sbs[s] = sp.hdr[H_BW + s];
+            sls[s] = sp.hdr[H_LEN + s];       sts[s] = sp.hdr[H_START + s];
+        }
+#pragma unroll
+        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) {
+            const int off = offs[s], sb = sbs[s], sl = sls[s];
+            if (s < n_seg && j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
+                if (sb >= 5) { mode = 2; c0 = sts[s] + (j - off); }
+                else         { mode = 1; bw = sb; c0 = sts[s]; clen = sl; idx = j - off; }
             }
         }
     }
@@ -208,6 +274,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xraw[r][src_dim]);
     __syncthreads();
 
+    ET(2);
     // ---- 2. group norms: thread (r, grp) runs one sequential chain ---------
     if (j < ROWS * BGTQ_MAX_SEGMENTS) {
         int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
@@ -216,14 +283,19 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             int s = 0, e = D;
             if constexpr (!IS_V) { s = sp.hdr[H_START + gg]; e = s + sp.hdr[H_LEN + gg]; }
             float ss = 0.f;
+            if constexpr (IS_V) {
+                ss = chain_sumsq(xs[r], s, e);
+            } else {                           // short ranges: the batches would mostly run masked
 #pragma unroll 8
-            for (int k = s; k < e; k++) ss = __builtin_fmaf(xs[r][k], xs[r][k], ss);
+                for (int k = s; k < e; k++) ss = __builtin_fmaf(xs[r][k], xs[r][k], ss);
+            }
             n = __builtin_sqrtf(ss + 1e-30f);
         }
         nrm[r][gg] = n;
     }
     __syncthreads();
 
+    ET(3);
     // ---- 3. normalise -------------------------------------------------------
     float xh[ROWS];
 #pragma unroll
@@ -237,8 +309,10 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         xh[r] = v;
         xs[r][j] = v;     // only this thread ever touched xs[r][j] since the barrier
     }
+    if constexpr (STAGED) park_rotation(rot_s, j, rst);   // (every tile of the walk: the registers stay as they are)
     __syncthreads();
 
+    ET(4);
     // ---- 4. rotate ------------------------------------------------------------
     // Same chain as written in the contract above; the matrix column is fetched in
     // batches of RB independent loads so the chain never waits on one load at a time.
@@ -249,15 +323,61 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     } else {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) y[r] = 0.f;
+        if constexpr (STAGED) {
+            // column j of the parked rotation against the rows, the LDS reads a batch ahead of
+            // the chain that consumes them
+            {
+                constexpr int CB = 16;
+                for (int k0 = gs; k0 < ge; k0 += CB) {
+                    float rk[CB], xv[ROWS][CB];
 #pragma unroll
-        for (int i = 0; i < PF; i++) {          // entries fetched at the top of the kernel
-            if (gs + i < ge) {
+                    for (int i = 0; i < CB; i++) {
+                        const int k = min(k0 + i, ge - 1);
+                        rk[i] = rot_s[k * D + j];
 #pragma unroll
-                for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xs[r][gs + i], rpre[i], y[r]);
+                        for (int r = 0; r < ROWS; r++) xv[r][i] = xs[r][k];
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int i = 0; i < CB; i++)
+                        if (k0 + i < ge) {
+#pragma unroll
+                            for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xv[r][i], rk[i], y[r]);
+                        }
+                }
+            }
+        }
+        if constexpr (PF > 0) {                 // V: the column fetched at the top of the kernel
+            // row values come from LDS a batch of 32 dims ahead of the chain that consumes them
+            constexpr int CB = 32;
+            float4 xv[2][ROWS][CB / 4];
+            auto load = [&](const int b) {
+#pragma unroll
+                for (int r = 0; r < ROWS; r++)
+#pragma unroll
+                    for (int i = 0; i < CB / 4; i++) xv[b & 1][r][i] = *(const float4*)&xs[r][b * CB + 4 * i];
+            };
+            load(0);
+#pragma unroll
+            for (int b = 0; b < PF / CB; b++) {
+                if (b + 1 < PF / CB) load(b + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < CB / 4; i++)
+#pragma unroll
+                    for (int r = 0; r < ROWS; r++) {
+                        const float4 x4 = xv[b & 1][r][i];
+                        const int k = b * CB + 4 * i;
+                        y[r] = __builtin_fmaf(x4.x, rpre[k], y[r]);
+                        y[r] = __builtin_fmaf(x4.y, rpre[k + 1], y[r]);
+                        y[r] = __builtin_fmaf(x4.z, rpre[k + 2], y[r]);
+                        y[r] = __builtin_fmaf(x4.w, rpre[k + 3], y[r]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         constexpr int RB = IS_V ? 32 : 16;
-        for (int k0 = gs + PF; k0 < ge; k0 += RB) {
+        for (int k0 = (STAGED || PF > 0) ? ge : gs; k0 < ge; k0 += RB) {
             float rt[RB];
 #pragma unroll
             for (int i = 0; i < RB; i++) rt[i] = RT[min(k0 + i, ge - 1) * D + j];
@@ -287,6 +407,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
 
+    ET(5);
     // ---- 5. scalar quantise ---------------------------------------------------
     const bool need_cent = IS_V || a.layout == BGTQ_K_MIXED || a.corrected;
 #pragma unroll
@@ -294,8 +415,13 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         int code = 0;
         if (IS_V) {
             if constexpr (IS_V) {
-                int nb = (1 << sp.v_bits) - 1;
-                for (int b = 0; b < nb; b++) code += (y[r] > sp.boundaries[b]) ? 1 : 0;
+                // (all 15 slots are read at once; those past the codebook's last boundary are skipped)
+                const int nb = (1 << sp.v_bits) - 1;
+                float bd[15];
+#pragma unroll
+                for (int b = 0; b < 15; b++) bd[b] = sp.boundaries[b];
+#pragma unroll
+                for (int b = 0; b < 15; b++) code += (b < nb && y[r] > bd[b]) ? 1 : 0;
             }
         } else if (g >= 0) {
             if constexpr (!IS_V) {
@@ -324,6 +450,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
     __syncthreads();
 
+    ET(6);
     // ---- 6. norms to store (raw or divided by ||centroids[codes]||) ---------
     if (j < ROWS * BGTQ_MAX_SEGMENTS) {
         int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
@@ -331,12 +458,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         if (gg < n_seg) {
             float n = nrm[r][gg];
             if (IS_V) {
-                float cs = 0.f;
-#pragma unroll 8
-                for (int k = 0; k < D; k++) {
-                    float c = xs[r][k];
-                    cs = __builtin_fmaf(c, c, cs);
-                }
+                const float cs = chain_sumsq(xs[r], 0, D);
                 float cn = __builtin_sqrtf(cs + 1e-20f);
                 out = n / (cn > 1e-10f ? cn : 1.0f);
             } else if (a.layout == BGTQ_K_MIXED || a.corrected) {
@@ -356,6 +478,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
     __syncthreads();
 
+    ET(7);
     // ---- 7a. unpacked outputs (codes path) ------------------------------------
     if (a.codes_out) {
 #pragma unroll
@@ -396,26 +519,28 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             split_row(n, a.S, b, s);
             int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             unsigned v = 0;
-            if (mode == 1)      v = stream_byte(&cds[r][c0], slot, bw);
+            if (mode == 1)      v = ROWS == 2 ? stream_byte_batched(&cds[r][c0], slot, bw) : stream_byte(&cds[r][c0], slot, bw);
             else if (mode == 2) v = cds[r][c0];
             a.packed[b * a.p_sb + h * a.p_sh + t * a.p_st + j] = (uint8_t)v;
         }
     }
     __syncthreads();            // the tile buffers are rewritten by the next tile
+    ET(8);
     }
 }
 
 template <int ROWS, bool IS_V>
 __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
     const int64_t N = (int64_t)a.B * a.S;
-    encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y, (N + ROWS - 1) / ROWS, gridDim.x);
+    __shared__ __align__(16) float rot_s[(ROWS == 2 && !IS_V) ? D * D : 4];
+    encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y, (N + ROWS - 1) / ROWS, gridDim.x, rot_s);
 }
 // The prefill-sized encoder is throughput bound: at least 4 waves per SIMD (128 registers a
 // lane), which the register allocator does not aim for by itself.
 template <bool IS_V>
 __global__ __launch_bounds__(NT, 4) void encode_kernel16(EncodeArgs a) {
     const int64_t N = (int64_t)a.B * a.S;
-    encode_rows<16, IS_V>(a, blockIdx.x, blockIdx.y, (N + 15) / 16, gridDim.x);
+    encode_rows<16, IS_V>(a, blockIdx.x, blockIdx.y, (N + 15) / 16, gridDim.x, nullptr);
 }
 
 template <bool IS_V>
@@ -448,15 +573,16 @@ struct RotQArgs {
     int n_rows, n_q, gqa;
 };
 
-__device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t row, const int hq) {
+__device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t row, const int hq,
+                                             float* rot_s) {
     __shared__ float xs[D];
     const int j = threadIdx.x;
+    ET(0);
     const bgtq_head_plan& P = a.plans[hq / a.gqa];
-    // One round of independent loads: the thread's whole column of the rotation, its source
-    // dim and its group; the group's range comes from the (wave-uniform) segment table.
-    float rcol[D];
-#pragma unroll
-    for (int i = 0; i < D; i++) rcol[i] = P.k_rot_T[i * D + j];
+    // One round of independent loads: the rotation (parked in LDS, as in the append), the
+    // thread's source dim and group; the group's range comes from the (wave-uniform) segment table.
+    rot_piece rst[D / 4];
+    fetch_rotation(P.k_rot_T, j, rst);
     const int src = P.head_perm[j];
     const int g = P.group_of[j];
     int s = 0, e = 0, ident = 0;
@@ -466,39 +592,54 @@ __device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t ro
         if (k == g) { s = ks; e = ks + kl; ident = ki; }
     }
     xs[j] = bgtq_h2f(a.q[row * a.q_sr + hq * a.q_sh + src]);
+    park_rotation(rot_s, j, rst);
     __syncthreads();
+    ET(1);
     float acc = 0.f;
     if (g >= 0) {
         if (ident) {
             acc = xs[j];
         } else {
-            // the same chain as over the group's own range: entries outside it are skipped
+            constexpr int CB = 16;              // LDS reads a batch ahead of the chain, as in the append
+            for (int k0 = s; k0 < e; k0 += CB) {
+                float rk[CB], xv[CB];
 #pragma unroll
-            for (int i = 0; i < D; i++)
-                if (i >= s && i < e) acc = __builtin_fmaf(xs[i], rcol[i], acc);
+                for (int i = 0; i < CB; i++) {
+                    const int k = min(k0 + i, e - 1);
+                    rk[i] = rot_s[k * D + j];
+                    xv[i] = xs[k];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < CB; i++)
+                    if (k0 + i < e) acc = __builtin_fmaf(xv[i], rk[i], acc);
+            }
         }
     }
     a.q_rot[row * a.qr_sr + hq * a.qr_sh + j] = bgtq_f2h(acc);
+    ET(8);
 }
 
 __global__ __launch_bounds__(NT) void rotate_q_kernel(RotQArgs a) {
-    rotate_q_row(a, blockIdx.x, blockIdx.y);
+    __shared__ __align__(16) float rot_s[D * D];
+    rotate_q_row(a, blockIdx.x, blockIdx.y, rot_s);
 }
 
 // ---- decode-step preparation: append-encode K and V and rotate the queries, one launch ----
 // Work-groups [0, nk) encode K row pairs, [nk, nk + nv) V row pairs, the rest one query row each.
 __global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs av, RotQArgs aq,
                                                      int k_tiles, int v_tiles) {
+    __shared__ __align__(16) float rot_s[D * D];       // the work-group's rotation, whatever its role
     int bid = blockIdx.x;
     const int nk = k_tiles * ak.n_kv, nv = v_tiles * av.n_kv;
     if (bid < nk) {
-        encode_rows<2, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles);
+        encode_rows<2, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles, rot_s);
     } else if (bid < nk + nv) {
         bid -= nk;
-        encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles);
+        encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles, rot_s);
     } else {
         bid -= nk + nv;
-        rotate_q_row(aq, bid / aq.n_q, bid % aq.n_q);
+        rotate_q_row(aq, bid / aq.n_q, bid % aq.n_q, rot_s);
     }
 }
 
@@ -656,5 +797,11 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
     hipLaunchKernelGGL(prepare_kernel, dim3(blocks), dim3(NT), 0, (hipStream_t)stream, ak, av, aq, tiles, tiles);
     return bgtq_launch_status();
 }
+
+#ifdef BGTQ_TRACE
+int bgtq_debug_set_etrace(void* buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_etrace), &buf, sizeof(buf));
+}
+#endif
 
 }  // extern "C"
