@@ -387,12 +387,21 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         steptab[i * 2] = (uint4){o & ~3u, o & 3u, r[2] + smem_lds + VTAB_BYTES, r[3]};     // table as an absolute LDS address
         steptab[i * 2 + 1] = (uint4){r[4], r[5], r[6] * MT / 64, r[7]};   // norm rows are MT tokens long here
     }
-    for (int i = tid; i < 16 * (QROW / 4); i += nthr) {     // query units, zero padded
-        const int hd = i / (QROW / 4), rem = i - hd * (QROW / 4), uid = rem >> 2, pp = rem & 3;
-        const int d0 = qu_s[uid] + 2 * pp, len = qu_s[32 + uid];
-        const uint16_t* row = q_s + hd * D;
-        const uint32_t lo = 2 * pp < len ? row[d0] : 0, hi = 2 * pp + 1 < len ? row[d0 + 1] : 0;
-        ((uint32_t*)qpad)[i] = lo | (hi << 16);
+    // query units, zero padded: one thread per 16-byte unit (two LDS round trips in all: the unit
+    // map, then the four words of the row, which start on an even dim)
+    for (int i = tid; i < 16 * (QROW / 16); i += nthr) {
+        const int hd = i / (QROW / 16), uid = i - hd * (QROW / 16);
+        const int d0 = qu_s[uid], len = qu_s[32 + uid];
+        const uint32_t* row = (const uint32_t*)(q_s + hd * D + d0);
+        uint32_t w[4];
+#pragma unroll
+        for (int pp = 0; pp < 4; pp++) w[pp] = row[min(pp, (D - d0) / 2 - 1)];
+#pragma unroll
+        for (int pp = 0; pp < 4; pp++) {
+            const uint32_t keep = (2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u);
+            w[pp] &= keep;
+        }
+        ((uint4*)qpad)[i] = uint4{w[0], w[1], w[2], w[3]};
     }
     __syncthreads();                                        // scratch is dead from here
     if (tile < t1 && !v_early) v_loads = issue_v(tile);
