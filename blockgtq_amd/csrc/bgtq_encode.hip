@@ -222,7 +222,10 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     ET(1);
     // ---- per-thread static data -------------------------------------------
     int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
+    float lut_off_j = 0.f, lut_scale_j = 0.f;          // K: this dim's cell-search parameters
     if constexpr (!IS_V) {
+        lut_off_j = sp.lut_offset[j];
+        lut_scale_j = sp.lut_inv_scale[j];
         n_seg = sp.hdr[H_NSEG];
         g = sp.group_of[j];
         src_dim = sp.head_perm[j];
@@ -429,7 +432,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
                     int nb = (1 << sp.hdr[H_BW + g]) - 1;
                     for (int b = 0; b < nb; b++) code += (P.k_boundaries[g][b] < y[r]) ? 1 : 0;
                 } else {
-                    float t = (y[r] - sp.lut_offset[j]) * sp.lut_inv_scale[j];
+                    float t = (y[r] - lut_off_j) * lut_scale_j;
                     t = fminf(fmaxf(t, 0.0f), (float)(BGTQ_LUT_BINS - 1));
                     code = sp.code_lut[g * BGTQ_LUT_BINS + (int)t];
                 }
