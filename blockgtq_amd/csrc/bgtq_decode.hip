@@ -288,6 +288,9 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     const float* R = plans[hq / gqa].v_rot;
     const float* po = part_out + row * n_splits * D + c4;
 
+    // loads land in issue order: the partitions' log-sum-exps go first, so that the maximum and
+    // the weights are worked out while the vectors and the un-rotation are still on their way
+    const float l_first = j < n_splits ? pl[j] : -INFINITY;
     constexpr int NB = 4;                      // rounds of 4 partial vectors fetched before anything else
     float4 pv[NB];
 #pragma unroll
@@ -298,8 +301,9 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
         for (int i = 0; i < D / 4; i++) rv[i] = *(const float4*)(R + (4 * i + cls) * D + c4);
     }
 
-    float m = -INFINITY;
-    for (int c = j; c < n_splits; c += D) { float l = pl[c]; wgt[c] = l; m = fmaxf(m, l); }
+    float m = l_first;
+    if (j < n_splits) wgt[j] = l_first;
+    for (int c = j + D; c < n_splits; c += D) { float l = pl[c]; wgt[c] = l; m = fmaxf(m, l); }
     for (int c = j; c < n_extra; c += D) m = fmaxf(m, el[c]);
     m = wave_max(m);
     if ((j & 63) == 0) red[j >> 6] = m;
