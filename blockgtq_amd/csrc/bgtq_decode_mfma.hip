@@ -523,12 +523,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             auto tables = [&]() {                           // table words
 #pragma unroll
                 for (int k = 0; k < NBLK; k++)
-#ifdef BGTQ_EXPERIMENT_NOKLUT
-                    w[k] = (uint4v){ad[k][0], ad[k][1], ad[k][2], ad[k][3]};
-#else
                     w[k] = (uint4v){lds_at<uint32_t>(ad[k][0]), lds_at<uint32_t>(ad[k][1]),
                                    lds_at<uint32_t>(ad[k][2]), lds_at<uint32_t>(ad[k][3])};
-#endif
             };
             // one MFMA per row block from a zero accumulator, scaled by the fp16 group norm of
             // its token rows in fp32
@@ -707,11 +703,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                         constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
                         const int fp = e * 2 * VBW;
                         const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
-#ifdef BGTQ_EXPERIMENT_NOVLUT
-                        W[r][e] = and_or(sh, fmask, vbank);
-#else
                         W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
-#endif
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
