@@ -411,6 +411,26 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
 
 static int g_decode_path = 0;
 
+// ---- with-buffer append: the token in ring slot slot[b] leaves, this step's token enters -----
+// One work-group per (KV head, batch row), thread j moves dim j of K and of V.  A slot outside
+// [0, W) moves nothing and leaves zeros in the outputs.
+__global__ __launch_bounds__(D) void window_swap_kernel(
+    uint16_t* kbuf, uint16_t* vbuf, int64_t w_sb, int64_t w_sh, int64_t w_st,
+    const uint16_t* new_k, const uint16_t* new_v, int64_t n_sb, int64_t n_sh,
+    const int32_t* slot, int W, int n_kv, uint16_t* old_k, uint16_t* old_v) {
+    const int j = threadIdx.x, h = blockIdx.x, b = blockIdx.y;
+    const int sl = slot[b];
+    const int64_t o = ((int64_t)b * n_kv + h) * D + j;
+    if (sl < 0 || sl >= W) { old_k[o] = 0; old_v[o] = 0; return; }
+    const int64_t at = b * w_sb + h * w_sh + (int64_t)sl * w_st + j;
+    const int64_t nw = b * n_sb + h * n_sh + j;
+    const uint16_t nk = new_k[nw], nv = new_v[nw];
+    old_k[o] = kbuf[at];
+    old_v[o] = vbuf[at];
+    kbuf[at] = nk;
+    vbuf[at] = nv;
+}
+
 extern "C" {
 
 int bgtq_set_decode_path(int path) {
@@ -517,6 +537,20 @@ int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
                        (hipStream_t)stream, (const uint16_t*)q, q_sb, q_sh,
                        (const uint16_t*)kbuf, (const uint16_t*)vbuf, w_sb, w_sh, w_st,
                        lens, W, n_kv * gqa, gqa, scale, part_out, part_lse);
+    return bgtq_launch_status();
+}
+
+int bgtq_window_swap(void* kbuf, void* vbuf, int64_t w_sb, int64_t w_sh, int64_t w_st,
+                     const void* new_k, const void* new_v, int64_t n_sb, int64_t n_sh,
+                     const int32_t* slot, int W, int B, int n_kv,
+                     void* old_k, void* old_v, void* stream) {
+    BGTQ_CHECK_ARG(kbuf && vbuf && new_k && new_v && slot && old_k && old_v);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && W >= 1);
+    if (B == 0 || n_kv == 0) return BGTQ_OK;
+    hipLaunchKernelGGL(window_swap_kernel, dim3((unsigned)n_kv, (unsigned)B), dim3(D), 0, (hipStream_t)stream,
+                       (uint16_t*)kbuf, (uint16_t*)vbuf, w_sb, w_sh, w_st,
+                       (const uint16_t*)new_k, (const uint16_t*)new_v, n_sb, n_sh, slot, W, n_kv,
+                       (uint16_t*)old_k, (uint16_t*)old_v);
     return bgtq_launch_status();
 }
 

@@ -182,6 +182,30 @@ def window_attention(q: torch.Tensor, kbuf: torch.Tensor, vbuf: torch.Tensor,
     return po, pl
 
 
+def window_swap(kbuf: torch.Tensor, vbuf: torch.Tensor, new_k: torch.Tensor, new_v: torch.Tensor,
+                slot: torch.Tensor):
+    """Ring update of the with-buffer append in one launch: for every batch row the fp16
+    token in slot ``slot[b]`` of ``kbuf`` / ``vbuf`` (B, n_kv, W, D) is returned and replaced by
+    ``new_k`` / ``new_v`` (B, n_kv, D).  ``slot`` int32 device tensor (B,); rows whose slot lies
+    outside [0, W) move nothing and return zeros.  Returns (old_k, old_v), each (B, n_kv, 1, D)."""
+    _capi.require_cuda(kbuf, "kbuf")
+    for t in (kbuf, vbuf, new_k, new_v):
+        assert t.dtype == torch.float16 and t.stride(-1) == 1
+    assert kbuf.shape == vbuf.shape and kbuf.stride() == vbuf.stride()
+    assert new_k.shape == new_v.shape and new_k.stride() == new_v.stride()
+    assert slot.dtype == torch.int32 and slot.is_contiguous()
+    B, n_kv, W, D = kbuf.shape
+    assert new_k.shape == (B, n_kv, D)
+    old_k = torch.empty((B, n_kv, 1, D), dtype=torch.float16, device=kbuf.device)
+    old_v = torch.empty_like(old_k)
+    _capi.check(_capi.lib().bgtq_window_swap(
+        _capi.ptr(kbuf), _capi.ptr(vbuf), kbuf.stride(0), kbuf.stride(1), kbuf.stride(2),
+        _capi.ptr(new_k), _capi.ptr(new_v), new_k.stride(0), new_k.stride(1),
+        _capi.ptr(slot), W, B, n_kv, _capi.ptr(old_k), _capi.ptr(old_v),
+        _capi.stream_ptr(kbuf.device)), "bgtq_window_swap")
+    return old_k, old_v
+
+
 @torch.no_grad()
 def dequant_kv(plans: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tensor,
                v_packed: torch.Tensor, v_norms: torch.Tensor, T: int, *,

@@ -213,7 +213,7 @@ class BlockGTQKVManager:
         buf_len = (p + 1).clamp(max=ns + w).to(torch.int32)
         ar = torch.arange(self.B, device=p.device)
         self._step_src = self._seq_lens
-        self._step_idx = (ar, slot, t_flush, packed_len, buf_len)
+        self._step_idx = (ar, slot.to(torch.int32), t_flush, packed_len, buf_len)
         return self._step_idx
 
     @torch.no_grad()
@@ -228,14 +228,13 @@ class BlockGTQKVManager:
         B = q.shape[0]
         q3 = q.reshape(B, self.n_q, self.hd).to(torch.float16).contiguous()
         bk, bv = self._buf_k[li], self._buf_v[li]
-        old_k = bk[ar, :, slot].unsqueeze(2)                # (B, n_kv, 1, D): tokens leaving the window
-        old_v = bv[ar, :, slot].unsqueeze(2)
+        # the tokens leaving the window come out (B, n_kv, 1, D), this step's tokens go in
+        old_k, old_v = ops.window_swap(bk, bv, k_new[:, :, 0].to(torch.float16),
+                                       v_new[:, :, 0].to(torch.float16), slot)
         q_rot = ops.decode_prepare(
             plans, old_k, old_v, q3, self._k_packed[li], self._k_norms[li],
             self._v_packed[li], self._v_norms[li], t_flush, self._k_rows[li],
             self._k_norms.shape[-1], self._vpb, self.n_kv, _plan.K_BITPACKED, _plan.V_BITPACKED)
-        bk[ar, :, slot] = k_new[:, :, 0].to(torch.float16)
-        bv[ar, :, slot] = v_new[:, :, 0].to(torch.float16)
         ext_out, ext_lse = ops.window_attention(q3, bk, bv, buf_len, self.n_kv, self.scale)
         T = max(self.seq_len + 1 - self.n_sink - self.window, 1)
         out = ops.decode_attention(

@@ -368,6 +368,25 @@ int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
                      float* part_out, float* part_lse, void* stream);
 
 /*
+ * With-buffer append, one launch for the ring update of a decode step: for every
+ * batch row the fp16 token in ring slot slot[b] leaves the window (it is copied to
+ * old_k / old_v, from where the caller encodes it into the packed cache) and this
+ * step's token takes its place.  One launch instead of the four indexed tensor
+ * copies per layer that the same update costs otherwise.  The reference keeps
+ * sink, quantised middle and fp16 tail in one growing fp16 cache and rewrites the
+ * oldest tail block in place once the tail exceeds the window
+ * (blockgtq/unaccelerated.py:204-240); here the tail is a ring of W slots.
+ *   kbuf, vbuf    fp16 [B][n_kv][W][128], common strides w_sb/w_sh/w_st in halves
+ *   new_k, new_v  fp16 [B][n_kv][128], common strides n_sb/n_sh in halves
+ *   slot          device int32[B]; a slot outside [0, W) moves nothing for that row
+ *   old_k, old_v  fp16 [B][n_kv][128] contiguous (zeros for rows that moved nothing)
+ */
+int bgtq_window_swap(void* kbuf, void* vbuf, int64_t w_sb, int64_t w_sh, int64_t w_st,
+                     const void* new_k, const void* new_v, int64_t n_sb, int64_t n_sh,
+                     const int32_t* slot, int W, int B, int n_kv,
+                     void* old_k, void* old_v, void* stream);
+
+/*
  * Packed records back to fp16 vectors, all KV heads of a layer in one launch:
  * the tile dequantisation of the reference's prompt-phase attention kernel
  * (blockgtq/kernels/fused_packed_attention.py:1876-2594, helpers :1384-1533)

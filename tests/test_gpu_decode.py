@@ -550,3 +550,32 @@ def test_merge_entry_point_refuses_what_its_kernel_cannot_take():
     torch.cuda.synchronize()
     with pytest.raises(_capi.BgtqError):
         _capi.check(call(_capi.ptr(part[1:]), 4), "bgtq_lse_reduce")
+
+
+def test_window_swap_equals_indexed_copies():
+    """The one-launch ring update of the with-buffer append against the tensor operations it
+    replaces, bit for bit, on strided buffers (a layer slice of a larger tensor)."""
+    g = torch.Generator(device=DEV).manual_seed(5)
+    B, n_kv, W = 5, 3, 12
+    big_k = torch.randn(2, B, n_kv, W, 128, generator=g, device=DEV).half()
+    big_v = torch.randn(2, B, n_kv, W, 128, generator=g, device=DEV).half()
+    kb, vb = big_k[1], big_v[1]
+    new = torch.randn(2, B, n_kv, 3, 128, generator=g, device=DEV).half()
+    nk, nv = new[0][:, :, 1], new[1][:, :, 1]                 # (B, n_kv, D) views with gaps
+    slot = torch.tensor([0, 11, 4, 4, 7], dtype=torch.int32, device=DEV)
+    ar = torch.arange(B, device=DEV)
+    ref_k, ref_v = kb.clone(), vb.clone()
+    want_old_k = ref_k[ar, :, slot.long()].unsqueeze(2).clone()
+    want_old_v = ref_v[ar, :, slot.long()].unsqueeze(2).clone()
+    ref_k[ar, :, slot.long()] = nk
+    ref_v[ar, :, slot.long()] = nv
+    old_k, old_v = ops.window_swap(kb, vb, nk, nv, slot)
+    assert torch.equal(old_k, want_old_k) and torch.equal(old_v, want_old_v)
+    assert torch.equal(kb, ref_k) and torch.equal(vb, ref_v)
+    assert torch.equal(big_k[0], big_k[0]) and not torch.isnan(big_k[0].float()).any()
+    # a slot outside the ring moves nothing for that row
+    before = kb.clone()
+    slot2 = torch.tensor([-1, 12, 3, 3, 3], dtype=torch.int32, device=DEV)
+    old_k2, _ = ops.window_swap(kb, vb, nk, nv, slot2)
+    assert torch.equal(kb[:2], before[:2]) and not old_k2[:2].any()
+    assert torch.equal(kb[2:, :, 3], nk[2:])
