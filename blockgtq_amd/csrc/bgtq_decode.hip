@@ -360,7 +360,7 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
 
 // ---- dense fp16 partial over the sink + recent-window tokens ------------------
 constexpr int WT = 256;
-__global__ __launch_bounds__(WT) void window_attn_kernel(
+__global__ __launch_bounds__(WT) void window_attn_generic_kernel(
     const uint16_t* q, int64_t q_sb, int64_t q_sh,
     const uint16_t* kbuf, const uint16_t* vbuf, int64_t w_sb, int64_t w_sh, int64_t w_st,
     const int32_t* lens, int W, int n_q, int gqa, float scale, float* part_out, float* part_lse) {
@@ -407,9 +407,175 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
     if (tid == 0) part_lse[row] = n > 0 ? m + __logf(l) : -INFINITY;
 }
 
-}  // namespace
 
-static int g_decode_path = 0;
+#ifdef BGTQ_TRACE
+__device__ unsigned long long* g_wtrace;
+#define WTR(slot) do { if (threadIdx.x == 0 && g_wtrace) g_wtrace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (slot)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define WTR(slot) do {} while (0)
+#endif
+// The same partial for buffers whose rows start on 16-byte boundaries (the manager's do): one
+// work-group per (batch row, KV head) serves all its query heads, HG at a time, so the window is
+// read once per HG heads, and every load is contiguous across the wave.  Scores: 16 lanes share a
+// token (8 dims each, one 16-byte load), 4 tokens per wave instruction; values: a wave covers
+// one token row per load (2 dims a lane), the four waves take every fourth token and their sums
+// meet in LDS.  wlog holds HG rows of W scores, then weights.
+// sum over the 16 lanes of a row, in every lane of it (rotations within the row: no LDS traffic)
+__device__ __forceinline__ float row16_sum(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x124, 0xf, 0xf, false));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x122, 0xf, 0xf, false));
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x121, 0xf, 0xf, false));
+    return x;
+}
+
+template <int HG>
+__global__ __launch_bounds__(WT) void window_attn_kernel(
+    const uint16_t* q, int64_t q_sb, int64_t q_sh,
+    const uint16_t* kbuf, const uint16_t* vbuf, int64_t w_sb, int64_t w_sh, int64_t w_st,
+    const int32_t* lens, int W, int n_q, int gqa, float scale, float* part_out, float* part_lse) {
+    extern __shared__ float wlog[];            // [HG][W]
+    __shared__ float red_m[HG], red_l[HG];
+    __shared__ float osum[WT / 64][HG][D];
+    constexpr int NW = WT / 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int h = blockIdx.x, b = blockIdx.y;
+    const int n = lens ? min(lens[b], W) : W;
+    const uint16_t* kb = kbuf + b * w_sb + h * w_sh;
+    const uint16_t* vb = vbuf + b * w_sb + h * w_sh;
+    const int sub = lane & 15, tq = lane >> 4;  // scores: dim chunk and token within a wave load
+    WTR(0);
+    // Loads run one batch ahead of the arithmetic that uses them (a batch waited for on the spot
+    // costs a trip to memory each); batches are small and the loops rolled, because code that
+    // runs once pays for its instruction-cache misses.
+    constexpr int SB = 3;                       // score passes (4 tokens per wave each) per batch
+    constexpr int PB = 8;                       // value rows per batch
+    auto fetch_k = [&](uint4 (&k4)[SB], const int t0) {
+#pragma unroll
+        for (int u = 0; u < SB; u++) {
+            const int t = t0 + u * 4 * NW + tq;
+            k4[u] = uint4{0, 0, 0, 0};
+            if (t < n) k4[u] = *(const uint4*)(kb + (int64_t)t * w_st + sub * 8);
+        }
+    };
+    auto fetch_v = [&](uint32_t (&vv)[PB], const int t0) {
+#pragma unroll
+        for (int u = 0; u < PB; u++) {
+            const int t = t0 + u * NW;
+            vv[u] = t < n ? *(const uint32_t*)(vb + (int64_t)t * w_st + 2 * lane) : 0u;
+        }
+    };
+    for (int g0 = 0; g0 < gqa; g0 += HG) {
+        const int ng = min(HG, gqa - g0);
+        // ---- scores: 16 lanes share a token ------------------------------------------------
+        float qf[HG][8];
+#pragma unroll
+        for (int g = 0; g < HG; g++) {
+            uint4 w4 = {0, 0, 0, 0};
+            if (g < ng) w4 = *(const uint4*)(q + b * q_sb + (int64_t)(h * gqa + g0 + g) * q_sh + sub * 8);
+            const uint32_t ws[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                qf[g][2 * i] = bgtq_h2f((uint16_t)(ws[i] & 0xFFFFu)) * scale;
+                qf[g][2 * i + 1] = bgtq_h2f((uint16_t)(ws[i] >> 16)) * scale;
+            }
+        }
+        uint4 kc[SB], kn[SB];
+        uint32_t vc[PB], vn[PB];
+        fetch_k(kc, wave * 4);
+        fetch_v(vc, wave);                      // the first value rows do not wait for the scores
+        WTR(1);
+#pragma unroll 1
+        for (int t0 = wave * 4; t0 < n; t0 += SB * 4 * NW) {
+            fetch_k(kn, t0 + SB * 4 * NW);
+#pragma unroll
+            for (int u = 0; u < SB; u++) {
+                const int t = t0 + u * 4 * NW + tq;
+                const uint32_t ks[4] = {kc[u].x, kc[u].y, kc[u].z, kc[u].w};
+                float kf[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    kf[2 * i] = bgtq_h2f((uint16_t)(ks[i] & 0xFFFFu));
+                    kf[2 * i + 1] = bgtq_h2f((uint16_t)(ks[i] >> 16));
+                }
+#pragma unroll
+                for (int g = 0; g < HG; g++) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc += qf[g][i] * kf[i];
+                    acc = row16_sum(acc);
+                    if (sub == 0 && t < n && g < ng) wlog[g * W + t] = acc;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < SB; u++) kc[u] = kn[u];
+        }
+        WTR(2);
+        __syncthreads();
+        WTR(3);
+        // ---- softmax weights: wave w owns heads w, w + 4, ... ----------------------------------
+        for (int g = wave; g < ng; g += NW) {
+            float mm = -INFINITY;
+            for (int t = lane; t < n; t += 64) mm = fmaxf(mm, wlog[g * W + t]);
+            mm = wave_max(mm);
+            float ll = 0.f;
+            for (int t = lane; t < n; t += 64) {
+                const float p = __expf(wlog[g * W + t] - mm);
+                wlog[g * W + t] = p;
+                ll += p;
+            }
+            ll = wave_sum(ll);
+            if (lane == 0) { red_m[g] = mm; red_l[g] = ll; }
+        }
+        __syncthreads();
+        WTR(4);
+        // ---- values: wave w takes tokens w, w + 4, ...; lane = dims 2 lane, 2 lane + 1 -------
+        float o0[HG], o1[HG];
+#pragma unroll
+        for (int g = 0; g < HG; g++) o0[g] = o1[g] = 0.f;
+#pragma unroll 1
+        for (int t0 = wave; t0 < n; t0 += PB * NW) {
+            fetch_v(vn, t0 + PB * NW);
+            float pw[PB][HG];                   // the batch's weights, read together
+#pragma unroll
+            for (int u = 0; u < PB; u++)
+#pragma unroll
+                for (int g = 0; g < HG; g++) {
+                    const int t = min(t0 + u * NW, n - 1);
+                    pw[u][g] = wlog[min(g, ng - 1) * W + t];
+                }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < PB; u++) {
+                const bool live = t0 + u * NW < n;
+                const float v0 = bgtq_h2f((uint16_t)(vc[u] & 0xFFFFu)), v1 = bgtq_h2f((uint16_t)(vc[u] >> 16));
+#pragma unroll
+                for (int g = 0; g < HG; g++) {
+                    const float p = (g < ng && live) ? pw[u][g] : 0.f;
+                    o0[g] += p * v0;
+                    o1[g] += p * v1;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < PB; u++) vc[u] = vn[u];
+        }
+        WTR(5);
+#pragma unroll
+        for (int g = 0; g < HG; g++) { osum[wave][g][2 * lane] = o0[g]; osum[wave][g][2 * lane + 1] = o1[g]; }
+        __syncthreads();
+        WTR(6);
+        for (int i = tid; i < ng * D; i += WT) {
+            const int g = i / D, d = i - g * D;
+            const float acc = (osum[0][g][d] + osum[1][g][d]) + (osum[2][g][d] + osum[3][g][d]);
+            const size_t row = (size_t)b * n_q + h * gqa + g0 + g;
+            const float mg = red_m[g], lg = red_l[g];
+            part_out[row * D + d] = n > 0 ? acc / lg : 0.f;
+            if (d == 0) part_lse[row] = n > 0 ? mg + __logf(lg) : -INFINITY;
+        }
+        __syncthreads();                        // wlog, red_* and osum are reused by the next heads
+        WTR(7);
+    }
+}
 
 // ---- with-buffer append: the token in ring slot slot[b] leaves, this step's token enters -----
 // One work-group per (KV head, batch row), thread j moves dim j of K and of V.  A slot outside
@@ -430,6 +596,10 @@ __global__ __launch_bounds__(D) void window_swap_kernel(
     kbuf[at] = nk;
     vbuf[at] = nv;
 }
+
+}  // namespace
+
+static int g_decode_path = 0;
 
 extern "C" {
 
@@ -532,8 +702,26 @@ int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && gqa >= 1 && W >= 0);
     if (W > 8192) return BGTQ_ELIMIT;
     if (B == 0 || n_kv == 0) return BGTQ_OK;
+    const size_t wbytes = (size_t)(W > 0 ? W : 1) * sizeof(float);
+    // rows and query vectors on 16-byte boundaries: one work-group per (row, KV head)
+    const bool wide = (((uintptr_t)q | (uintptr_t)kbuf | (uintptr_t)vbuf) & 15) == 0 &&
+                      ((q_sb | q_sh | w_sb | w_sh | w_st) & 7) == 0;
+    if (wide) {
+        dim3 grid((unsigned)n_kv, (unsigned)B);
+        if (gqa > 1 && 4 * wbytes <= 48 * 1024)
+            hipLaunchKernelGGL((window_attn_kernel<4>), grid, dim3(WT), 4 * wbytes,
+                               (hipStream_t)stream, (const uint16_t*)q, q_sb, q_sh,
+                               (const uint16_t*)kbuf, (const uint16_t*)vbuf, w_sb, w_sh, w_st,
+                               lens, W, n_kv * gqa, gqa, scale, part_out, part_lse);
+        else
+            hipLaunchKernelGGL((window_attn_kernel<1>), grid, dim3(WT), wbytes,
+                               (hipStream_t)stream, (const uint16_t*)q, q_sb, q_sh,
+                               (const uint16_t*)kbuf, (const uint16_t*)vbuf, w_sb, w_sh, w_st,
+                               lens, W, n_kv * gqa, gqa, scale, part_out, part_lse);
+        return bgtq_launch_status();
+    }
     dim3 grid((unsigned)(n_kv * gqa), (unsigned)B);
-    hipLaunchKernelGGL(window_attn_kernel, grid, dim3(WT), (size_t)(W > 0 ? W : 1) * sizeof(float),
+    hipLaunchKernelGGL(window_attn_generic_kernel, grid, dim3(WT), wbytes,
                        (hipStream_t)stream, (const uint16_t*)q, q_sb, q_sh,
                        (const uint16_t*)kbuf, (const uint16_t*)vbuf, w_sb, w_sh, w_st,
                        lens, W, n_kv * gqa, gqa, scale, part_out, part_lse);
@@ -566,5 +754,11 @@ const char* bgtq_strerror(int code) {
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }
+
+#ifdef BGTQ_TRACE
+int bgtq_debug_set_wtrace(void* buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_wtrace), &buf, sizeof(buf));
+}
+#endif
 
 }  // extern "C"

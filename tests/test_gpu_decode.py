@@ -579,3 +579,35 @@ def test_window_swap_equals_indexed_copies():
     old_k2, _ = ops.window_swap(kb, vb, nk, nv, slot2)
     assert torch.equal(kb[:2], before[:2]) and not old_k2[:2].any()
     assert torch.equal(kb[2:, :, 3], nk[2:])
+
+
+@pytest.mark.parametrize("B,n_kv,gqa,W,lens,offset", [
+    (3, 2, 4, 132, [132, 77, 0], 0),        # four heads per pass, an empty row
+    (2, 1, 7, 40, [40, 1], 0),              # two passes, the second with three heads
+    (2, 2, 1, 200, [200, 129], 0),          # one head per KV head
+    (1, 1, 2, 4000, [3999], 0),             # window too long for four score rows in LDS
+    (2, 2, 4, 50, [50, 13], 1),             # rows off the 16-byte boundaries: the general kernel
+])
+def test_window_attention_every_path(B, n_kv, gqa, W, lens, offset):
+    """fp16 window partial against a float64 softmax: out within 1e-3, lse within 1e-3."""
+    g = torch.Generator(device=DEV).manual_seed(W + gqa)
+    n_q = n_kv * gqa
+
+    def buf(*shape):                         # optionally shifted by `offset` halves inside a larger block
+        flat = torch.randn(int(np.prod(shape)) + 8, generator=g, device=DEV).half()
+        return flat[offset:offset + int(np.prod(shape))].view(*shape)
+
+    q, kb, vb = buf(B, n_q, 128), buf(B, n_kv, W, 128), buf(B, n_kv, W, 128)
+    lens_t = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    po, pl = ops.window_attention(q, kb, vb, lens_t, n_kv)
+    for b in range(B):
+        n = lens[b]
+        for hq in range(n_q):
+            if n == 0:
+                assert float(pl[b, hq]) == float("-inf") and not po[b, hq].any()
+                continue
+            h = hq // gqa
+            lw = (q[b, hq].double() @ kb[b, h, :n].double().T) / np.sqrt(128)
+            want = torch.softmax(lw, 0) @ vb[b, h, :n].double()
+            assert (po[b, hq].double() - want).abs().max() < 1e-3
+            assert abs(float(pl[b, hq]) - float(torch.logsumexp(lw, 0))) < 1e-3
