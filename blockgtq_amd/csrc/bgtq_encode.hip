@@ -574,16 +574,22 @@ struct RotQArgs {
     const uint16_t* q;  int64_t q_sr, q_sh;
     uint16_t* q_rot;    int64_t qr_sr, qr_sh;
     int n_rows, n_q, gqa;
+    int group;          // query heads per work-group: 1 or 4
 };
 
-__device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t row, const int hq,
-                                             float* rot_s) {
-    __shared__ float xs[D];
+// QG query heads (h_first ..) of one (row, KV head): the rotation is fetched and parked once for
+// all of them, the rows come in with the same round of loads (un-permuted, so that their
+// addresses do not wait for head_perm; the gather by head_perm then runs through LDS), and a
+// batch of the rotation column read from LDS serves every row.  Each row's chain is the one
+// written in the contract above; rows past the group's last head are zeros and are not stored.
+template <int QG>
+__device__ __forceinline__ void rotate_q_group(const RotQArgs& a, const int64_t row, const int h,
+                                               const int h_first, float* rot_s) {
+    __shared__ uint16_t qraw[QG][D];
+    __shared__ float xs[QG][D];
     const int j = threadIdx.x;
     ET(0);
-    const bgtq_head_plan& P = a.plans[hq / a.gqa];
-    // One round of independent loads: the rotation (parked in LDS, as in the append), the
-    // thread's source dim and group; the group's range comes from the (wave-uniform) segment table.
+    const bgtq_head_plan& P = a.plans[h];
     rot_piece rst[D / 4];
     fetch_rotation(P.k_rot_T, j, rst);
     const int src = P.head_perm[j];
@@ -594,42 +600,74 @@ __device__ __forceinline__ void rotate_q_row(const RotQArgs& a, const int64_t ro
         const int ks = P.seg_start[k], kl = P.seg_len[k], ki = P.seg_identity[k];
         if (k == g) { s = ks; e = ks + kl; ident = ki; }
     }
-    xs[j] = bgtq_h2f(a.q[row * a.q_sr + hq * a.q_sh + src]);
+    const int gqa = a.gqa;
+#pragma unroll
+    for (int r = 0; r < QG; r++)
+        qraw[r][j] = h_first + r < gqa ? a.q[row * a.q_sr + (int64_t)(h * gqa + h_first + r) * a.q_sh + j] : (uint16_t)0;
     park_rotation(rot_s, j, rst);
     __syncthreads();
+#pragma unroll
+    for (int r = 0; r < QG; r++) xs[r][j] = bgtq_h2f(qraw[r][src]);
+    __syncthreads();
     ET(1);
-    float acc = 0.f;
+    float acc[QG];
+#pragma unroll
+    for (int r = 0; r < QG; r++) acc[r] = 0.f;
     if (g >= 0) {
         if (ident) {
-            acc = xs[j];
+#pragma unroll
+            for (int r = 0; r < QG; r++) acc[r] = xs[r][j];
         } else {
-            constexpr int CB = 16;              // LDS reads a batch ahead of the chain, as in the append
+            constexpr int CB = QG == 1 ? 16 : 8;    // LDS reads a batch ahead of the chains
             for (int k0 = s; k0 < e; k0 += CB) {
-                float rk[CB], xv[CB];
+                float rk[CB], xv[QG][CB];
 #pragma unroll
                 for (int i = 0; i < CB; i++) {
                     const int k = min(k0 + i, e - 1);
                     rk[i] = rot_s[k * D + j];
-                    xv[i] = xs[k];
+#pragma unroll
+                    for (int r = 0; r < QG; r++) xv[r][i] = xs[r][k];
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < CB; i++)
-                    if (k0 + i < e) acc = __builtin_fmaf(xv[i], rk[i], acc);
+                    if (k0 + i < e) {
+#pragma unroll
+                        for (int r = 0; r < QG; r++) acc[r] = __builtin_fmaf(xv[r][i], rk[i], acc[r]);
+                    }
             }
         }
     }
-    a.q_rot[row * a.qr_sr + hq * a.qr_sh + j] = bgtq_f2h(acc);
+#pragma unroll
+    for (int r = 0; r < QG; r++)
+        if (h_first + r < gqa)
+            a.q_rot[row * a.qr_sr + (int64_t)(h * gqa + h_first + r) * a.qr_sh + j] = bgtq_f2h(acc[r]);
     ET(8);
+}
+
+// Work-group `bid` of the query part: a.group heads of one (row, KV head).  One head per
+// work-group where that still leaves the chip partly idle (every work-group fetches the 64 KB
+// rotation), four where the rows are many.
+__device__ __forceinline__ void rotate_q_block(const RotQArgs& a, const int bid, float* rot_s) {
+    const int n_kv = a.n_q / a.gqa;
+    const int per = (a.gqa + a.group - 1) / a.group;            // work-groups per (row, KV head)
+    const int rowh = bid / per, part = bid - rowh * per;
+    if (a.group == 1) rotate_q_group<1>(a, rowh / n_kv, rowh % n_kv, part, rot_s);
+    else              rotate_q_group<4>(a, rowh / n_kv, rowh % n_kv, part * 4, rot_s);
+}
+__host__ inline int rotate_q_group_size(int64_t n_rows, int n_q) { return n_rows * n_q > 256 ? 4 : 1; }
+__host__ inline unsigned rotate_q_blocks(int64_t n_rows, int n_kv, int gqa, int group) {
+    return (unsigned)(n_rows * n_kv * ((gqa + group - 1) / group));
 }
 
 __global__ __launch_bounds__(NT) void rotate_q_kernel(RotQArgs a) {
     __shared__ __align__(16) float rot_s[D * D];
-    rotate_q_row(a, blockIdx.x, blockIdx.y, rot_s);
+    rotate_q_block(a, blockIdx.x, rot_s);
 }
 
 // ---- decode-step preparation: append-encode K and V and rotate the queries, one launch ----
-// Work-groups [0, nk) encode K row pairs, [nk, nk + nv) V row pairs, the rest one query row each.
+// Work-groups [0, nk) encode K row pairs, [nk, nk + nv) V row pairs, the rest rotate one or four
+// query heads each.
 __global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs av, RotQArgs aq,
                                                      int k_tiles, int v_tiles) {
     __shared__ __align__(16) float rot_s[D * D];       // the work-group's rotation, whatever its role
@@ -641,8 +679,7 @@ __global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs a
         bid -= nk;
         encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles, rot_s);
     } else {
-        bid -= nk + nv;
-        rotate_q_row(aq, bid / aq.n_q, bid % aq.n_q, rot_s);
+        rotate_q_block(aq, bid - (nk + nv), rot_s);
     }
 }
 
@@ -758,9 +795,10 @@ int bgtq_rotate_q(const bgtq_head_plan* plans,
     BGTQ_CHECK_ARG(plans && q && q_rot);
     BGTQ_CHECK_ARG(n_rows >= 0 && n_kv >= 0 && gqa >= 1);
     if (n_rows == 0 || n_kv == 0) return BGTQ_OK;
-    RotQArgs a{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, n_rows, n_kv * gqa, gqa};
-    dim3 grid((unsigned)n_rows, (unsigned)(n_kv * gqa));
-    hipLaunchKernelGGL(rotate_q_kernel, grid, dim3(NT), 0, (hipStream_t)stream, a);
+    const int group = rotate_q_group_size(n_rows, n_kv * gqa);
+    RotQArgs a{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, n_rows, n_kv * gqa, gqa, group};
+    hipLaunchKernelGGL(rotate_q_kernel, dim3(rotate_q_blocks(n_rows, n_kv, gqa, group)), dim3(NT), 0,
+                       (hipStream_t)stream, a);
     return bgtq_launch_status();
 }
 
@@ -794,9 +832,10 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
         if (rc != BGTQ_OK) return rc;
         return bgtq_rotate_q(plans, q, q_sr, q_sh, q_rot, qr_sr, qr_sh, B, n_kv, gqa, stream);
     }
-    RotQArgs aq{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, B, n_kv * gqa, gqa};
+    const int group = rotate_q_group_size(B, n_kv * gqa);
+    RotQArgs aq{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, B, n_kv * gqa, gqa, group};
     const int tiles = (int)((N + 1) / 2);
-    const unsigned blocks = (unsigned)(2 * tiles * n_kv + B * n_kv * gqa);
+    const unsigned blocks = (unsigned)(2 * tiles * n_kv) + rotate_q_blocks(B, n_kv, gqa, group);
     hipLaunchKernelGGL(prepare_kernel, dim3(blocks), dim3(NT), 0, (hipStream_t)stream, ak, av, aq, tiles, tiles);
     return bgtq_launch_status();
 }
