@@ -823,19 +823,20 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
     rc = fill_v_args(av, plans, v, v_sb, v_sh, v_ss, B, n_kv, S, v_packed, vp_sb, vp_sh, vp_st, v_row_width,
                      v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, v_layout);
     if (rc != BGTQ_OK) return rc;
-    BGTQ_CHECK_ARG(q && q_rot);
+    BGTQ_CHECK_ARG((q == nullptr) == (q_rot == nullptr));     // both, or neither (queries rotated elsewhere)
+    const bool with_q = q != nullptr;
     const int64_t N = (int64_t)B * S;
     if (N > 64) {          // prefill-sized append: the three stages are big enough on their own
         rc = launch_encode<false>(ak, (hipStream_t)stream);
         if (rc != BGTQ_OK) return rc;
         rc = launch_encode<true>(av, (hipStream_t)stream);
-        if (rc != BGTQ_OK) return rc;
+        if (rc != BGTQ_OK || !with_q) return rc;
         return bgtq_rotate_q(plans, q, q_sr, q_sh, q_rot, qr_sr, qr_sh, B, n_kv, gqa, stream);
     }
     const int group = rotate_q_group_size(B, n_kv * gqa);
     RotQArgs aq{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, B, n_kv * gqa, gqa, group};
     const int tiles = (int)((N + 1) / 2);
-    const unsigned blocks = (unsigned)(2 * tiles * n_kv) + rotate_q_blocks(B, n_kv, gqa, group);
+    const unsigned blocks = (unsigned)(2 * tiles * n_kv) + (with_q ? rotate_q_blocks(B, n_kv, gqa, group) : 0u);
     hipLaunchKernelGGL(prepare_kernel, dim3(blocks), dim3(NT), 0, (hipStream_t)stream, ak, av, aq, tiles, tiles);
     return bgtq_launch_status();
 }

@@ -128,15 +128,17 @@ def decode_prepare(plans: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q: tor
     """One launch for everything a decode step does before attention: encode
     ``k`` / ``v`` (B, n_kv, S, D) fp16 into the cache views at ``t_pos`` (int or
     int32 device tensor (B,)) and rotate ``q`` (B, n_q, D) fp16.  Returns the
-    rotated queries; same results as ``encode_k_into`` + ``encode_v_into`` + ``rotate_q``."""
+    rotated queries; same results as ``encode_k_into`` + ``encode_v_into`` + ``rotate_q``.
+    ``q`` may be None (queries rotated elsewhere): K and V are appended in one launch and
+    None is returned."""
     _capi.require_cuda(k, "k")
-    for t in (k, v, q):
+    for t in (k, v) + ((q,) if q is not None else ()):
         assert t.dtype == torch.float16 and t.stride(-1) == 1
     assert k_packed.dtype == torch.uint8 and v_packed.dtype == torch.uint8
     assert k_norms.dtype == torch.float16 and v_norms.dtype == torch.float16
     B, H, S, _ = k.shape
-    n_q = q.shape[1]
-    q_rot = torch.empty((B, n_q, q.shape[2]), dtype=torch.float16, device=q.device)
+    n_q = q.shape[1] if q is not None else n_kv
+    q_rot = torch.empty((B, n_q, q.shape[2]), dtype=torch.float16, device=q.device) if q is not None else None
     if isinstance(t_pos, torch.Tensor):
         assert t_pos.dtype == torch.int32 and t_pos.is_cuda
         tp, ts = _capi.ptr(t_pos), 0
@@ -151,7 +153,8 @@ def decode_prepare(plans: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q: tor
         _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), v_row_width,
         _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
         tp, ts, k_layout, v_layout, quant_mode,
-        _capi.ptr(q), q.stride(0), q.stride(1), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1),
+        _capi.ptr(q), q.stride(0) if q is not None else 0, q.stride(1) if q is not None else 0,
+        _capi.ptr(q_rot), q_rot.stride(0) if q is not None else 0, q_rot.stride(1) if q is not None else 0,
         n_q // n_kv, _capi.stream_ptr(k.device)), "bgtq_decode_prepare")
     return q_rot
 

@@ -157,6 +157,12 @@ class BlockGTQKVManager:
             k16 = k16.contiguous()
         if v16.stride(-1) != 1:
             v16 = v16.contiguous()
+        if k16.shape[0] * k16.shape[2] <= 64:          # a decode append: K and V in one launch
+            ops.decode_prepare(plans, k16, v16, None, self._k_packed[li], self._k_norms[li],
+                               self._v_packed[li], self._v_norms[li], t_pos, self._k_rows[li],
+                               self._k_norms.shape[-1], self._vpb, self.n_kv,
+                               _plan.K_BITPACKED, _plan.V_BITPACKED)
+            return
         encode_k_into(plans, k16, self._k_packed[li], self._k_norms[li], t_pos,
                       self._k_rows[li], self._k_norms.shape[-1], _plan.K_BITPACKED)
         encode_v_into(plans, v16, self._v_packed[li], self._v_norms[li], t_pos,

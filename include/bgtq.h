@@ -266,7 +266,9 @@ int bgtq_rotate_q(const bgtq_head_plan* plans,
  * _compress_and_store K, V, then rotate_q_for_packed_kernel per KV head) and in
  * BlockGTQProductionCache.encode_and_attend (blockgtq/production_cache.py:207-245).
  * Arguments have the meaning they have in those three entry points; q has
- * B rows of n_kv * gqa heads.
+ * B rows of n_kv * gqa heads.  q and q_rot may both be NULL: then only K and V
+ * are appended, still in one launch (the caller's queries are rotated already,
+ * e.g. by a q_proj with the rotation folded in, blockgtq/quantizer.py:1190-1243).
  */
 int bgtq_decode_prepare(const bgtq_head_plan* plans,
                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss,

@@ -611,3 +611,28 @@ def test_window_attention_every_path(B, n_kv, gqa, W, lens, offset):
             want = torch.softmax(lw, 0) @ vb[b, h, :n].double()
             assert (po[b, hq].double() - want).abs().max() < 1e-3
             assert abs(float(pl[b, hq]) - float(torch.logsumexp(lw, 0))) < 1e-3
+
+
+def test_manager_with_rotated_queries_equals_manager_that_rotates_them():
+    """Queries that arrive rotated (rotation folded into q_proj) take the K/V-only append; cache
+    bytes and outputs equal those of the manager that rotates the queries itself."""
+    w = wl.Workload("t", 2, 16, 2, 2, 300, 1e6, min_bits=1, max_bits=5, seed=99)
+    a, energies = wl.build_manager(w, DEV)
+    b, _ = wl.build_manager(w, DEV)
+    wl.fill_cache(a, w, energies, DEV)
+    wl.fill_cache(b, w, energies, DEV)
+    for li in range(2):
+        for qz in b.quantizers[li]:
+            qz._q_perm_baked = True                      # b's caller hands over rotated queries
+    for step in range(2):
+        for li in range(2):
+            T = a.seq_len
+            q = wl.draw_q(w, li + 7 * step, DEV, T)
+            k1, v1 = wl.draw_kv(w, energies[li], 1, 31 + li + 7 * step, DEV, pos0=T)
+            out_a = a.append_and_attend(li, q, k1, v1)
+            q_rot = ops.rotate_q(a._batched_args[li]['plans'], q[:, :, 0].contiguous(), w.n_kv)
+            out_b = b.append_and_attend(li, q_rot.unsqueeze(2), k1, v1)
+            assert torch.equal(out_a, out_b)
+            assert torch.equal(a._k_packed[li], b._k_packed[li]) and torch.equal(a._v_packed[li], b._v_packed[li])
+            assert torch.equal(a._k_norms[li], b._k_norms[li]) and torch.equal(a._v_norms[li], b._v_norms[li])
+        a.increment_seq_len(); b.increment_seq_len()
