@@ -42,6 +42,8 @@
 //        above every score seen so far.  It is only moved (to the new maximum
 //        plus a headroom of 4 in log2 units) when a score of the tile exceeds it;
 //        otherwise the tile needs no cross-lane traffic at all.
+#include <atomic>
+
 #include "bgtq_decode.h"
 
 namespace {
@@ -837,8 +839,10 @@ int launch_kernel(const DecodeArgs& a, hipStream_t st) {
     const size_t smem = mfma_smem_bytes(a.k_layout, a.k_row_width, VST, (int)a.kn_st, nw);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
     auto kern = decode_mfma_kernel<VBW, VST, DENSE>;
-    static int ready = 0;                    // 1: usable, -1: not usable
-    if (ready == 0) {
+    // 1: usable, -1: not usable.  Two threads racing through the first call both run the idempotent
+    // set-up below and store the same value.
+    static std::atomic<int> ready{0};
+    if (ready.load(std::memory_order_acquire) == 0) {
         // the kernel addresses its V table as "LDS offset 0": that holds only while it has
         // no static LDS in front of the dynamic block
         hipFuncAttributes fa;
@@ -846,9 +850,9 @@ int launch_kernel(const DecodeArgs& a, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
         e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_LIMIT);
         if (e != hipSuccess) return (int)e;
-        ready = fa.sharedSizeBytes == 0 ? 1 : -1;
+        ready.store(fa.sharedSizeBytes == 0 ? 1 : -1, std::memory_order_release);
     }
-    if (ready < 0) return BGTQ_EUNSUPPORTED;
+    if (ready.load(std::memory_order_acquire) < 0) return BGTQ_EUNSUPPORTED;
     dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)a.B);
     hipLaunchKernelGGL(kern, grid, dim3(nw * 64), smem, st, a);
     return bgtq_launch_status();
