@@ -26,9 +26,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per attention launch from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy
-# kernel of known size (profiles/decode_mfma_kernel_<workload>_hbm_traffic.txt); valid for the
+# kernel of known size (profiles/decode_mfma_kernel_*_hbm_traffic.txt); valid for the
 # workload's own context, batch and default partition count only.
-MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 66.12e6}
+MEASURED_TRAFFIC_BYTES = {"qwen3b_b8_32k_k3v3": 66.12e6, "llama8b_4k_k3v3": 7.01e6,
+                          "llama8b_128k_k2v2": 88.68e6, "qwen3_8b_b32_ragged_buffered": 267.36e6}
 
 
 def parse():
