@@ -127,20 +127,24 @@ __device__ __forceinline__ void park_rotation(float* rot_s, const int j, const r
     for (int i = 0; i < D / 4; i++) ((rot_piece*)rot_s)[i * NT + j] = st[i];
 }
 
-// sum of x[k]^2 over [s, e) in LDS as ONE fmaf chain in increasing k.  The reads of a batch are all
-// issued before its first fmaf (left to itself the compiler waits for every few reads in turn, and
-// the chain then costs an LDS round trip per step instead of per batch).
-__device__ __forceinline__ float chain_sumsq(const float* x, const int s, const int e) {
-    constexpr int CB = 32;
+// Sum of x[k]^2 over a whole row of D values in LDS (V) as ONE fmaf chain in increasing k.  The reads
+// of a batch are all issued before its first fmaf (left to itself the compiler waits for every few
+// reads in turn); the chain itself runs at the 8 clocks of a dependent instruction.
+__device__ __forceinline__ float chain_sumsq_row(const float* x) {
     float ss = 0.f;
-    for (int k0 = s; k0 < e; k0 += CB) {
-        float v[CB];
 #pragma unroll
-        for (int i = 0; i < CB; i++) v[i] = x[min(k0 + i, e - 1)];
+    for (int k0 = 0; k0 < D; k0 += 32) {
+        float4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = *(const float4*)&x[k0 + 4 * i];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < CB; i++)
-            if (k0 + i < e) ss = __builtin_fmaf(v[i], v[i], ss);
+        for (int i = 0; i < 8; i++) {
+            ss = __builtin_fmaf(v[i].x, v[i].x, ss);
+            ss = __builtin_fmaf(v[i].y, v[i].y, ss);
+            ss = __builtin_fmaf(v[i].z, v[i].z, ss);
+            ss = __builtin_fmaf(v[i].w, v[i].w, ss);
+        }
     }
     return ss;
 }
@@ -287,7 +291,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             if constexpr (!IS_V) { s = sp.hdr[H_START + gg]; e = s + sp.hdr[H_LEN + gg]; }
             float ss = 0.f;
             if constexpr (IS_V) {
-                ss = chain_sumsq(xs[r], s, e);
+                ss = chain_sumsq_row(xs[r]);
             } else {                           // short ranges: the batches would mostly run masked
 #pragma unroll 8
                 for (int k = s; k < e; k++) ss = __builtin_fmaf(xs[r][k], xs[r][k], ss);
@@ -461,7 +465,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         if (gg < n_seg) {
             float n = nrm[r][gg];
             if (IS_V) {
-                const float cs = chain_sumsq(xs[r], 0, D);
+                const float cs = chain_sumsq_row(xs[r]);
                 float cn = __builtin_sqrtf(cs + 1e-20f);
                 out = n / (cn > 1e-10f ? cn : 1.0f);
             } else if (a.layout == BGTQ_K_MIXED || a.corrected) {
