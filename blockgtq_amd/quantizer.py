@@ -229,21 +229,31 @@ class BlockGTQQuantizer:
                                     kv_head_idx: int, n_kv_heads: int, n_q_heads: int,
                                     q_proj_bias: Optional[torch.Tensor] = None) -> None:
         """Fold permutation + rotation into the ``q_proj`` rows of this KV head's
-        query group, in place: ``W' = (R^T W[head_perm])`` (blockgtq/quantizer.py:1190-1243)."""
+        query group, in place, so that the projection's output equals
+        ``rotate_q_for_packed_kernel`` of the original projection's output.
+
+        The kernels and ``rotate_q_for_packed_kernel`` compute
+        ``q' = q[head_perm] @ block_rot_T`` (blockgtq/quantizer.py:1180-1187), i.e.
+        ``q' = block_rot_T^T (W x + b)[head_perm]``, hence
+        ``W' = block_rot_T^T W[head_perm]`` and ``b' = block_rot_T^T b[head_perm]``.
+        The reference's own baking routine multiplies by ``block_rot_T`` without the
+        transpose (blockgtq/quantizer.py:1232), which disagrees with its query rotation
+        for every non-symmetric rotation block; this implementation follows the query
+        rotation, the one the attention kernel's results are defined by."""
         assert self._calibrated, "calibrate() must be called before baking"
         assert kv_head_idx < n_kv_heads
         hd = self.head_dim
         gqa = n_q_heads // n_kv_heads
         assert q_proj_weight.shape[0] == n_q_heads * hd
         hp = self._head_perm.cpu()
-        rot_T = self._block_rot_T.cpu().float()
+        rot = self._block_rot_T.cpu().float().t().contiguous()
         for g in range(gqa):
             lo = (kv_head_idx * gqa + g) * hd
             w = q_proj_weight[lo:lo + hd].detach().clone().cpu()[hp].float()
-            q_proj_weight[lo:lo + hd] = (rot_T @ w).to(q_proj_weight.dtype).to(q_proj_weight.device)
+            q_proj_weight[lo:lo + hd] = (rot @ w).to(q_proj_weight.dtype).to(q_proj_weight.device)
             if q_proj_bias is not None:
                 bvec = q_proj_bias[lo:lo + hd].detach().clone().cpu()[hp].float()
-                q_proj_bias[lo:lo + hd] = (rot_T @ bvec).to(q_proj_bias.dtype).to(q_proj_bias.device)
+                q_proj_bias[lo:lo + hd] = (rot @ bvec).to(q_proj_bias.dtype).to(q_proj_bias.device)
         self._q_perm_baked = True
 
     # -------------------------------------------------------------- K side

@@ -636,3 +636,44 @@ def test_manager_with_rotated_queries_equals_manager_that_rotates_them():
             assert torch.equal(a._k_packed[li], b._k_packed[li]) and torch.equal(a._v_packed[li], b._v_packed[li])
             assert torch.equal(a._k_norms[li], b._k_norms[li]) and torch.equal(a._v_norms[li], b._v_norms[li])
         a.increment_seq_len(); b.increment_seq_len()
+
+
+def test_manager_with_baked_q_proj_equals_manager_that_rotates_queries():
+    """bake_q_permutations folds permutation + rotation into q_proj.  A manager whose model went
+    through it, fed the baked projection's output, must fill a byte-identical cache and return the
+    same attention (within 2e-3) as the plain manager fed the original projection's output."""
+    import copy
+    import types
+    w = wl.Workload("t", 2, 16, 2, 2, 300, 1e6, min_bits=1, max_bits=5, seed=101)
+    a, energies = wl.build_manager(w, DEV)
+    b, _ = wl.build_manager(w, DEV)
+    wl.fill_cache(a, w, energies, DEV)
+    wl.fill_cache(b, w, energies, DEV)
+    hid = 96
+    torch.manual_seed(5)
+
+    def fake_model():
+        layers = [types.SimpleNamespace(self_attn=types.SimpleNamespace(
+            q_proj=torch.nn.Linear(hid, w.n_q * 128, bias=(li == 0)).to(DEV))) for li in range(2)]
+        return types.SimpleNamespace(model=types.SimpleNamespace(layers=layers))
+
+    plain = fake_model()
+    baked = copy.deepcopy(plain)
+    b.bake_q_permutations(baked, w.n_kv, w.n_q)
+    assert all(qz._q_perm_baked for li in range(2) for qz in b.quantizers[li])
+    assert not any(qz._q_perm_baked for li in range(2) for qz in a.quantizers[li])
+    g = torch.Generator(device=DEV).manual_seed(17)
+    with torch.no_grad():
+        for step in range(2):
+            for li in range(2):
+                T = a.seq_len
+                x = torch.randn(w.batch, hid, generator=g, device=DEV)
+                k1, v1 = wl.draw_kv(w, energies[li], 1, 41 + li + 7 * step, DEV, pos0=T)
+                qa = plain.model.layers[li].self_attn.q_proj(x).view(w.batch, w.n_q, 1, 128).half()
+                qb = baked.model.layers[li].self_attn.q_proj(x).view(w.batch, w.n_q, 1, 128).half()
+                out_a = a.append_and_attend(li, qa, k1, v1)
+                out_b = b.append_and_attend(li, qb, k1, v1)
+                assert (out_a.float() - out_b.float()).abs().max() < TOL
+                assert torch.equal(a._k_packed[li], b._k_packed[li]) and torch.equal(a._v_packed[li], b._v_packed[li])
+                assert torch.equal(a._k_norms[li], b._k_norms[li]) and torch.equal(a._v_norms[li], b._v_norms[li])
+            a.increment_seq_len(); b.increment_seq_len()

@@ -423,3 +423,36 @@ def test_saved_calibration_rebuilds_identical_plans(tmp_path):
     np.savez(tmp_path / "other.npz", **fields)
     with pytest.raises(ValueError):
         calibration.load_calibration(tmp_path / "other.npz", device='cpu')
+
+
+# ---------------------------------------------------------------- q_proj baking
+@pytest.mark.parametrize("seed,with_bias", [(3, True), (11, False)])
+def test_baked_q_proj_equals_rotation_of_the_projection(oracle_lib, seed, with_bias):
+    """A q_proj with permutation + rotation folded in must produce what the checker's query
+    rotation makes of the original projection's output, to fp32 rounding.  The head has rotated
+    (non-identity, non-symmetric) groups; a transposed rotation misses by O(1)."""
+    n_kv, gqa, hid = 2, 3, 40
+    heads = [make_quantizer(seed=seed + h, head=h)[0] for h in range(n_kv)]
+    assert any(int(q.plan()['seg_identity'][0][g]) == 0 for q in heads for g in range(int(q.plan()['n_seg'][0])))
+    gen = torch.Generator().manual_seed(seed)
+    W = torch.randn(n_kv * gqa * 128, hid, generator=gen)
+    b = torch.randn(n_kv * gqa * 128, generator=gen) if with_bias else None
+    x = torch.randn(5, hid, generator=gen)
+    y = x @ W.T + (b if with_bias else 0.0)                    # original projection, (5, n_q * 128)
+    Wb, bb = W.clone(), (b.clone() if with_bias else None)
+    for h, q in enumerate(heads):
+        q.bake_permutation_into_qproj(Wb, h, n_kv, n_kv * gqa, q_proj_bias=bb)
+        assert q._q_perm_baked
+    yb = x @ Wb.T + (bb if with_bias else 0.0)
+    for h, q in enumerate(heads):
+        rot = q._block_rot_T.double().numpy()
+        hp = q._head_perm.numpy()
+        for g in range(gqa):
+            lo = (h * gqa + g) * 128
+            want = y[:, lo:lo + 128].double().numpy()[:, hp] @ rot       # q[head_perm] @ block_rot_T
+            got = yb[:, lo:lo + 128].double().numpy()
+            assert np.abs(got - want).max() < 2e-4 * max(1.0, np.abs(want).max())
+            # and the checker's rotation of the fp16-rounded projection agrees with both
+            y16 = y[:, lo:lo + 128].half().numpy()
+            ref = oracle_lib.rotate_q(q.plan(), y16).astype(np.float64)
+            assert np.abs(got - ref).max() < 2e-2 * max(1.0, np.abs(want).max())     # fp16 in and out
