@@ -44,12 +44,6 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
-    ap.add_argument("--k-row-bytes", type=int, default=0,
-                    help="force the row width of every layer's K cache (measurement knob: 64 shows the "
-                         "LDS bank collisions the default widths avoid); 0 = the manager's choice")
-    ap.add_argument("--copy-probe-mib", type=int, default=0,
-                    help="also run a device-to-device copy of this many MiB (a kernel of known HBM "
-                         "traffic, to calibrate FETCH_SIZE / WRITE_SIZE counter readings)")
     return ap.parse_args()
 
 
@@ -119,8 +113,6 @@ def main():
 
     t_setup = time.perf_counter()
     mgr, energies = wl.build_manager(w, dev, max_T=w.context + 8, n_layers=L)
-    if args.k_row_bytes:
-        mgr.force_k_row_bytes(args.k_row_bytes)
     wl.fill_cache(mgr, w, energies, dev)
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t_setup
@@ -141,14 +133,6 @@ def main():
         # append at position T (the same slot every step, so the context stays fixed)
         for li in range(L):
             outs[li] = mgr.append_and_attend(li, qs[li], kvs[li][0], kvs[li][1])
-
-    if args.copy_probe_mib:
-        src = torch.empty(args.copy_probe_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
 
     # --- warm up eagerly, then capture the step once -----------------------
     step()
@@ -258,7 +242,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": (MEASURED_TRAFFIC_BYTES.get(w.name)
-                                 if not (args.context or args.splits or args.k_row_bytes) else None),
+                                 if not (args.context or args.splits) else None),
                      "kernel": "decode attention",
                      "algorithmic_bytes_per_launch": int(alg_bytes),
                      "avg_launch_us": round(attn_us, 3)},

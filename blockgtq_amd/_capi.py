@@ -27,11 +27,11 @@ _SIGNATURES = {
     "bgtq_encode_k": (c_i, [c_p, c_p, c_i64, c_i64, c_i64, c_i, c_i, c_i,
                             c_p, c_i64, c_i64, c_i64, c_i,
                             c_p, c_i64, c_i64, c_i64, c_i,
-                            c_p, c_i, c_i, c_i, c_p]),
+                            c_p, c_i, c_i, c_i, c_i, c_p]),
     "bgtq_encode_v": (c_i, [c_p, c_p, c_i64, c_i64, c_i64, c_i, c_i, c_i,
                             c_p, c_i64, c_i64, c_i64, c_i,
                             c_p, c_i64, c_i64, c_i64,
-                            c_p, c_i, c_i, c_p]),
+                            c_p, c_i, c_i, c_i, c_p]),
     "bgtq_compress_k_codes": (c_i, [c_p, c_p, c_i64, c_p, c_p, c_i, c_i, c_i, c_p]),
     "bgtq_compress_v_codes": (c_i, [c_p, c_p, c_i64, c_p, c_p, c_p]),
     "bgtq_rotate_q": (c_i, [c_p, c_p, c_i64, c_i64, c_p, c_i64, c_i64, c_i, c_i, c_i, c_p]),
@@ -40,7 +40,7 @@ _SIGNATURES = {
                                   c_p, c_i64, c_i64, c_i64, c_i,
                                   c_p, c_i64, c_i64, c_i64, c_i,
                                   c_p, c_i64, c_i64, c_i64,
-                                  c_p, c_i, c_i, c_i, c_i,
+                                  c_p, c_i, c_i, c_i, c_i, c_i,
                                   c_p, c_i64, c_i64, c_p, c_i64, c_i64, c_i, c_p]),
     "bgtq_set_decode_path": (c_i, [c_i]),
     "bgtq_workspace_bytes": (ctypes.c_size_t, [c_i, c_i, c_i]),

@@ -408,12 +408,6 @@ __global__ __launch_bounds__(WT) void window_attn_generic_kernel(
 }
 
 
-#ifdef BGTQ_TRACE
-__device__ unsigned long long* g_wtrace;
-#define WTR(slot) do { if (threadIdx.x == 0 && g_wtrace) g_wtrace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (slot)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define WTR(slot) do {} while (0)
-#endif
 // The same partial for buffers whose rows start on 16-byte boundaries (the manager's do): one
 // work-group per (batch row, KV head) serves all its query heads, HG at a time, so the window is
 // read once per HG heads, and every load is contiguous across the wave.  Scores: 16 lanes share a
@@ -444,7 +438,6 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
     const uint16_t* kb = kbuf + b * w_sb + h * w_sh;
     const uint16_t* vb = vbuf + b * w_sb + h * w_sh;
     const int sub = lane & 15, tq = lane >> 4;  // scores: dim chunk and token within a wave load
-    WTR(0);
     // Loads run one batch ahead of the arithmetic that uses them (a batch waited for on the spot
     // costs a trip to memory each); small batches in rolled loops measured as fast as large
     // unrolled ones.
@@ -484,7 +477,6 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
         uint32_t vc[PB], vn[PB];
         fetch_k(kc, wave * 4);
         fetch_v(vc, wave);                      // the first value rows do not wait for the scores
-        WTR(1);
 #pragma unroll 1
         for (int t0 = wave * 4; t0 < n; t0 += SB * 4 * NW) {
             fetch_k(kn, t0 + SB * 4 * NW);
@@ -510,9 +502,7 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
 #pragma unroll
             for (int u = 0; u < SB; u++) kc[u] = kn[u];
         }
-        WTR(2);
         __syncthreads();
-        WTR(3);
         // ---- softmax weights: wave w owns heads w, w + 4, ... ----------------------------------
         for (int g = wave; g < ng; g += NW) {
             float mm = -INFINITY;
@@ -528,7 +518,6 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
             if (lane == 0) { red_m[g] = mm; red_l[g] = ll; }
         }
         __syncthreads();
-        WTR(4);
         // ---- values: wave w takes tokens w, w + 4, ...; lane = dims 2 lane, 2 lane + 1 -------
         float o0[HG], o1[HG];
 #pragma unroll
@@ -559,11 +548,9 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
 #pragma unroll
             for (int u = 0; u < PB; u++) vc[u] = vn[u];
         }
-        WTR(5);
 #pragma unroll
         for (int g = 0; g < HG; g++) { osum[wave][g][2 * lane] = o0[g]; osum[wave][g][2 * lane + 1] = o1[g]; }
         __syncthreads();
-        WTR(6);
         for (int i = tid; i < ng * D; i += WT) {
             const int g = i / D, d = i - g * D;
             const float acc = (osum[0][g][d] + osum[1][g][d]) + (osum[2][g][d] + osum[3][g][d]);
@@ -573,7 +560,6 @@ __global__ __launch_bounds__(WT) void window_attn_kernel(
             if (d == 0) part_lse[row] = n > 0 ? mg + __logf(lg) : -INFINITY;
         }
         __syncthreads();                        // wlog, red_* and osum are reused by the next heads
-        WTR(7);
     }
 }
 
@@ -755,10 +741,5 @@ const char* bgtq_strerror(int code) {
     }
 }
 
-#ifdef BGTQ_TRACE
-int bgtq_debug_set_wtrace(void* buf) {
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_wtrace), &buf, sizeof(buf));
-}
-#endif
 
 }  // extern "C"

@@ -22,12 +22,6 @@ namespace {
 constexpr int D = BGTQ_D;
 constexpr int NT = 128;  // threads per work-group
 
-#ifdef BGTQ_TRACE
-__device__ unsigned long long* g_etrace;
-#define ET(slot) do { if (threadIdx.x == 0 && g_etrace) g_etrace[(size_t)blockIdx.x * 16 + (slot)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define ET(slot) do {} while (0)
-#endif
 
 struct EncodeArgs {
     const bgtq_head_plan* plans;
@@ -42,6 +36,7 @@ struct EncodeArgs {
     int norm_width;
     const int32_t* t_pos;
     int t_pos_scalar;
+    int max_T;                  // token capacity of the cache: records at positions outside [0, max_T) are dropped
     int layout;
     int quant_mode;
     uint8_t* codes_out;         // [N][128] unpacked codes, or nullptr
@@ -161,7 +156,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     __shared__ typename std::conditional<IS_V, StagedV, StagedK>::type sp;
 
     const int j = threadIdx.x;
-    ET(0);
     const bgtq_head_plan& P = a.plans[h];
     const int64_t N = (int64_t)a.B * a.S;
     const float* RT = IS_V ? P.v_rot_T : P.k_rot_T;
@@ -223,7 +217,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
     __syncthreads();
 
-    ET(1);
     // ---- per-thread static data -------------------------------------------
     int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
     float lut_off_j = 0.f, lut_scale_j = 0.f;          // K: this dim's cell-search parameters
@@ -281,7 +274,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xraw[r][src_dim]);
     __syncthreads();
 
-    ET(2);
     // ---- 2. group norms: thread (r, grp) runs one sequential chain ---------
     if (j < ROWS * BGTQ_MAX_SEGMENTS) {
         int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
@@ -302,7 +294,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
     __syncthreads();
 
-    ET(3);
     // ---- 3. normalise -------------------------------------------------------
     float xh[ROWS];
 #pragma unroll
@@ -319,7 +310,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     if constexpr (STAGED) park_rotation(rot_s, j, rst);   // (every tile of the walk: the registers stay as they are)
     __syncthreads();
 
-    ET(4);
     // ---- 4. rotate ------------------------------------------------------------
     // Same chain as written in the contract above; the matrix column is fetched in
     // batches of RB independent loads so the chain never waits on one load at a time.
@@ -414,7 +404,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
 
-    ET(5);
     // ---- 5. scalar quantise ---------------------------------------------------
     const bool need_cent = IS_V || a.layout == BGTQ_K_MIXED || a.corrected;
 #pragma unroll
@@ -457,7 +446,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
     __syncthreads();
 
-    ET(6);
     // ---- 6. norms to store (raw or divided by ||centroids[codes]||) ---------
     if (j < ROWS * BGTQ_MAX_SEGMENTS) {
         int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
@@ -485,7 +473,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
     __syncthreads();
 
-    ET(7);
     // ---- 7a. unpacked outputs (codes path) ------------------------------------
     if (a.codes_out) {
 #pragma unroll
@@ -512,7 +499,8 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             int b, s;
             split_row(n, a.S, b, s);
             int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
-            a.norms[b * a.n_sb + h * a.n_sh + t * a.n_st + gg] = bgtq_f2h(nrm_out[r][gg]);
+            if (t >= 0 && t < a.max_T)
+                a.norms[b * a.n_sb + h * a.n_sh + t * a.n_st + gg] = bgtq_f2h(nrm_out[r][gg]);
         }
     }
 
@@ -525,6 +513,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             int b, s;
             split_row(n, a.S, b, s);
             int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            if (t < 0 || t >= a.max_T) continue;
             unsigned v = 0;
             if (mode == 1)      v = ROWS == 2 ? stream_byte_batched(&cds[r][c0], slot, bw) : stream_byte(&cds[r][c0], slot, bw);
             else if (mode == 2) v = cds[r][c0];
@@ -532,7 +521,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
     __syncthreads();            // the tile buffers are rewritten by the next tile
-    ET(8);
     }
 }
 
@@ -592,7 +580,6 @@ __device__ __forceinline__ void rotate_q_group(const RotQArgs& a, const int64_t 
     __shared__ uint16_t qraw[QG][D];
     __shared__ float xs[QG][D];
     const int j = threadIdx.x;
-    ET(0);
     const bgtq_head_plan& P = a.plans[h];
     rot_piece rst[D / 4];
     fetch_rotation(P.k_rot_T, j, rst);
@@ -613,7 +600,6 @@ __device__ __forceinline__ void rotate_q_group(const RotQArgs& a, const int64_t 
 #pragma unroll
     for (int r = 0; r < QG; r++) xs[r][j] = bgtq_h2f(qraw[r][src]);
     __syncthreads();
-    ET(1);
     float acc[QG];
 #pragma unroll
     for (int r = 0; r < QG; r++) acc[r] = 0.f;
@@ -646,7 +632,6 @@ __device__ __forceinline__ void rotate_q_group(const RotQArgs& a, const int64_t 
     for (int r = 0; r < QG; r++)
         if (h_first + r < gqa)
             a.q_rot[row * a.qr_sr + (int64_t)(h * gqa + h_first + r) * a.qr_sh + j] = bgtq_f2h(acc[r]);
-    ET(8);
 }
 
 // Work-group `bid` of the query part: a.group heads of one (row, KV head).  One head per
@@ -692,13 +677,16 @@ int fill_k_args(EncodeArgs& a, const bgtq_head_plan* plans,
                 const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss, int B, int n_kv, int S,
                 void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
                 void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
-                const int32_t* t_pos, int t_pos_scalar, int k_layout, int quant_mode) {
+                const int32_t* t_pos, int t_pos_scalar, int max_T, int k_layout, int quant_mode) {
     BGTQ_CHECK_ARG(plans && k && k_packed && k_norms);
     BGTQ_CHECK_ARG(k_row_width >= 0 && k_row_width <= NT);
     BGTQ_CHECK_ARG(norm_width >= 0 && norm_width <= BGTQ_MAX_SEGMENTS);
     BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
     BGTQ_CHECK_ARG(quant_mode == BGTQ_QUANT_LUT256 || quant_mode == BGTQ_QUANT_EXACT);
     BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
+    BGTQ_CHECK_ARG(max_T >= 0);
+    if (!t_pos && (int64_t)t_pos_scalar + S > max_T) return BGTQ_ELIMIT;   // would run past the cache
+    a.max_T = max_T;
     a.plans = plans; a.x = (const uint16_t*)k; a.x_sb = k_sb; a.x_sh = k_sh; a.x_ss = k_ss;
     a.B = B; a.n_kv = n_kv; a.S = S;
     a.packed = (uint8_t*)k_packed; a.p_sb = kp_sb; a.p_sh = kp_sh; a.p_st = kp_st;
@@ -714,11 +702,14 @@ int fill_v_args(EncodeArgs& a, const bgtq_head_plan* plans,
                 const void* v, int64_t v_sb, int64_t v_sh, int64_t v_ss, int B, int n_kv, int S,
                 void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
                 void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
-                const int32_t* t_pos, int t_pos_scalar, int v_layout) {
+                const int32_t* t_pos, int t_pos_scalar, int max_T, int v_layout) {
     BGTQ_CHECK_ARG(plans && v && v_packed && v_norms);
     BGTQ_CHECK_ARG(v_row_width >= 0 && v_row_width <= NT);
     BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
     BGTQ_CHECK_ARG(t_pos || t_pos_scalar >= 0);
+    BGTQ_CHECK_ARG(max_T >= 0);
+    if (!t_pos && (int64_t)t_pos_scalar + S > max_T) return BGTQ_ELIMIT;
+    a.max_T = max_T;
     a.plans = plans; a.x = (const uint16_t*)v; a.x_sb = v_sb; a.x_sh = v_sh; a.x_ss = v_ss;
     a.B = B; a.n_kv = n_kv; a.S = S;
     a.packed = (uint8_t*)v_packed; a.p_sb = vp_sb; a.p_sh = vp_sh; a.p_st = vp_st;
@@ -739,13 +730,13 @@ int bgtq_encode_k(const bgtq_head_plan* plans,
                   int B, int n_kv, int S,
                   void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
                   void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
-                  const int32_t* t_pos, int t_pos_scalar,
+                  const int32_t* t_pos, int t_pos_scalar, int max_T,
                   int k_layout, int quant_mode, void* stream) {
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
     if (B == 0 || n_kv == 0 || S == 0) return BGTQ_OK;     // nothing to encode
     EncodeArgs a{};
     int rc = fill_k_args(a, plans, k, k_sb, k_sh, k_ss, B, n_kv, S, k_packed, kp_sb, kp_sh, kp_st, k_row_width,
-                         k_norms, kn_sb, kn_sh, kn_st, norm_width, t_pos, t_pos_scalar, k_layout, quant_mode);
+                         k_norms, kn_sb, kn_sh, kn_st, norm_width, t_pos, t_pos_scalar, max_T, k_layout, quant_mode);
     if (rc != BGTQ_OK) return rc;
     return launch_encode<false>(a, (hipStream_t)stream);
 }
@@ -755,13 +746,13 @@ int bgtq_encode_v(const bgtq_head_plan* plans,
                   int B, int n_kv, int S,
                   void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
                   void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
-                  const int32_t* t_pos, int t_pos_scalar,
+                  const int32_t* t_pos, int t_pos_scalar, int max_T,
                   int v_layout, void* stream) {
     BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && S >= 0);
     if (B == 0 || n_kv == 0 || S == 0) return BGTQ_OK;
     EncodeArgs a{};
     int rc = fill_v_args(a, plans, v, v_sb, v_sh, v_ss, B, n_kv, S, v_packed, vp_sb, vp_sh, vp_st, v_row_width,
-                         v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, v_layout);
+                         v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, max_T, v_layout);
     if (rc != BGTQ_OK) return rc;
     return launch_encode<true>(a, (hipStream_t)stream);
 }
@@ -814,7 +805,7 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
                         void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
                         void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
                         void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
-                        const int32_t* t_pos, int t_pos_scalar,
+                        const int32_t* t_pos, int t_pos_scalar, int max_T,
                         int k_layout, int v_layout, int quant_mode,
                         const void* q, int64_t q_sr, int64_t q_sh,
                         void* q_rot, int64_t qr_sr, int64_t qr_sh, int gqa, void* stream) {
@@ -822,10 +813,10 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
     if (B == 0 || n_kv == 0) return BGTQ_OK;
     EncodeArgs ak{}, av{};
     int rc = fill_k_args(ak, plans, k, k_sb, k_sh, k_ss, B, n_kv, S, k_packed, kp_sb, kp_sh, kp_st, k_row_width,
-                         k_norms, kn_sb, kn_sh, kn_st, norm_width, t_pos, t_pos_scalar, k_layout, quant_mode);
+                         k_norms, kn_sb, kn_sh, kn_st, norm_width, t_pos, t_pos_scalar, max_T, k_layout, quant_mode);
     if (rc != BGTQ_OK) return rc;
     rc = fill_v_args(av, plans, v, v_sb, v_sh, v_ss, B, n_kv, S, v_packed, vp_sb, vp_sh, vp_st, v_row_width,
-                     v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, v_layout);
+                     v_norms, vn_sb, vn_sh, vn_st, t_pos, t_pos_scalar, max_T, v_layout);
     if (rc != BGTQ_OK) return rc;
     BGTQ_CHECK_ARG((q == nullptr) == (q_rot == nullptr));     // both, or neither (queries rotated elsewhere)
     const bool with_q = q != nullptr;
@@ -845,10 +836,5 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
     return bgtq_launch_status();
 }
 
-#ifdef BGTQ_TRACE
-int bgtq_debug_set_etrace(void* buf) {
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_etrace), &buf, sizeof(buf));
-}
-#endif
 
 }  // extern "C"

@@ -144,6 +144,8 @@ def decode_prepare(plans: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q: tor
         tp, ts = _capi.ptr(t_pos), 0
     else:
         tp, ts = None, int(t_pos)
+    from .quantizer import _cache_capacity
+    max_T = _cache_capacity(t_pos, S, k_packed, k_norms, v_packed, v_norms)
     L = _capi.lib()
     _capi.check(L.bgtq_decode_prepare(
         _capi.ptr(plans), _capi.ptr(k), k.stride(0), k.stride(1), k.stride(2),
@@ -152,7 +154,7 @@ def decode_prepare(plans: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q: tor
         _capi.ptr(k_norms), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2), norm_width,
         _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), v_row_width,
         _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
-        tp, ts, k_layout, v_layout, quant_mode,
+        tp, ts, max_T, k_layout, v_layout, quant_mode,
         _capi.ptr(q), q.stride(0) if q is not None else 0, q.stride(1) if q is not None else 0,
         _capi.ptr(q_rot), q_rot.stride(0) if q is not None else 0, q_rot.stride(1) if q is not None else 0,
         n_q // n_kv, _capi.stream_ptr(k.device)), "bgtq_decode_prepare")

@@ -111,8 +111,6 @@ class BlockGTQKVManager:
         # every layer's K cache has its own row width (the widest record of that layer)
         self._k_rows = [_plan.cache_row_bytes(max(ba['max_tpb'], 1) if ba is not None else self._max_k_packed_bytes)
                         for ba in self._batched_args]
-        if getattr(self, '_forced_k_row', 0):
-            self._k_rows = [self._forced_k_row] * self.n_layers
         self._k_row = max(self._k_rows)
         self._vpb = packed_v_bytes(self.hd, self.v_bits)
         ng = max(self._max_n_groups, 1)
@@ -127,14 +125,6 @@ class BlockGTQKVManager:
             bshape = (self.n_layers, self.B, self.n_kv, self.n_sink + self.window, self.hd)
             self._buf_k = torch.zeros(bshape, dtype=torch.float16, device=dev)
             self._buf_v = torch.zeros(bshape, dtype=torch.float16, device=dev)
-
-    def force_k_row_bytes(self, row_bytes: int):
-        """Use ``row_bytes`` as the K row width of every layer instead of the
-        widths ``_ensure_storage`` would choose (measurement knob; call before the
-        first append).  Must hold the widest record and be a multiple of 4."""
-        assert self._k_packed is None, "storage is already allocated"
-        assert row_bytes % 4 == 0 and row_bytes >= self._max_k_packed_bytes
-        self._forced_k_row = int(row_bytes)
 
     def set_seq_lens(self, seq_lens):
         """Per-row visible lengths (ragged batch); ``None`` returns to one shared length."""
@@ -169,12 +159,13 @@ class BlockGTQKVManager:
                       self._vpb, _plan.V_BITPACKED)
 
     def init_from_cache(self, past_key_value):
-        """Pack an fp16 prefill cache (``.key_cache[li]`` / ``.value_cache[li]``,
-        each (B, n_kv, T, D))."""
+        """Pack an fp16 prefill cache: K, V (B, n_kv, T, D) per layer, read from
+        ``.key_cache[li]`` / ``.value_cache[li]`` (blockgtq/packed_kv_manager.py:259) or,
+        for a ``DynamicCache`` that no longer has those lists, from ``.layers[li].keys / .values``."""
+        from .production_decode import _layer_kv
         T = 0
         for li in range(self.n_layers):
-            k = past_key_value.key_cache[li]
-            v = past_key_value.value_cache[li]
+            k, v = _layer_kv(past_key_value, li)
             T = k.shape[2]
             self._encode_kv(li, k, v, 0)
         self.seq_len = T

@@ -382,6 +382,17 @@ def _t_pos_args(t_pos):
     return None, int(t_pos)
 
 
+def _cache_capacity(t_pos, S: int, *cache_tensors) -> int:
+    """Token capacity of the cache views an append writes to (their common size along the
+    token axis).  A host position that would run past it raises here, before any launch, as the
+    reference's slice assignment would; device positions are bounded by the kernels, which drop
+    records outside the capacity."""
+    max_T = min(int(t.shape[2]) for t in cache_tensors)
+    if not isinstance(t_pos, torch.Tensor) and int(t_pos) + int(S) > max_T:
+        raise ValueError(f"append of {S} token(s) at position {int(t_pos)} exceeds the cache capacity {max_T}")
+    return max_T
+
+
 def encode_k_into(plans: torch.Tensor, k: torch.Tensor, k_packed: torch.Tensor,
                   k_norms: torch.Tensor, t_pos, row_width: int, norm_width: int,
                   k_layout: int, quant_mode: int = _plan.QUANT_LUT256):
@@ -394,12 +405,13 @@ def encode_k_into(plans: torch.Tensor, k: torch.Tensor, k_packed: torch.Tensor,
     assert k_norms.dtype == torch.float16 and k_norms.stride(-1) == 1
     B, H, S, _ = k.shape
     tp, ts = _t_pos_args(t_pos)
+    max_T = _cache_capacity(t_pos, S, k_packed, k_norms)
     L = _capi.lib()
     _capi.check(L.bgtq_encode_k(
         _capi.ptr(plans), _capi.ptr(k), k.stride(0), k.stride(1), k.stride(2), B, H, S,
         _capi.ptr(k_packed), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2), row_width,
         _capi.ptr(k_norms), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2), norm_width,
-        tp, ts, k_layout, quant_mode, _capi.stream_ptr(k.device)), "bgtq_encode_k")
+        tp, ts, max_T, k_layout, quant_mode, _capi.stream_ptr(k.device)), "bgtq_encode_k")
 
 
 def encode_v_into(plans: torch.Tensor, v: torch.Tensor, v_packed: torch.Tensor,
@@ -412,12 +424,13 @@ def encode_v_into(plans: torch.Tensor, v: torch.Tensor, v_packed: torch.Tensor,
     assert v_norms.dtype == torch.float16
     B, H, S, _ = v.shape
     tp, ts = _t_pos_args(t_pos)
+    max_T = _cache_capacity(t_pos, S, v_packed, v_norms)
     L = _capi.lib()
     _capi.check(L.bgtq_encode_v(
         _capi.ptr(plans), _capi.ptr(v), v.stride(0), v.stride(1), v.stride(2), B, H, S,
         _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), row_width,
         _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
-        tp, ts, v_layout, _capi.stream_ptr(v.device)), "bgtq_encode_v")
+        tp, ts, max_T, v_layout, _capi.stream_ptr(v.device)), "bgtq_encode_v")
 
 
 # ===========================================================================

@@ -203,13 +203,19 @@ const char* bgtq_strerror(int code);
  *              bytes beyond the head's own record up to k_row_width are zeroed
  *   k_norms    fp16 [B][n_kv][T][norm_width], strides in halves; entries beyond the
  *              head's own n_seg up to norm_width are zeroed
+ *   max_T      token capacity of the cache tensors.  With a host position the call is
+ *              refused (BGTQ_ELIMIT) when t_pos_scalar + S > max_T, before anything is
+ *              launched; with device positions a record whose position falls outside
+ *              [0, max_T) is dropped by the kernel, so an append past the end never
+ *              writes outside the cache (the reference's slice assignment raises there,
+ *              blockgtq/packed_kv_manager.py:172-178)
  */
 int bgtq_encode_k(const bgtq_head_plan* plans,
                   const void* k, int64_t k_sb, int64_t k_sh, int64_t k_ss,
                   int B, int n_kv, int S,
                   void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
                   void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
-                  const int32_t* t_pos, int t_pos_scalar,
+                  const int32_t* t_pos, int t_pos_scalar, int max_T,
                   int k_layout, int quant_mode, void* stream);
 
 /*
@@ -224,7 +230,7 @@ int bgtq_encode_v(const bgtq_head_plan* plans,
                   int B, int n_kv, int S,
                   void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
                   void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
-                  const int32_t* t_pos, int t_pos_scalar,
+                  const int32_t* t_pos, int t_pos_scalar, int max_T,
                   int v_layout, void* stream);
 
 /*
@@ -278,7 +284,7 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
                         void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st, int norm_width,
                         void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
                         void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
-                        const int32_t* t_pos, int t_pos_scalar,
+                        const int32_t* t_pos, int t_pos_scalar, int max_T,
                         int k_layout, int v_layout, int quant_mode,
                         const void* q, int64_t q_sr, int64_t q_sh,
                         void* q_rot, int64_t qr_sr, int64_t qr_sh, int gqa, void* stream);

@@ -223,3 +223,51 @@ def test_fused_prepare_equals_the_three_separate_calls(S):
         assert torch.equal(a, b)
     assert torch.equal(kn0.view(torch.int16), kn1.view(torch.int16))
     assert torch.equal(vn0.view(torch.int16), vn1.view(torch.int16))
+
+
+def test_appends_past_the_cache_capacity_write_nothing(oracle_lib):
+    """A host position beyond the capacity raises before any launch; device positions beyond it
+    are dropped by the kernels (both append sizes: the 2-row decode tiles and the 16-row tiles,
+    and the fused prepare launch), and rows inside the capacity are still written correctly.
+    The cache tensors are views into a larger buffer so that a stray write would be seen."""
+    from blockgtq_amd import ops
+    from blockgtq_amd.quantizer import build_batched_encode_args, encode_k_into, encode_v_into
+    qs, ens = zip(*[make_quantizer(seed=50 + h, head=h, device=DEV) for h in range(2)])
+    args = build_batched_encode_args(list(qs), device=DEV)
+    kw, ng, H, cap = (args['max_tpb'] + 3) // 4 * 4, args['max_n_groups'], 2, 12
+    for B, S in ((3, 1), (3, 30)):                       # decode-sized and prefill-sized launches
+        big_k = torch.full((B, H, cap + 40, kw), 0xEE, dtype=torch.uint8, device=DEV)
+        big_n = torch.full((B, H, cap + 40, ng), 5.0, dtype=torch.float16, device=DEV)
+        big_v = torch.full((B, H, cap + 40, 48), 0xEE, dtype=torch.uint8, device=DEV)
+        big_vn = torch.full((B, H, cap + 40), 5.0, dtype=torch.float16, device=DEV)
+        kp, kn, vp, vn = big_k[:, :, :cap], big_n[:, :, :cap], big_v[:, :, :cap], big_vn[:, :, :cap]
+        gen = torch.Generator().manual_seed(S)
+        k = torch.randn(B, H, S, 128, generator=gen).half().to(DEV)
+        v = torch.randn(B, H, S, 128, generator=gen).half().to(DEV)
+        q = torch.randn(B, H * 4, 128, generator=gen).half().to(DEV)
+        with pytest.raises(ValueError):
+            encode_k_into(args['plans'], k, kp, kn, cap - S + 1, kw, ng, 0)
+        with pytest.raises(ValueError):
+            ops.decode_prepare(args['plans'], k, v, q, kp, kn, vp, vn, cap, kw, ng, 48, H, 0, 0)
+        pos = torch.tensor([cap - S - 1 if S < cap else 0, cap - 1, cap + 5], dtype=torch.int32, device=DEV)
+        for fused in (False, True):
+            big_k.fill_(0xEE); big_n.fill_(5.0); big_v.fill_(0xEE); big_vn.fill_(5.0)
+            if fused:
+                ops.decode_prepare(args['plans'], k, v, q, kp, kn, vp, vn, pos, kw, ng, 48, H, 0, 0)
+            else:
+                encode_k_into(args['plans'], k, kp, kn, pos, kw, ng, 0)
+                encode_v_into(args['plans'], v, vp, vn, pos, 48, 0)
+            torch.cuda.synchronize()
+            assert (big_k[:, :, cap:] == 0xEE).all() and (big_v[:, :, cap:] == 0xEE).all()
+            assert (big_n[:, :, cap:] == 5.0).all() and (big_vn[:, :, cap:] == 5.0).all()
+            for b in range(B):
+                t0 = int(pos[b])
+                n_in = max(0, min(S, cap - t0))           # rows of this batch row that fit
+                for h in range(H):
+                    pl = args['plans_np'][h:h + 1]
+                    codes, raw, _ = oracle_lib.encode_k(pl, k[b, h].cpu().numpy())
+                    want = oracle_lib.pack_k(pl, codes, 0, kw)
+                    assert np.array_equal(kp[b, h, t0:t0 + n_in].cpu().numpy(), want[:n_in])
+                    vc, wn = oracle_lib.encode_v(pl, v[b, h].cpu().numpy())
+                    assert np.array_equal(vp[b, h, t0:t0 + n_in].cpu().numpy(), oracle_lib.pack_v(vc, 3)[:n_in])
+                    assert (kp[b, h, :min(t0, cap)] == 0xEE).all()

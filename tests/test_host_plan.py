@@ -1,4 +1,5 @@
 """Host-side plan builders against closed forms, invariants and brute force."""
+import ctypes
 import itertools
 import math
 import re
@@ -385,10 +386,14 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert lib.bgtq_strerror(-1).decode() == "invalid argument"
     # argument validation happens on the host before any launch
     assert lib.bgtq_encode_k(None, None, 0, 0, 0, 1, 1, 1, None, 0, 0, 0, 8,
-                             None, 0, 0, 0, 1, None, 0, 0, 0, None) == -1
+                             None, 0, 0, 0, 1, None, 0, 4, 0, 0, None) == -1
     # an empty call is legal and launches nothing
     assert lib.bgtq_encode_k(None, None, 0, 0, 0, 1, 1, 0, None, 0, 0, 0, 8,
-                             None, 0, 0, 0, 1, None, 0, 0, 0, None) == 0
+                             None, 0, 0, 0, 1, None, 0, 4, 0, 0, None) == 0
+    # an append that would run past the cache capacity is refused before any launch
+    one = ctypes.c_void_p(16)          # non-null placeholders: the capacity check comes before any use
+    assert lib.bgtq_encode_k(one, one, 0, 0, 0, 1, 1, 2, one, 0, 0, 0, 8,
+                             one, 0, 0, 0, 1, None, 3, 4, 0, 0, None) == -3
 
 
 def test_device_paths_refuse_cpu_tensors():
