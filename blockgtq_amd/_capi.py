@@ -52,6 +52,13 @@ _SIGNATURES = {
                                c_p, c_i64, c_i64, c_i64,
                                c_p, c_i, c_i, c_i, c_i, c_i,
                                c_p, c_p, c_i, c_i, c_f, c_p]),
+    "bgtq_decode_attend_static": (c_i, [c_p, c_p, c_i64, c_i64,
+                                        c_p, c_i64, c_i64, c_i64, c_i,
+                                        c_p, c_i64, c_i64, c_i64,
+                                        c_p, c_i64, c_i64, c_i64, c_i,
+                                        c_p, c_i64, c_i64, c_i64,
+                                        c_p, c_i, c_i, c_i, c_i, c_i,
+                                        c_i, c_i, c_f, c_i, c_p, c_i64, c_i64, c_p, c_p]),
     "bgtq_window_attn": (c_i, [c_p, c_i64, c_i64, c_p, c_p, c_i64, c_i64, c_i64, c_p, c_i,
                                c_i, c_i, c_i, c_f, c_p, c_p, c_p]),
     "bgtq_window_swap": (c_i, [c_p, c_p, c_i64, c_i64, c_i64, c_p, c_p, c_i64, c_i64, c_p, c_i, c_i, c_i,

@@ -11,6 +11,8 @@
 // work-group, and thread (d, half) accumulates output dim d for one half of
 // the query heads over the tile's tokens.
 #include "bgtq_common.h"
+#include <mutex>
+
 #include "bgtq_decode.h"
 
 namespace {
@@ -587,6 +589,38 @@ __global__ __launch_bounds__(D) void window_swap_kernel(
 
 static int g_decode_path = 0;
 
+// ---- partition results of bgtq_decode_attend_static ------------------------------------------
+// The partial vectors and log-sum-exps of the entry point that allocates nothing live in
+// this array: one copy per GPU the library runs on, held until the process ends.  Host code
+// never uses the array's name as an address; it asks the runtime once per device for the
+// device address of that GPU's copy and passes that to the kernels.
+static __device__ __align__(256) unsigned char scratch[BGTQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES];        // device address of `scratch` on device i, once known
+
+// Device address of the current device's scratch array (asked for on the first call on
+// that device, with that device current).
+int scratch_of_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return BGTQ_ELIMIT;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return BGTQ_EINVAL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return BGTQ_OK;
+}
+}  // namespace
+
 extern "C" {
 
 int bgtq_set_decode_path(int path) {
@@ -676,6 +710,37 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
                        n_extra ? extra_out : nullptr, n_extra ? extra_lse : nullptr, n_extra,
                        n_kv * gqa, gqa, unrotate, (uint16_t*)out, o_sb, o_sh, lse_out);
     return bgtq_launch_status();
+}
+
+int bgtq_decode_attend_static(const bgtq_head_plan* plans,
+                              const void* q_rot, int64_t q_sb, int64_t q_sh,
+                              const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                              const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                              const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                              const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                              const int32_t* seq_lens, int T,
+                              int B, int n_kv, int gqa, int n_splits,
+                              int k_layout, int v_layout, float scale, int unrotate,
+                              void* out, int64_t o_sb, int64_t o_sh, float* lse_out, void* stream) {
+    BGTQ_CHECK_ARG(out);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv >= 0 && gqa >= 1 && gqa <= BGTQ_MAX_GQA);
+    if (n_splits <= 0) n_splits = bgtq_default_splits(B, n_kv, T > 0 ? T : 1);
+    if (n_splits > BGTQ_MAX_SPLITS) return BGTQ_ELIMIT;
+    if (B == 0 || n_kv == 0) return BGTQ_OK;
+    const size_t rows = (size_t)B * n_kv * gqa * n_splits;         // (batch row, query head, partition)
+    if (bgtq_workspace_bytes(B, n_kv * gqa, n_splits) > (size_t)BGTQ_STATIC_SCRATCH_BYTES) return BGTQ_ELIMIT;
+    void* base = nullptr;
+    int rc = scratch_of_current_device(&base);
+    if (rc != BGTQ_OK) return rc;
+    float* part_out = (float*)base;                                 // [rows][128], 16-byte aligned
+    float* part_lse = part_out + rows * D;                          // [rows]
+    rc = bgtq_decode_attn(plans, q_rot, q_sb, q_sh, k_packed, kp_sb, kp_sh, kp_st, k_row_width,
+                          k_norms, kn_sb, kn_sh, kn_st, v_packed, vp_sb, vp_sh, vp_st, v_row_width,
+                          v_norms, vn_sb, vn_sh, vn_st, seq_lens, T, B, n_kv, gqa, n_splits,
+                          part_out, part_lse, k_layout, v_layout, scale, stream);
+    if (rc != BGTQ_OK) return rc;
+    return bgtq_lse_reduce(plans, part_out, part_lse, n_splits, nullptr, nullptr, 0,
+                           B, n_kv, gqa, unrotate, out, o_sb, o_sh, lse_out, stream);
 }
 
 int bgtq_window_attn(const void* q, int64_t q_sb, int64_t q_sh,

@@ -28,6 +28,7 @@ extern "C" {
 #define BGTQ_LUT_BINS      256
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
+#define BGTQ_STATIC_SCRATCH_BYTES (8u << 20)  /* partition results of bgtq_decode_attend_static */
 #define BGTQ_MAX_STEPS     12    /* MFMA steps of one K record, see bgtq_head_plan.step */
 /* byte offsets inside bgtq_head_plan.lut_image (= LDS offsets in the decode kernel) */
 #define BGTQ_LUT_K1      0                       /* 4 entries   x 32 replicas */
@@ -354,6 +355,36 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
                     int B, int n_kv, int gqa, int unrotate,
                     void* out, int64_t o_sb, int64_t o_sh,
                     float* lse_out, void* stream);
+
+/*
+ * Decode attention of one layer, partitions merged, without any allocation:
+ * bgtq_decode_attn followed by bgtq_lse_reduce (no extra partials), with the
+ * partition results kept in a fixed array inside the library instead of a
+ * caller-provided workspace.  This entry point has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory or size a
+ * workspace at call time: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid allocation.  It calls no allocating routine.
+ *
+ *   arguments  as for bgtq_decode_attn (inputs) and bgtq_lse_reduce (unrotate, out,
+ *              o_sb, o_sh, lse_out); n_splits <= 0 picks bgtq_default_splits
+ *   limit      bgtq_workspace_bytes(B, n_kv * gqa, n_splits) must not exceed
+ *              BGTQ_STATIC_SCRATCH_BYTES (8 MiB; BGTQ_ELIMIT otherwise) - e.g.
+ *              B * n_q * n_splits <= 16256
+ * Every GPU the library runs on holds one such array until the process ends, and
+ * every call on a GPU uses that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race and must be serialised by the caller.  Nothing in the
+ * array has to start at zero: each call overwrites every entry it later reads.
+ */
+int bgtq_decode_attend_static(const bgtq_head_plan* plans,
+                              const void* q_rot, int64_t q_sb, int64_t q_sh,
+                              const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                              const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                              const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                              const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                              const int32_t* seq_lens, int T,
+                              int B, int n_kv, int gqa, int n_splits,
+                              int k_layout, int v_layout, float scale, int unrotate,
+                              void* out, int64_t o_sb, int64_t o_sh, float* lse_out, void* stream);
 
 /*
  * Dense fp16 attention partial for the with-buffer setting: sink tokens and a
