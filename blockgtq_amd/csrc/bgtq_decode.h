@@ -2,6 +2,11 @@
 #pragma once
 #include "bgtq_common.h"
 
+// LDS bytes of one wave's tile buffers in the MFMA kernel (filled in by its launcher)
+struct TileLayout {
+    int kt, vt, knr, vnr, kbuf;    // K, V, K-norm, V-norm areas; K + both norm areas
+};
+
 struct DecodeArgs {
     const bgtq_head_plan* plans;
     const uint16_t* q;  int64_t q_sb, q_sh;
@@ -16,6 +21,8 @@ struct DecodeArgs {
     float scale;
     int k_row_width;       // widest K record over the heads (LDS sizing)
     int v_row_width;
+    int nw;                // MFMA kernel: waves per work-group
+    TileLayout tl;
 };
 
 // Fast path: MFMA kernel for bit-packed K and V records (bgtq_decode_mfma.hip).

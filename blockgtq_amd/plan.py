@@ -12,7 +12,7 @@ HEAD_DIM = 128
 MAX_SEGMENTS = 8
 MAX_CENTROIDS = 256
 LUT_BINS = 256
-MAX_STEPS = 12
+MAX_STEPS = 8
 
 K_BITPACKED, K_MIXED = 0, 1
 V_BITPACKED, V_NIBBLE = 0, 1
@@ -36,22 +36,16 @@ PLAN_DTYPE = np.dtype([
     ('v_centroids', '<f4', (16,)), ('v_boundaries', '<f4', (16,)),
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
-    ('n_steps', '<i4'), ('reserved1', '<i4', (3,)), ('step', '<i4', (MAX_STEPS, 8)),
-    ('n_packed_steps', '<i4'), ('reserved2', '<i4', (3,)),
-    ('steptab', '<u4', (MAX_STEPS, 4, 8)), ('qunit_dim', '<i4', (32,)), ('qunit_len', '<i4', (32,)),
-    ('lut_image', '<u4', (29184 // 4,)),
-    ('n_steps_mixed', '<i4'), ('n_packed_steps_mixed', '<i4'), ('reserved3', '<i4', (2,)),
-    ('steptab_mixed', '<u4', (MAX_STEPS, 4, 8)), ('qunit_dim_mixed', '<i4', (32,)),
-    ('qunit_len_mixed', '<i4', (32,)), ('lut_image_mixed', '<u4', (43008 // 4,)),
-    ('n_steps_dense', '<i4'), ('n_packed_steps_dense', '<i4'),
-    ('n_steps_dense_mixed', '<i4'), ('n_packed_steps_dense_mixed', '<i4'),
-    ('steptab_dense', '<u4', (MAX_STEPS, 2, 4, 8)), ('steptab_dense_mixed', '<u4', (MAX_STEPS, 2, 4, 8)),
+    ('n_steps', '<i4', (2,)), ('n_packed_steps', '<i4', (2,)),
+    ('steptab', '<u4', (2, MAX_STEPS, 4, 8)),
+    ('lut_image', '<u4', (2, 13824 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
 ], align=True)
 
-# byte offsets inside lut_image (BGTQ_LUT_* of include/bgtq.h)
+# byte offsets inside lut_image[K_BITPACKED] / lut_image[K_MIXED] (BGTQ_LUT_* / BGTQ_LUTM_* of include/bgtq.h)
 LUT_K = {1: 0, 2: 512, 3: 2560, 4: 10752}
-LUT_KRAW, LUT_V, LUT_IMAGE_BYTES = 18944, 20992, 29184
-LUTM_KRAW, LUTM_V, LUTM_IMAGE_BYTES = 32768, 34816, 43008      # BGTQ_LUTM_*
+LUT_KRAW, LUT_IMAGE_BYTES = 11776, 13824
+LUTM_KRAW = 4096
+VLUT_BYTES = 8192          # the kernel's table area starts with the V table; the K image follows it
 
 
 def segment_bytes(bw: int, length: int) -> int:
@@ -67,175 +61,93 @@ def segment_bytes(bw: int, length: int) -> int:
     return length
 
 
+def _replicas(bw: int) -> int:
+    """Copies of every pair-table entry: 32 (one per lane of a half-wave) for tables of at most
+    64 entries, none for the 256-entry table."""
+    return 32 if bw <= 3 else 1
+
+
 def _pair_table(cb16: np.ndarray, bw: int) -> np.ndarray:
-    """Bank-replicated pair table of one code width: entry (c0 | c1 << bw)."""
+    """Pair table of one code width, entry (c0 | c1 << bw), bank-replicated for bw <= 3."""
     e = np.arange(1 << (2 * bw))
     pairs = cb16[e & ((1 << bw) - 1)].astype(np.uint32) | (cb16[e >> bw].astype(np.uint32) << 16)
-    return np.repeat(pairs, 8 if bw == 4 else 32)
-
-
-def fill_decode_steps(p) -> None:
-    """Derive the MFMA step schedule of the bit-packed K record, its LDS-ready
-    form and the pair tables from the segment table, codebooks and V LUT
-    already stored in plan ``p`` (a 0-d structured array)."""
-    m, n_packed, unit = 0, 0, 1
-    p['step'][...] = 0
-    p['steptab'][...] = 0
-    p['qunit_dim'][...] = 0
-    p['qunit_len'][...] = 0
-    for s in range(int(p['n_seg'])):
-        bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
-        start, end = int(p['seg_start'][s]), int(p['seg_start'][s]) + ln
-        n_units = (ln + 7) // 8
-        unit_bytes = bw if bw <= 4 else 8
-        for u0 in range(0, n_units, 4):
-            if m >= MAX_STEPS:
-                raise ValueError("segment table needs more MFMA steps than the plan holds")
-            nu = min(4, n_units - u0)
-            off0 = int(p['seg_pack_off'][s]) + u0 * unit_bytes
-            p['step'][m] = (off0, unit_bytes, 2 * bw if bw <= 4 else 0, bw, s,
-                            int(u0 + 4 >= n_units), nu, start + u0 * 8)
-            for g in range(4):
-                gg = min(g, nu - 1)
-                table = LUT_K[bw] if bw <= 4 else LUT_KRAW + (bw - 5) * 512
-                mask = 7 * 4 if bw == 4 else (31 * 4 if bw <= 3 else 0)
-                q_off = 0
-                if g < nu:
-                    d0 = start + (u0 + g) * 8
-                    p['qunit_dim'][unit], p['qunit_len'][unit] = d0, min(8, end - d0)
-                    q_off = 16 * unit
-                    unit += 1
-                p['steptab'][m, g] = (off0 + gg * unit_bytes, 0, table, mask,
-                                      2 * bw if bw <= 4 else 0, 5 if bw == 4 else 7, s * 128, q_off)
-            n_packed += bw <= 4
-            m += 1
-    p['n_steps'] = m
-    p['n_packed_steps'] = n_packed
-
-    img = np.zeros(LUT_IMAGE_BYTES // 4, dtype=np.uint32)
-    for s in range(int(p['n_seg'])):
-        bw = int(p['seg_bw'][s])
-        cb = p['k_codebook_f16'][s]
-        if bw <= 4:
-            t = _pair_table(cb, bw)
-            img[LUT_K[bw] // 4:LUT_K[bw] // 4 + t.size] = t
-        else:
-            raw = np.zeros(256, dtype=np.uint16)
-            raw[:1 << bw] = cb[:1 << bw]
-            o = (LUT_KRAW + (bw - 5) * 512) // 4
-            img[o:o + 128] = raw.view(np.uint32)
-    vb = int(p['v_bits'])
-    if 1 <= vb <= 4:
-        t = _pair_table(p['v_lut_f16'], vb)
-        img[LUT_V // 4:LUT_V // 4 + t.size] = t
-    p['lut_image'] = img
-    _fill_dense(p, '')
-    _fill_mixed_tables(p)
-
-
-def _fill_dense(p, suffix: str) -> None:
-    """Two-segment schedule for query groups of at most 8 heads, derived from the
-    one-segment schedule ``steptab<suffix>``: the packed units keep their order and
-    their table entries, but a step takes the next four of them as long as they
-    belong to at most two segments; the first segment of a step owns column half
-    0, the second half 1.  Raw-byte steps follow unchanged (half 1 all zero)."""
-    tab = p['steptab' + suffix]
-    n_steps, n_packed = int(p['n_steps' + suffix]), int(p['n_packed_steps' + suffix])
-    units = []                                   # table rows of the real packed units, in order
-    for m in range(n_packed):
-        for g in range(4):
-            row = tab[m, g]
-            if int(row[7]) != 0:
-                units.append(row.copy())
-    dense = p['steptab_dense' + suffix]
-    dense[...] = 0
-    m = i = 0
-    while i < len(units):
-        step, segs = [], []
-        while i < len(units) and len(step) < 4:
-            seg = int(units[i][6])
-            if seg not in segs:
-                if len(segs) == 2:
-                    break
-                segs.append(seg)
-            step.append(units[i])
-            i += 1
-        for half in range(2):
-            own = segs[min(half, len(segs) - 1)]
-            for g in range(4):
-                row = step[min(g, len(step) - 1)].copy()
-                mine = g < len(step) and int(row[6]) == own and (half == 0 or len(segs) == 2)
-                row[7] = row[7] if mine else 0
-                row[6] = own
-                dense[m, half, g] = row
-        m += 1
-    n_dense_packed = m
-    for r in range(n_packed, n_steps):           # raw-byte steps: half 0 as it is, half 1 silent
-        if m >= MAX_STEPS:
-            raise ValueError("segment table needs more MFMA steps than the plan holds")
-        dense[m, 0] = tab[r]
-        dense[m, 1] = tab[r]
-        dense[m, 1, :, 7] = 0
-        m += 1
-    p['n_steps_dense' + suffix] = m
-    p['n_packed_steps_dense' + suffix] = n_dense_packed
+    return np.repeat(pairs, _replicas(bw))
 
 
 def _byte_pair_table(cb16: np.ndarray, bw: int) -> np.ndarray:
-    """Pair table indexed by a byte that holds two codes as nibbles (low nibble first)."""
+    """256-entry pair table indexed by a byte that holds two codes as nibbles (low nibble first)."""
     b = np.arange(256)
     lo, hi = b & 15, b >> 4
     ok = (lo < (1 << bw)) & (hi < (1 << bw))
     pairs = cb16[np.where(ok, lo, 0)].astype(np.uint32) | (cb16[np.where(ok, hi, 0)].astype(np.uint32) << 16)
-    return np.repeat(np.where(ok, pairs, 0).astype(np.uint32), 8)
+    return np.where(ok, pairs, 0).astype(np.uint32)
 
 
-def _fill_mixed_tables(p) -> None:
-    """Step schedule, query units and table image of the mixed K / nibble V layouts."""
-    m, n_packed, unit, n_ptab = 0, 0, 1, 0
-    p['steptab_mixed'][...] = 0
-    p['qunit_dim_mixed'][...] = 0
-    p['qunit_len_mixed'][...] = 0
-    img = np.zeros(LUTM_IMAGE_BYTES // 4, dtype=np.uint32)
-    for s in range(int(p['n_seg'])):
-        bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
-        start, end = int(p['seg_start'][s]), int(p['seg_start'][s]) + ln
-        n_units = (ln + 7) // 8
-        unit_bytes = 4 if bw <= 4 else 8
-        cb = p['k_codebook_f16'][s]
-        if bw <= 4:
-            table = n_ptab * 8192                 # at most 4 distinct widths <= 4 bits
-            img[table // 4:table // 4 + 2048] = _byte_pair_table(cb, bw)
-            n_ptab += 1
-        else:
-            table = LUTM_KRAW + (bw - 5) * 512
-            raw = np.zeros(256, dtype=np.uint16)
-            raw[:1 << bw] = cb[:1 << bw]
-            img[table // 4:table // 4 + 128] = raw.view(np.uint32)
-        for u0 in range(0, n_units, 4):
-            if m >= MAX_STEPS:
-                raise ValueError("segment table needs more MFMA steps than the plan holds")
-            nu = min(4, n_units - u0)
-            off0 = int(p['seg_mixed_off'][s]) + u0 * unit_bytes
-            for g in range(4):
-                gg = min(g, nu - 1)
-                q_off = 0
-                if g < nu:
-                    d0 = start + (u0 + g) * 8
-                    p['qunit_dim_mixed'][unit], p['qunit_len_mixed'][unit] = d0, min(8, end - d0)
-                    q_off = 16 * unit
-                    unit += 1
-                p['steptab_mixed'][m, g] = (off0 + gg * unit_bytes, 0, table, 7 * 4 if bw <= 4 else 0,
-                                            8 if bw <= 4 else 0, 5, s * 128, q_off)
-            n_packed += bw <= 4
-            m += 1
-    p['n_steps_mixed'] = m
-    p['n_packed_steps_mixed'] = n_packed
+def _raw_table(cb16: np.ndarray, bw: int) -> np.ndarray:
+    raw = np.zeros(256, dtype=np.uint16)
+    raw[:1 << bw] = cb16[:1 << bw]
+    return raw.view(np.uint32)
+
+
+def fill_decode_steps(p) -> None:
+    """Derive the MFMA step schedules of both K record layouts and the table images from the
+    segment table, codebooks and V LUT already stored in plan ``p`` (a 0-d structured array)."""
+    p['steptab'][...] = 0
+    p['n_steps'][...] = 0
+    p['n_packed_steps'][...] = 0
+    for layout in (K_BITPACKED, K_MIXED):
+        img = np.zeros(LUT_IMAGE_BYTES // 4, dtype=np.uint32)
+        packed, raw = [], []                      # unit rows (the eight words of a steptab entry)
+        n_ptab = 0
+        for s in range(int(p['n_seg'])):
+            bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
+            start = int(p['seg_start'][s])
+            cb = p['k_codebook_f16'][s]
+            if bw <= 4:
+                if layout == K_BITPACKED:
+                    table, unit_bytes, pw = LUT_K[bw], bw, 2 * bw
+                    mask, tsh = (31 * 4, 7) if bw <= 3 else (0, 2)
+                    t = _pair_table(cb, bw)
+                    seg_off = int(p['seg_pack_off'][s])
+                else:
+                    table, unit_bytes, pw, mask, tsh = n_ptab * 1024, 4, 8, 0, 2
+                    t = _byte_pair_table(cb, bw)
+                    seg_off = int(p['seg_mixed_off'][s])
+                    n_ptab += 1
+                img[table // 4:table // 4 + t.size] = t
+            else:
+                table = (LUT_KRAW if layout == K_BITPACKED else LUTM_KRAW) + (bw - 5) * 512
+                unit_bytes, pw, mask, tsh = 8, 0, 0, 1
+                img[table // 4:table // 4 + 128] = _raw_table(cb, bw)
+                seg_off = int(p['seg_pack_off' if layout == K_BITPACKED else 'seg_mixed_off'][s])
+            for u in range((ln + 7) // 8):
+                off = seg_off + u * unit_bytes
+                d0 = start + 8 * u
+                row = (off & ~3, off & 3, VLUT_BYTES + table, mask, pw, tsh, 2 * s, d0 | (min(8, start + ln - d0) << 8))
+                (packed if bw <= 4 else raw).append(row)
+        m = 0
+        for units in (packed, raw):
+            for u0 in range(0, len(units), 4):
+                if m >= MAX_STEPS:
+                    raise ValueError("segment table needs more MFMA steps than the plan holds")
+                for g in range(4):
+                    if u0 + g < len(units):
+                        p['steptab'][layout, m, g] = units[u0 + g]
+                    else:                          # repeat the last unit with an empty query range
+                        row = list(units[-1])
+                        row[7] &= 0xFF
+                        p['steptab'][layout, m, g] = row
+                m += 1
+            if units is packed:
+                p['n_packed_steps'][layout] = m
+        p['n_steps'][layout] = m
+        p['lut_image'][layout] = img
     vb = int(p['v_bits'])
+    p['vlut_image'][...] = 0
     if 1 <= vb <= 4:
-        img[LUTM_V // 4:LUTM_V // 4 + 2048] = _byte_pair_table(p['v_lut_f16'], vb)
-    p['lut_image_mixed'] = img
-    _fill_dense(p, '_mixed')
+        t = _pair_table(p['v_lut_f16'], vb)
+        p['vlut_image'][V_BITPACKED, :t.size] = t
+        p['vlut_image'][V_NIBBLE, :256] = _byte_pair_table(p['v_lut_f16'], vb)
 
 
 def build_head_plan(quantizer) -> np.ndarray:

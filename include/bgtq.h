@@ -29,20 +29,20 @@ extern "C" {
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
 #define BGTQ_STATIC_SCRATCH_BYTES (8u << 20)  /* partition results of bgtq_decode_attend_static */
-#define BGTQ_MAX_STEPS     12    /* MFMA steps of one K record, see bgtq_head_plan.step */
-/* byte offsets inside bgtq_head_plan.lut_image (= LDS offsets in the decode kernel) */
+#define BGTQ_MAX_STEPS     8     /* MFMA steps of one K record, see bgtq_head_plan.steptab */
+/* byte offsets inside bgtq_head_plan.lut_image[BGTQ_K_BITPACKED] (= offsets in the decode kernel's table area) */
 #define BGTQ_LUT_K1      0                       /* 4 entries   x 32 replicas */
 #define BGTQ_LUT_K2      512                     /* 16 entries  x 32 replicas */
 #define BGTQ_LUT_K3      2560                    /* 64 entries  x 32 replicas */
-#define BGTQ_LUT_K4      10752                   /* 256 entries x 8 replicas  */
-#define BGTQ_LUT_KRAW    18944                   /* 4 tables x 256 fp16       */
-#define BGTQ_LUT_V       20992                   /* V pair table, up to 8192 B */
-#define BGTQ_LUT_IMAGE_BYTES 29184
-/* the same for lut_image_mixed */
-#define BGTQ_LUTM_K0     0                       /* up to 4 packed segments x 256 entries x 8 replicas */
-#define BGTQ_LUTM_KRAW   32768
-#define BGTQ_LUTM_V      34816
-#define BGTQ_LUTM_IMAGE_BYTES 43008
+#define BGTQ_LUT_K4      10752                   /* 256 entries, not replicated */
+#define BGTQ_LUT_KRAW    11776                   /* 4 tables x 256 fp16       */
+#define BGTQ_LUT_KEND    13824                   /* end of the K tables       */
+/* the same for lut_image[BGTQ_K_MIXED]: up to 4 byte-indexed tables of 256 entries, then the raw tables */
+#define BGTQ_LUTM_K0     0
+#define BGTQ_LUTM_KRAW   4096
+#define BGTQ_LUTM_KEND   6144
+#define BGTQ_LUT_IMAGE_BYTES 13824               /* room for either K image */
+#define BGTQ_VLUT_BYTES  8192                    /* a V pair table: 64 entries x 32 replicas at most */
 
 /* error codes (negative); positive return values are hipError_t */
 #define BGTQ_OK            0
@@ -100,83 +100,47 @@ typedef struct bgtq_head_plan {
     float    v_rot_T[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];  /* encode: y = vhat @ v_rot_T */
     float    v_rot[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];    /* decode: out = acc @ v_rot */
     /*
-     * Decode schedule of the bit-packed K record.  A "unit" is 8 consecutive
-     * dims of one segment; a step covers up to 4 units of ONE segment (one
-     * 16x16x32 MFMA).  step[m] = { byte offset of the step's first unit in the
-     * record, bytes per unit (bw, or 8 for raw-byte segments), bits per code
-     * pair (2*bw, 0 for raw bytes), bw, segment index, 1 if last step of its
-     * segment, real units in the step (1..4), first dim of the step }.
-     */
-    int32_t  n_steps;
-    int32_t  reserved1[3];
-    int32_t  step[BGTQ_MAX_STEPS][8];
-
-    /*
-     * The same schedule in the form the MFMA decode kernel copies into LDS, built
-     * on the host so that a work-group starts streaming right away.
+     * Decode schedule of the K record for the MFMA attention kernel, one per K
+     * layout (index BGTQ_K_BITPACKED / BGTQ_K_MIXED), in the form the kernel
+     * copies into LDS.  A "unit" is 8 consecutive packed dims of one segment
+     * (zero padded at the segment's end); a step is one 16x16x32 MFMA whose four
+     * lane groups hold one unit each.  Units of segments with at most 4 bits per
+     * code ("packed" units: two codes select one pair-table entry) fill the first
+     * n_packed_steps steps four at a time in segment order, whatever segment
+     * they belong to; the raw-byte units (5..8 bits, one byte and one table read
+     * per code) fill the steps after them.  Every unit is scaled by its own
+     * segment's norm before the MFMA, so a step may mix segments freely.  Lane
+     * groups past the last unit of either kind repeat that unit with an empty
+     * query range.
+     * steptab[l][m][g] (layout l, step m, lane group g):
+     *   [0] byte offset of the unit in the record, rounded down to 4
+     *   [1] byte offset modulo 4
+     *   [2] byte offset of the unit's table from the start of the kernel's table
+     *       area: BGTQ_VLUT_BYTES + offset inside lut_image[l]
+     *   [3] bank-replica mask (lane * 4 & mask selects the replica; 0: not replicated)
+     *   [4] bits per code pair (2 * bw; 8 in the mixed layout; 0 for raw-byte units)
+     *   [5] log2 of the table's entry stride in bytes
+     *   [6] byte offset of the segment's norm inside a token's norm row (2 * segment)
+     *   [7] first packed dim of the unit | number of real dims (0..8) << 8
      *
-     * steptab[m][g] (step m, lane group g = unit g of the step, units past the
-     * step's last real unit repeat that unit and point at query unit 0):
-     *   [0] byte offset of the unit in the record   [1] 0
-     *   [2] byte offset of the unit's table in lut_image   [3] bank-replica mask
-     *       (lane*4 & mask selects the replica)
-     *   [4] bits per code pair (0: raw bytes)        [5] log2 of the table's entry stride
-     *   [6] byte offset of the segment's norm row, segment * 128
-     *   [7] byte offset of the unit's query operand, 16 * query unit
-     * Query units: unit 0 is all zero; unit u >= 1 covers packed dims
-     * [qunit_dim[u], qunit_dim[u] + qunit_len[u]), zero padded to 8 dims.
-     *
-     * lut_image: pair tables, entry (c0 | c1 << bw) = fp16 centroid pair
-     * (c0 in the low half), every entry replicated over consecutive dwords so
-     * that lanes with different codes hit different LDS banks:
-     *   K bw 1..3 at BGTQ_LUT_K1/K2/K3, 32 replicas; K bw 4 at BGTQ_LUT_K4, 8 replicas;
-     *   K bw 5..8: 256 single fp16 entries each at BGTQ_LUT_KRAW + (bw - 5) * 512
-     *   (0 beyond 2^bw); V table for v_bits at BGTQ_LUT_V (replicas as for K).
+     * lut_image[l]: pair tables, entry (c0 | c1 << bw) = fp16 centroid pair (c0 in the
+     * low half).  Bit-packed layout: bw 1..3 at BGTQ_LUT_K1/K2/K3 with every entry
+     * replicated over 32 consecutive dwords (the 32 lanes of a half-wave then read 32
+     * different LDS banks whatever their codes), bw 4 at BGTQ_LUT_K4 unreplicated
+     * (fewer bank collisions than 8 or 16 replicas give); raw tables of 256 single fp16
+     * entries (0 beyond 2^bw) at BGTQ_LUT_KRAW + (bw - 5) * 512.  Mixed layout: a pair of
+     * codes is one byte, so the i-th packed segment has its own 256-entry table indexed by
+     * that byte at BGTQ_LUTM_K0 + i * 1024 (0 where a nibble is not a code of the segment),
+     * raw tables at BGTQ_LUTM_KRAW + (bw - 5) * 512.
+     * vlut_image[v]: V pair table for V layout v (BGTQ_V_BITPACKED: entry (c0 | c1 <<
+     * v_bits), 32 replicas for v_bits <= 3, unreplicated for 4; BGTQ_V_NIBBLE: 256
+     * byte-indexed entries, unreplicated).
      */
-    int32_t  n_packed_steps;       /* steps with bw <= 4 (they come first) */
-    int32_t  reserved2[3];
-    uint32_t steptab[BGTQ_MAX_STEPS][4][8];
-    int32_t  qunit_dim[32];
-    int32_t  qunit_len[32];
-    uint32_t lut_image[BGTQ_LUT_IMAGE_BYTES / 4];
-
-    /*
-     * The same three tables for the mixed K layout (nibbles of every code of at most
-     * 4 bits, then raw bytes) and the nibble V layout.  A pair of codes is one
-     * byte there, so each packed segment gets its own 256-entry table indexed by
-     * that byte (entry = centroids of the low and the high nibble, 0 where a
-     * nibble is not a code of the segment), 8 replicas: the i-th packed segment at
-     * BGTQ_LUTM_K0 + i * 8192, raw-byte tables at BGTQ_LUTM_KRAW + (bw - 5) * 512,
-     * the byte-indexed V table at BGTQ_LUTM_V.
-     */
-    int32_t  n_steps_mixed;
-    int32_t  n_packed_steps_mixed;
-    int32_t  reserved3[2];
-    uint32_t steptab_mixed[BGTQ_MAX_STEPS][4][8];
-    int32_t  qunit_dim_mixed[32];
-    int32_t  qunit_len_mixed[32];
-    uint32_t lut_image_mixed[BGTQ_LUTM_IMAGE_BYTES / 4];
-
-    /*
-     * Denser schedules for query groups of at most 8 heads, where half of the
-     * MFMA's 16 output columns is free: a packed step may hold units of TWO
-     * segments.  The units of the step's first segment multiply query units
-     * that are non-zero only in columns 0..7, those of its second segment only in
-     * columns 8..15, so every segment still accumulates on its own, is scaled by
-     * its own norm, and the two column halves are added once per tile.
-     * steptab_dense[m][c][g]: as steptab[m][g], for the lanes of column half c;
-     * [6] is the norm row of the segment that owns half c in step m and [7] is
-     * query unit 0 (all zero) unless unit g's segment owns half c.  Steps of one
-     * segment (all raw-byte steps among them) give half 1 nothing but zero query
-     * units.  Query unit numbers are those of qunit_dim / qunit_len (or their
-     * _mixed forms).
-     */
-    int32_t  n_steps_dense;
-    int32_t  n_packed_steps_dense;
-    int32_t  n_steps_dense_mixed;
-    int32_t  n_packed_steps_dense_mixed;
-    uint32_t steptab_dense[BGTQ_MAX_STEPS][2][4][8];
-    uint32_t steptab_dense_mixed[BGTQ_MAX_STEPS][2][4][8];
+    int32_t  n_steps[2];
+    int32_t  n_packed_steps[2];
+    uint32_t steptab[2][BGTQ_MAX_STEPS][4][8];
+    uint32_t lut_image[2][BGTQ_LUT_IMAGE_BYTES / 4];
+    uint32_t vlut_image[2][BGTQ_VLUT_BYTES / 4];
 } bgtq_head_plan;
 
 /* sizeof(bgtq_head_plan) as the library was compiled; the host mirror checks it. */

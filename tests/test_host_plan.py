@@ -213,64 +213,79 @@ def test_plan_struct_mirrors_the_quantizer():
 
 @pytest.mark.parametrize("seed,min_bits,max_bits,budget", [(9, 1, 7, 200), (4, 0, 4, 128), (5, 1, 5, 192)])
 def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, budget):
-    """The MFMA step schedule and the LDS table image in the plan, checked against what
-    they stand for: every packed dim of every segment is read exactly once through a
-    query unit, unit byte offsets walk each segment's stream, and a pair-table entry
-    (c0 | c1 << bw) holds the two fp16 centroids, in every bank replica."""
+    """The MFMA step schedules and the table images in the plan, checked against what they stand
+    for: every packed dim of every segment is read exactly once through a query range, unit byte
+    offsets walk each segment's stream, packed units come before raw-byte units, and a pair-table
+    entry (c0 | c1 << bw) holds the two fp16 centroids, in every bank replica."""
     from blockgtq_amd import plan as P
     q, _ = make_quantizer(seed=seed, min_bits=min_bits, max_bits=max_bits, budget=budget)
     p = q.plan()[0]
-    n_seg, n_steps = int(p['n_seg']), int(p['n_steps'])
-    assert 1 <= n_steps <= P.MAX_STEPS
-    seen = np.zeros(128, dtype=int)
-    unit_of_seg = {s: 0 for s in range(n_seg)}
-    n_packed = 0
-    for m in range(n_steps):
-        off0, ub, pw, bw, s, last, nu, d0 = (int(x) for x in p['step'][m])
-        assert bw == int(p['seg_bw'][s]) and ub == (bw if bw <= 4 else 8) and pw == (2 * bw if bw <= 4 else 0)
-        n_packed += bw <= 4
-        assert n_packed == m + 1 or bw > 4           # raw-byte steps come last
-        for g in range(4):
-            e = [int(x) for x in p['steptab'][m, g]]
-            gg = min(g, nu - 1)
-            u = unit_of_seg[s] + gg
-            assert e[0] == int(p['seg_pack_off'][s]) + u * ub
-            assert e[4] == pw and e[6] == s * 128
-            if g < nu:
-                uid = e[7] // 16
-                assert uid >= 1 and e[7] % 16 == 0
-                a, ln = int(p['qunit_dim'][uid]), int(p['qunit_len'][uid])
-                assert a == int(p['seg_start'][s]) + u * 8
-                assert ln == min(8, int(p['seg_start'][s]) + int(p['seg_len'][s]) - a)
-                seen[a:a + ln] += 1
-            else:
-                assert e[7] == 0                     # padding lanes meet the all-zero query unit
-        unit_of_seg[s] += nu
-        assert last == (unit_of_seg[s] * 8 >= int(p['seg_len'][s]))
-    assert int(p['n_packed_steps']) == n_packed
-    z = int(p['n_zero_dims'])
-    assert (seen[z:] == 1).all() and (seen[:z] == 0).all()
-    img = p['lut_image']
+    n_seg = int(p['n_seg'])
+    for layout in (P.K_BITPACKED, P.K_MIXED):
+        n_steps, n_packed = int(p['n_steps'][layout]), int(p['n_packed_steps'][layout])
+        assert 0 <= n_packed <= n_steps <= P.MAX_STEPS and n_steps >= 1
+        seen = np.zeros(128, dtype=int)
+        next_unit = {s: 0 for s in range(n_seg)}
+        n_ptab = {}
+        for m in range(n_steps):
+            for g in range(4):
+                lo, ph, table, mask, pw, tsh, noff, qd = (int(x) for x in p['steptab'][layout, m, g])
+                off, s, d0, ln = lo + ph, noff // 2, qd & 0xFF, qd >> 8
+                assert lo % 4 == 0 and 0 <= ph < 4 and noff % 2 == 0 and 0 <= s < n_seg
+                bw = int(p['seg_bw'][s])
+                assert (bw <= 4) == (m < n_packed)             # packed units first, raw-byte units after them
+                start, length = int(p['seg_start'][s]), int(p['seg_len'][s])
+                if ln == 0:                                     # a padding lane repeats a real unit
+                    assert (d0 - start) % 8 == 0 and start <= d0 < start + length
+                    continue
+                u = next_unit[s]
+                next_unit[s] += 1
+                assert d0 == start + 8 * u and ln == min(8, start + length - d0)
+                seen[d0:d0 + ln] += 1
+                seg_off = int(p['seg_mixed_off' if layout else 'seg_pack_off'][s])
+                if bw > 4:
+                    assert off == seg_off + 8 * u and pw == 0 and tsh == 1 and mask == 0
+                    assert table == P.VLUT_BYTES + (P.LUTM_KRAW if layout else P.LUT_KRAW) + (bw - 5) * 512
+                elif layout == P.K_BITPACKED:
+                    assert off == seg_off + bw * u and pw == 2 * bw
+                    assert table == P.VLUT_BYTES + P.LUT_K[bw]
+                    assert (mask, tsh) == ((124, 7) if bw <= 3 else (0, 2))
+                else:
+                    assert off == seg_off + 4 * u and pw == 8 and (mask, tsh) == (0, 2)
+                    n_ptab.setdefault(s, len(n_ptab))
+                    assert table == P.VLUT_BYTES + 1024 * n_ptab[s]
+        z = int(p['n_zero_dims'])
+        assert (seen[z:] == 1).all() and (seen[:z] == 0).all()
+        assert all(next_unit[s] == (int(p['seg_len'][s]) + 7) // 8 for s in range(n_seg))
+    img = p['lut_image'][P.K_BITPACKED]
+    imgm = p['lut_image'][P.K_MIXED]
+    i_ptab = 0
     for s in range(n_seg):
         bw = int(p['seg_bw'][s])
         cb = p['k_codebook_f16'][s]
         if bw <= 4:
-            rep = 8 if bw == 4 else 32
+            rep = 1 if bw == 4 else 32
             t = img[P.LUT_K[bw] // 4:][:(1 << 2 * bw) * rep].reshape(-1, rep)
             assert (t == t[:, :1]).all()
+            tm = imgm[256 * i_ptab:256 * (i_ptab + 1)]
+            i_ptab += 1
             for c0 in range(1 << bw):
                 for c1 in range(1 << bw):
                     assert int(t[c0 | (c1 << bw), 0]) == int(cb[c0]) | (int(cb[c1]) << 16)
+                    assert int(tm[c0 | (c1 << 4)]) == int(cb[c0]) | (int(cb[c1]) << 16)
         else:
-            raw = img[(P.LUT_KRAW + (bw - 5) * 512) // 4:][:128].view(np.uint16)
-            assert np.array_equal(raw[:1 << bw], cb[:1 << bw]) and not raw[1 << bw:].any()
+            for im, base in ((img, P.LUT_KRAW), (imgm, P.LUTM_KRAW)):
+                raw = im[(base + (bw - 5) * 512) // 4:][:128].view(np.uint16)
+                assert np.array_equal(raw[:1 << bw], cb[:1 << bw]) and not raw[1 << bw:].any()
     vb = int(p['v_bits'])
-    rep = 8 if vb == 4 else 32
-    tv = img[P.LUT_V // 4:][:(1 << 2 * vb) * rep].reshape(-1, rep)
+    rep = 1 if vb == 4 else 32
+    tv = p['vlut_image'][P.V_BITPACKED][:(1 << 2 * vb) * rep].reshape(-1, rep)
+    tn = p['vlut_image'][P.V_NIBBLE][:256]
     vl = p['v_lut_f16']
     for c0 in range(1 << vb):
         for c1 in range(1 << vb):
             assert (tv[c0 | (c1 << vb)] == (int(vl[c0]) | (int(vl[c1]) << 16))).all()
+            assert int(tn[c0 | (c1 << 4)]) == int(vl[c0]) | (int(vl[c1]) << 16)
 
 
 # ---------------------------------------------------------------- V packing
@@ -291,48 +306,38 @@ def test_v_packing_matches_a_plain_bit_stream(bits):
 
 
 # ---------------------------------------------------------------- library surface
-def _emulate_steps(p, rec, norms, qrot, dense, mixed):
-    """Scores of one token record computed the way the MFMA kernel walks the plan's step
-    tables: per (step, column half, lane group) one unit of 8 codes through the pair table
-    (or the raw-byte table), times the query unit, scaled by the norm row of the half."""
-    sfx = '_mixed' if mixed else ''
-    img = (p['lut_image_mixed'] if mixed else p['lut_image']).view(np.uint8)
-    qd, ql = p['qunit_dim' + sfx], p['qunit_len' + sfx]
-    if dense:
-        tab, ns, npk = p['steptab_dense' + sfx], int(p['n_steps_dense' + sfx]), int(p['n_packed_steps_dense' + sfx])
-    else:
-        t = p['steptab' + sfx]
-        tab, ns, npk = np.stack([t, t], 1), int(p['n_steps' + sfx]), int(p['n_packed_steps' + sfx])
-    out = np.zeros((2, qrot.shape[0]))
+def _emulate_steps(p, rec, norms, qrot, layout):
+    """Scores of one token record computed the way the MFMA kernel walks the plan's step table:
+    per (step, lane group) one unit of 8 codes through the pair table (or the raw-byte table),
+    times the unit's query range, times the norm of the unit's segment."""
+    from blockgtq_amd import plan as P
+    img = p['lut_image'][layout].view(np.uint8)
+    ns, npk = int(p['n_steps'][layout]), int(p['n_packed_steps'][layout])
+    out = np.zeros(qrot.shape[0])
     recp = np.concatenate([rec, np.zeros(16, np.uint8)])
     for m in range(ns):
-        for half in range(2):
-            acc = np.zeros(qrot.shape[0])
-            for g in range(4):
-                off, _, table, _mask, pw, tsh, nrm_off, qoff = (int(x) for x in tab[m, half, g])
-                uid = qoff // 16
-                if uid == 0:
-                    continue
-                d0, ln = int(qd[uid]), int(ql[uid])
-                if m < npk:
-                    raw = int.from_bytes(recp[off:off + 8].tobytes(), 'little')
-                    vals = []
-                    for i in range(4):
-                        a = table + (((raw >> (i * pw)) & ((1 << pw) - 1)) << tsh)
-                        vals += list(img[a:a + 4].view(np.float16))
-                else:
-                    vals = [img[table + 2 * int(recp[off + i]):][:2].view(np.float16)[0] for i in range(8)]
-                acc += qrot[:, d0:d0 + ln].astype(np.float64) @ np.array(vals[:ln], np.float64)
-            out[half] += acc * float(norms[int(tab[m, half, 0][6]) // 128])
-    return out.sum(0) if dense else out[0]
+        for g in range(4):
+            lo, ph, table, _mask, pw, tsh, noff, qd = (int(x) for x in p['steptab'][layout, m, g])
+            off, d0, ln = lo + ph, qd & 0xFF, qd >> 8
+            if ln == 0:
+                continue
+            table -= P.VLUT_BYTES
+            if m < npk:
+                raw = int.from_bytes(recp[off:off + 8].tobytes(), 'little')
+                vals = []
+                for i in range(4):
+                    a = table + (((raw >> (i * pw)) & ((1 << pw) - 1)) << tsh)
+                    vals += list(img[a:a + 4].view(np.float16))
+            else:
+                vals = [img[table + (int(recp[off + i]) << tsh):][:2].view(np.float16)[0] for i in range(8)]
+            out += (qrot[:, d0:d0 + ln].astype(np.float64) @ np.array(vals[:ln], np.float64)) * float(norms[noff // 2])
+    return out
 
 
 @pytest.mark.parametrize("seed,min_bits,max_bits,budget", [(9, 1, 7, 200), (4, 0, 4, 128), (5, 1, 5, 192), (2, 2, 2, 128)])
 def test_step_tables_reproduce_the_checker_scores(oracle_lib, seed, min_bits, max_bits, budget):
-    """Both schedules (one segment per step; two segments per step in separate column
-    halves) and both record layouts, walked on the CPU, give q . dequant(k) of the checker
-    exactly; the two-segment schedule never needs more steps and its halves agree on
-    everything but query unit and norm row."""
+    """The step schedules of both record layouts, walked on the CPU, give q . dequant(k) of the
+    checker exactly."""
     q, en = make_quantizer(seed=seed, min_bits=min_bits, max_bits=max_bits, budget=budget)
     k, _, qq = make_kv(en, 4, seed=seed)
     plan = q.plan()
@@ -341,22 +346,13 @@ def test_step_tables_reproduce_the_checker_scores(oracle_lib, seed, min_bits, ma
     codes, raw, corr = oracle_lib.encode_k(plan, k)
     qr = oracle_lib.rotate_q(plan, qq).astype(np.float32)
     for mixed in (False, True):
-        sfx = '_mixed' if mixed else ''
-        assert 1 <= int(p['n_steps_dense' + sfx]) <= int(p['n_steps' + sfx])
-        d = p['steptab_dense' + sfx][:int(p['n_steps_dense' + sfx])]
-        assert np.array_equal(d[:, 0, :, :6], d[:, 1, :, :6])
-        for m in range(d.shape[0]):
-            both = (d[m, 0, :, 7] != 0) & (d[m, 1, :, 7] != 0)
-            assert not both.any()                        # a unit feeds one half only
-            assert len({int(x) for x in d[m, :, :, 6].ravel()}) <= 2
         kp = oracle_lib.pack_k(plan, codes, int(mixed))
         nr = (corr if mixed else raw)[:, :max(ng, 1)]
         kn = oracle_lib.f2h(nr).view(np.float16).astype(np.float32)
         for t in range(k.shape[0]):
             ref = qr.astype(np.float64) @ oracle_lib.dequant_k(plan, codes[t:t + 1], oracle_lib.f2h(nr[t:t + 1]))[0].astype(np.float64)
-            for dense in (False, True):
-                got = _emulate_steps(p, kp[t], kn[t], qr, dense, mixed)
-                assert np.abs(got - ref).max() < 1e-9
+            got = _emulate_steps(p, kp[t], kn[t], qr, int(mixed))
+            assert np.abs(got - ref).max() < 1e-9
 
 
 def test_cache_rows_avoid_strides_that_collide_in_lds():
