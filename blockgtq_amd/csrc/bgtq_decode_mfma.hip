@@ -1,4 +1,4 @@
-// MFMA decode attention over packed K and V records (gfx950).
+// MFMA decode attention over packed K and V records (gfx950), query groups of at most 8 heads.
 //
 // One work-group of up to 12 waves (3 per SIMD, as many as the tile buffers leave
 // room for in LDS) owns one partition of one (batch row, KV head).  The 64-token
@@ -20,28 +20,29 @@
 // Tables of at most 64 entries are replicated 32 times (entry stride 128 bytes), so
 // that the 32 lanes of a half-wave, which LDS serves together, always read 32
 // different banks; the 256-entry tables are not replicated (8 or 16 copies collide
-// more often than none).  A unit costs one raw read, four {bit-field extract,
-// shift-add, table read} triples and yields the eight fp16 operands of one MFMA
-// k-group.
+// more often than none).  A unit costs one raw read, four {rotate, and-or, table read}
+// triples and yields the eight fp16 operands of one MFMA k-group.
 //
-// QK^T:  v_mfma_f32_16x16x32_f16, A = dequantised K (row = token, lane group g
-//        supplies unit g of step m; field width, table and norm column come from the
-//        plan's step table per lane group), B = rotated queries per step, gathered
-//        once per work-group into LDS (zero on padding dims).  Every table word is
-//        multiplied by the fp16 norm of its own segment before the MFMA and enters it as
-//        the rounded fp16 product plus its exact rounding error (a second MFMA), which
-//        keeps the scores at fp32 accuracy; a step may therefore mix units of several
-//        segments and the steps of a token block accumulate in the MFMA itself.
-// PV:    the D layout of a 16-token block is the A layout of the value product
-//        (row = head, lane group g holds 4 tokens), so P never leaves its lane.  With
-//        at most 8 query heads the product runs over (token, dim parity) pairs and a
-//        V table word is an MFMA operand as it comes; with 9..16 heads V words are
-//        transposed with v_perm_b32.  The V norm is folded into P in fp32 before P is
-//        rounded to fp16.
-// Softmax: exponentials are taken relative to a per-head reference that is kept
-//        above every score seen so far.  It is only moved (to the new maximum
+// QK^T:  lane = token.  Every lane decodes the same unit of its own token, so the field
+//        positions, masks and tables of a unit are the same in every lane: the plan's
+//        per-unit parameter rows are copied to LDS once and read (all lanes one address)
+//        as the units go by, together with the unit's query operands, through one
+//        running pointer.  v_mfma_f32_16x16x32_f16 with B = dequantised K (column j of
+//        lane group g is token 16g + j) and A = the unit's rotated queries, zero outside
+//        lane group g for rows 4g..4g+3: D[4g + r][j] is then q_head(r) . k_token(16g + j),
+//        i.e. every lane receives the scores of its own token, 4 heads per MFMA.  The
+//        units of a segment accumulate in the MFMA and the segment's sum is scaled by
+//        the token's fp16 norm of that segment in fp32: one multiply-add per head and lane.
+// Softmax: lane = token, exponentials relative to a per-head reference (wave-uniform) that
+//        is kept above every score seen so far.  It is only moved (to the new maximum
 //        plus a headroom of 4 in log2 units) when a score of the tile exceeds it;
 //        otherwise the tile needs no cross-lane traffic at all.
+// PV:    P * v_norm goes through LDS once (2 bytes per head and token) into the A layout of
+//        the value product.  That product runs over (token, dim parity) pairs: A row
+//        (head h, parity e) holds P[h][t] in slot (t, e), B column c holds the V table word
+//        of token t, so a table word is an MFMA operand as it comes.
+// Merge: every wave leaves its reference, denominator and sums in its own (then dead) tile
+//        buffers; after one barrier the first 32 * gqa threads fold the waves.
 #include <atomic>
 
 #include "bgtq_decode.h"
@@ -58,26 +59,38 @@ typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
 
 constexpr int D = BGTQ_D;
 constexpr int MT = 64;             // tokens per wave tile = 4 MFMA row blocks
-constexpr int MAX_STEPS = BGTQ_MAX_STEPS;
+constexpr int MAX_UNITS = BGTQ_MAX_UNITS;
 constexpr int MAX_WAVES = 12;
 constexpr int MAX_KN = 8;          // norm columns per token row
 constexpr int LDS_LIMIT = 160 * 1024;
-constexpr int MERGE_STRIDE = BGTQ_D + 8;   // most floats from one row of a wave's result to the next in the merge area
-constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
+constexpr float REFRESH = 4.0f;
+//    // log2 headroom put above the largest score when the reference is refreshed
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
-// [ V pair table | K tables of the record layout in use | step table | query operands | per wave: K tile + K norms
-//   + V norms, V tile, fp32 V norms ]
+// [ V pair table | K tables of the record layout in use | query units | per wave: K tile + K norms + V norms,
+//   V tile, P ]
+// (query units are followed by the segment parameters)
 constexpr int VTAB_BYTES = BGTQ_VLUT_BYTES;
 constexpr int KTAB_BYTES = BGTQ_LUT_IMAGE_BYTES;
-constexpr int STEPTAB_OFF = VTAB_BYTES + KTAB_BYTES;            // [step][lane group] x 32 B
-constexpr int QB_OFF = STEPTAB_OFF + MAX_STEPS * 4 * 32;        // [step][lane] x 16 B: the MFMA B operand
-constexpr int WAVES_OFF = QB_OFF + MAX_STEPS * 1024;
+constexpr int UROW = MAX_UNITS * 16;                            // one 16-byte slot per unit
+// What a lane reads per unit sits behind one pointer: its A rows for both MFMAs and the unit's
+// parameters.  One struct per A row 0..3 (heads r and r + 4) and one whose A rows are zero (for the
+// lanes outside the unit's lane group); the parameters are repeated in each.  The stride puts the
+// five structs on different banks.
+constexpr int QS_A2 = UROW, QS_PA = 2 * UROW, QS_PB = 3 * UROW;
+constexpr int QSTRUCT = 4 * UROW + 16;
+constexpr int QS_OFF = VTAB_BYTES + KTAB_BYTES;
+constexpr int N_QJOBS = 8 * MAX_UNITS + 5 * 2 * MAX_UNITS + 2 * MAX_UNITS;   // query units, parameter halves, zero rows
+constexpr int WAVES_OFF = QS_OFF + 5 * QSTRUCT;
+constexpr int PROW = MT * 4 + 64;                                // bytes from one head's P row to the next: rows land 16 banks apart
+constexpr int PBUF_BYTES = 8 * PROW;                          // P of a tile: [head][token], fp16 in the low half of a dword
 
 __host__ __device__ constexpr int kimg_bytes(int k_layout) { return k_layout == BGTQ_K_MIXED ? BGTQ_LUTM_KEND : BGTQ_LUT_KEND; }
 __host__ __device__ constexpr int vlut_bytes(int vbw, bool nibble) {
     return (nibble || vbw == 4) ? 1024 : (1 << (2 * vbw)) * 128;
 }
+
+constexpr int MERGE_BYTES = 64 + 8 * 32 * 16;                    // what a wave leaves for the merge: m, l, 8 heads x 128 floats
 
 __host__ __device__ inline TileLayout tile_layout(int krow, int vrow, int kn_st) {
     TileLayout t;
@@ -88,7 +101,12 @@ __host__ __device__ inline TileLayout tile_layout(int krow, int vrow, int kn_st)
     t.kbuf = t.kt + t.knr + t.vnr;
     return t;
 }
-constexpr int VNF_BYTES = MT * 4;      // fp32 V norms of the tile, per wave
+
+// LDS bytes of one wave: its tile buffers, which also take its contribution to the merge
+__host__ __device__ inline int wave_lds_bytes(const TileLayout& t) {
+    const int tiles = t.kbuf + t.vt + PBUF_BYTES;
+    return tiles > MERGE_BYTES ? tiles : MERGE_BYTES;
+}
 
 // (a & mask) | c in one instruction; the mask travels in a scalar register
 __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t c) {
@@ -96,12 +114,27 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t c
     asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(c));
     return r;
 }
-// Both halves of a table word times the fp16 in the low half of n, as an unevaluated sum of two
-// fp16 pairs: hi is the rounded product and lo the rounding error (a fused multiply-add returns it
-// exactly), so hi + lo is the 22-bit product itself.
-__device__ __forceinline__ void scale_pair(uint32_t w, uint32_t n, uint32_t& hi, uint32_t& lo) {
-    asm("v_pk_mul_f16 %0, %1, %2 op_sel_hi:[1,0]" : "=v"(hi) : "v"(w), "v"(n));
-    asm("v_pk_fma_f16 %0, %1, %2, %3 op_sel_hi:[1,0,1] neg_lo:[0,0,1] neg_hi:[0,0,1]" : "=v"(lo) : "v"(w), "v"(n), "v"(hi));
+// two consecutive dwords at a 4-byte aligned LDS address (one ds_read2_b32; a plain load, so that the
+// compiler places the wait for it)
+typedef uint32_t dword_pair __attribute__((ext_vector_type(2), aligned(4)));
+__device__ __forceinline__ void lds_read2(uint32_t addr, uint32_t& lo, uint32_t& hi) {
+    const dword_pair r = *(const __attribute__((address_space(3))) dword_pair*)(uintptr_t)addr;
+    lo = r.x;
+    hi = r.y;
+}
+
+// 4 / 8 bytes from any LDS byte address: aligned dword reads and a byte funnel shift (unaligned LDS
+// reads are legal on this target but several times slower)
+__device__ __forceinline__ uint32_t lds_codes4(uint32_t addr) {
+    uint32_t lo, hi;
+    lds_read2(addr & ~3u, lo, hi);
+    return __builtin_amdgcn_alignbyte(hi, lo, addr & 3u);
+}
+__device__ __forceinline__ uint2v lds_codes8(uint32_t addr) {
+    uint32_t lo, hi;
+    lds_read2(addr & ~3u, lo, hi);
+    const uint32_t hi2 = *(const __attribute__((address_space(3))) uint32_t*)(uintptr_t)((addr & ~3u) + 8);
+    return (uint2v){__builtin_amdgcn_alignbyte(hi, lo, addr & 3u), __builtin_amdgcn_alignbyte(hi2, hi, addr & 3u)};
 }
 
 // Read through an absolute LDS address (the kernel has no static LDS, so the dynamic block
@@ -173,16 +206,50 @@ __device__ __forceinline__ void wait_loads(int n) {
 #undef BGTQ_WAIT_CASE
 }
 
-static_assert(offsetof(bgtq_head_plan, steptab) % 16 == 0 && offsetof(bgtq_head_plan, lut_image) % 16 == 0 &&
-              offsetof(bgtq_head_plan, vlut_image) % 16 == 0 && (sizeof(uint32_t) * MAX_STEPS * 4 * 8) % 16 == 0 &&
-              BGTQ_LUT_IMAGE_BYTES % 16 == 0 && BGTQ_VLUT_BYTES % 16 == 0,
+
+static_assert(offsetof(bgtq_head_plan, kprog) % 16 == 0 && offsetof(bgtq_head_plan, lut_image) % 16 == 0 &&
+              offsetof(bgtq_head_plan, vlut_image) % 16 == 0 && BGTQ_LUT_IMAGE_BYTES % 16 == 0 && BGTQ_VLUT_BYTES % 16 == 0,
               "plan tables are copied 16 bytes at a time");
+
+
+// (a & mask) | c with all three operands in vector registers
+__device__ __forceinline__ uint32_t and_or_v(uint32_t a, uint32_t mask, uint32_t c) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(mask), "v"(c));
+    return r;
+}
+
+// Wave-wide sum / maximum through the DPP lane crossbar (no LDS traffic): quads, half rows, rows of
+// 16, then the row results travel to the rows behind them; lane 63 ends up with the total (the
+// maximum is handed to every lane, the sum stays in lane 63).
+template <int CTRL, int ROWS>
+__device__ __forceinline__ float dpp_move(float keep, float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, x),
+                                                                 CTRL, ROWS, 0xF, false));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp_move<0xB1, 0xF>(0.f, x);          // quad_perm [1,0,3,2]
+    x += dpp_move<0x4E, 0xF>(0.f, x);          // quad_perm [2,3,0,1]
+    x += dpp_move<0x141, 0xF>(0.f, x);         // row_half_mirror
+    x += dpp_move<0x140, 0xF>(0.f, x);         // row_mirror
+    x += dpp_move<0x142, 0xA>(0.f, x);         // row_bcast:15 into rows 1 and 3
+    x += dpp_move<0x143, 0xC>(0.f, x);         // row_bcast:31 into rows 2 and 3
+    return x;                                  // (the total is in lane 63 only)
+}
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp_move<0xB1, 0xF>(x, x));
+    x = fmaxf(x, dpp_move<0x4E, 0xF>(x, x));
+    x = fmaxf(x, dpp_move<0x141, 0xF>(x, x));
+    x = fmaxf(x, dpp_move<0x140, 0xF>(x, x));
+    x = fmaxf(x, dpp_move<0x142, 0xA>(x, x));
+    x = fmaxf(x, dpp_move<0x143, 0xC>(x, x));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
 
 // VBW: bits per V code; VST: bytes from one V record to the next (the record itself is
 // 16 * VBW bytes; a padded stride keeps the rows of a tile on different LDS banks)
-// DENSE: at most 8 query heads per KV head (a PV product that uses the eight spare head
-// rows of the MFMA instead of transposing V)
-template <int VBW, int VST, bool DENSE>
+// TWO: more than 4 query heads per KV head (a second MFMA per unit for heads 4..7)
+template <int VBW, int VST, bool TWO>
 __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -194,7 +261,6 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const int li = lane & 15, lg = lane >> 4;           // MFMA row/col index, lane group
     const int kl = a.k_layout;
     const bool vnib = a.v_layout == BGTQ_V_NIBBLE;
-    constexpr uint32_t smem_lds = 0;                     // no static LDS: checked by the launcher
 
     // ---- this partition's tiles: the tiles of the row are dealt to the partitions as evenly as
     // whole tiles allow (partition sizes differ by at most one tile)
@@ -204,61 +270,73 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const int tile_lo = c * per + min(c, rem), tile_hi = tile_lo + per + (c < rem ? 1 : 0);
     const int t0 = tile_lo * MT, t1 = min(tile_hi * MT, T);
 
-    // ---- query operand, part 1: which dims unit (step, lane group) covers -> this thread's 16 bytes
-    // of the rotated queries.  Thread i builds B operand (step i / 64, lane i % 64): head = column.
     const int krow = a.k_row_width;
     constexpr int vrow = VST;
     const int kn_st = (int)a.kn_st;
     const TileLayout tl = a.tl;
     const uint16_t* q_src = a.q + b * a.q_sb + (int64_t)h * gqa * a.q_sh;
-    // Wave w builds the operand of step w (and w + nw, ... when there are fewer waves than steps):
-    // the four descriptors of a step are wave-uniform, so they arrive through the scalar cache and
-    // do not queue behind the copies below.
-    uint32_t qd[4] = {0, 0, 0, 0};
-    if (wave < MAX_STEPS) {
+    const int n_units = min(P.n_units[kl], MAX_UNITS);
+    const int n_pair = min(P.n_pair_units[kl], n_units);
+    const uint32_t kend = P.kend[kl], kfirst = P.kfirst[kl];
+    // Job j < N_QJOBS fills one 16-byte slot of the structs: a query unit (head j / MAX_UNITS), one half
+    // of a unit's parameters for one struct, or a slot of the all-zero A rows.  The loads of a thread's
+    // first job go out here, the slots are written once the streaming loads have been issued.
+    auto job_load = [&](int j) -> uint4v {
+        uint4v w = {0, 0, 0, 0};
+        if (j < 8 * MAX_UNITS) {
+            const int jh = j / MAX_UNITS, ju = j - jh * MAX_UNITS;
+            const uint32_t dsc = P.kunit[kl][ju];
+            const int d0 = (int)(dsc & 0xFF), len = (int)(dsc >> 8);
+            if (jh < gqa && len > 0) {
+                const uint32_t* row = (const uint32_t*)(q_src + jh * a.q_sh + d0);        // d0 is even
 #pragma unroll
-        for (int g = 0; g < 4; g++) qd[g] = P.steptab[kl][wave][g][7];
-    }
-    const int n_steps = min(P.n_steps[kl], MAX_STEPS);
-    const int n_packed = min(P.n_packed_steps[kl], n_steps);   // raw-byte steps come last
-    auto load_q = [&](uint32_t dsc, uint32_t (&w)[4]) {
-        const int col = DENSE ? (li & 7) : li;
-        const int d0 = (int)(dsc & 0xFF), len = (int)(dsc >> 8);
-#pragma unroll
-        for (int pp = 0; pp < 4; pp++) w[pp] = 0;
-        if (col < gqa && len > 0) {
-            const uint32_t* row = (const uint32_t*)(q_src + col * a.q_sh + d0);      // d0 is even
-#pragma unroll
-            for (int pp = 0; pp < 4; pp++)
-                w[pp] = row[min(pp, (D - d0) / 2 - 1)] &
-                        ((2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u));
+                for (int pp = 0; pp < 4; pp++)
+                    w[pp] = row[min(pp, (D - d0) / 2 - 1)] &
+                            ((2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u));
+            }
+        } else if (j < 8 * MAX_UNITS + 10 * MAX_UNITS) {
+            const int r = (j - 8 * MAX_UNITS) % (2 * MAX_UNITS);
+            w = *(const uint4v*)&P.kprog[kl][r >> 1][(r & 1) * 4];
         }
+        return w;
     };
+    auto job_slot = [&](int j) -> uint32_t {
+        if (j < 8 * MAX_UNITS) {
+            const int jh = j / MAX_UNITS, ju = j - jh * MAX_UNITS;
+            return QS_OFF + (jh & 3) * QSTRUCT + (jh >> 2) * QS_A2 + ju * 16;
+        }
+        if (j < 8 * MAX_UNITS + 10 * MAX_UNITS) {
+            const int s5 = (j - 8 * MAX_UNITS) / (2 * MAX_UNITS), r = (j - 8 * MAX_UNITS) % (2 * MAX_UNITS);
+            return QS_OFF + s5 * QSTRUCT + ((r & 1) ? QS_PB : QS_PA) + (r >> 1) * 16;
+        }
+        return QS_OFF + 4 * QSTRUCT + (j - 18 * MAX_UNITS) * 16;
+    };
+    uint4v job0 = {0, 0, 0, 0};
+    if (tid < N_QJOBS) job0 = job_load(tid);
 
-    // ---- tables by DMA: V table at LDS offset 0, K tables behind it, then the step table; the chunks
-    // are dealt round-robin to the waves
+    // ---- tables by DMA: V table at LDS offset 0, K tables behind it; the chunks are dealt round-robin
+    // to the waves
     const uint32_t voff = (uint32_t)lane * 16;
     {
         const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
         const uint8_t* kimg_src = (const uint8_t*)P.lut_image[kl];
-        const uint8_t* st_src = (const uint8_t*)&P.steptab[kl][0][0][0];
         const int vbytes = vlut_bytes(VBW, vnib), kbytes = kimg_bytes(kl);
         const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
-        for (int cc = wave; cc < vch + kch + 1; cc += nw) {
+        for (int cc = wave; cc < vch + kch; cc += nw) {
             const uint8_t* src;
             uint32_t dst;
             int left;
             if (cc < vch) { src = vimg + cc * 1024; dst = cc * 1024; left = vbytes - cc * 1024; }
-            else if (cc < vch + kch) { src = kimg_src + (cc - vch) * 1024; dst = VTAB_BYTES + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
-            else { src = st_src; dst = STEPTAB_OFF; left = MAX_STEPS * 4 * 32; }
-            dma16(voff, src, __builtin_amdgcn_readfirstlane(smem_lds + dst), __builtin_amdgcn_ballot_w64((int)voff < left));
+            else { src = kimg_src + (cc - vch) * 1024; dst = VTAB_BYTES + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
+            dma16(voff, src, __builtin_amdgcn_readfirstlane(dst), __builtin_amdgcn_ballot_w64((int)voff < left));
         }
     }
 
     // ---- per-wave buffers and streaming sources: 16-byte aligned bases and phases (constant per tile) ----
-    const uint32_t kbuf = WAVES_OFF + wave * tl.kbuf;                          // K records, K norms, V norms
-    const uint32_t vbuf = WAVES_OFF + nw * tl.kbuf + wave * (tl.vt + VNF_BYTES); // V records, then fp32 V norms
-    const uint32_t vnf = vbuf + tl.vt;
+    const int wave_bytes = wave_lds_bytes(tl);
+    const uint32_t kbuf = WAVES_OFF + wave * wave_bytes;                       // K records, K norms, V norms
+    const uint32_t vbuf = kbuf + tl.kbuf;                                     // V records
+    const uint32_t pbuf = vbuf + tl.vt;                                       // P * v_norm of the tile
     const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
     const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
     const uint8_t* kn_base = (const uint8_t*)(a.kn + b * a.kn_sb + h * a.kn_sh);
@@ -294,184 +372,135 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     int v_loads = 0;                 // loads of the V tile issued after the current K tile
     if (tile < t1) issue_k(tile);
 
-    // ---- query operand, part 2: rows of the rotated queries straight from memory, cut to the dims
-    // of the unit (the wait for them also covers the tables and the first K tile: all are needed now)
-    for (int m = wave; m < MAX_STEPS; m += nw) {
-        uint32_t dsc;
-        if (m == wave) dsc = lg == 0 ? qd[0] : lg == 1 ? qd[1] : lg == 2 ? qd[2] : qd[3];
-        else dsc = P.steptab[kl][m][lg][7];
-        uint32_t w[4];
-        load_q(dsc, w);
-        lds_put<uint4v>(QB_OFF + m * 1024 + lane * 16, (uint4v){w[0], w[1], w[2], w[3]});
+    // ---- the structs' slots; the P buffers' high halves (the wait for the query rows also covers the
+    // tables and the first K tile: all are needed now)
+    {
+        if (tid < N_QJOBS) lds_put<uint4v>(job_slot(tid), job0);
+        for (int j = tid + nthr; j < N_QJOBS; j += nthr) lds_put<uint4v>(job_slot(j), job_load(j));
+#pragma unroll
+        for (int i = 0; i < PBUF_BYTES; i += 1024)
+            if (i + 1024 <= PBUF_BYTES || lane * 16 < PBUF_BYTES - i) lds_put<uint4v>(pbuf + i + lane * 16, (uint4v){0, 0, 0, 0});
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // waves without a step to build wait for their copies here
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's table chunks and its first K tile
     if (tile < t1) v_loads = issue_v(tile);
     __syncthreads();
 
-    const float c2 = a.scale * 1.44269504088896340736f;      // logits go through exp2
-    const uint32_t lane4 = (uint32_t)lane * 4;
-    // V table replica of this lane (the table sits at LDS address 0, so field bits OR-ed in never
-    // meet the base); the 256-entry tables are not replicated
+    const float c2 = a.scale * 1.44269504088896340736f;      // scores are kept in log2 units
+    constexpr bool two = TWO;
+    const uint32_t rep = ((uint32_t)lane & 31u) * 4u;          // this lane's replica of the 32-fold tables
+    // QK^T operands: this lane's record and norm row; its A rows (4 lg' + h' with lg' = li >> 2: the queries of
+    // head h' (+ 4 for the second MFMA) where lg' is this lane's own group, the all-zero head elsewhere)
+    const uint32_t krow_l = kbuf + kph + (uint32_t)lane * krow;
+    const uint32_t knrow_l = kbuf + tl.kt + knph + (uint32_t)lane * kn_st * 2;
+    const uint32_t vn_l = kbuf + tl.kt + tl.knr + vnph + (uint32_t)lane * 2;
+    const bool q_live = (li >> 2) == lg;
+    const uint32_t qs_l = QS_OFF + (q_live ? (li & 3) : 4) * QSTRUCT;
+    // PV operands: V table replica (the table sits at LDS address 0, so field bits OR-ed in never meet the
+    // base; the 256-entry tables are not replicated), raw codes, P rows
     constexpr bool V_UNREP = VBW == 4;                        // also every nibble record (VBW 4 by construction)
-    const uint32_t vbank = V_UNREP ? 0u : (lane4 & 124u);
+    const uint32_t vbank = V_UNREP ? 0u : rep;
     constexpr int vshift = V_UNREP ? 2 : 7;
-    const uint32_t kstride = 16u * krow;
-    const uint32_t krow0 = kbuf + kph + (uint32_t)li * krow;                 // record of token li of block 0
-    const uint32_t knrow0 = kbuf + tl.kt + knph + (uint32_t)li * kn_st * 2;  // its norm row
     const uint32_t vc = vph + (uint32_t)li * VBW;
     const uint32_t vbase = vbuf + (vc & ~3u) + (uint32_t)lg * 4 * vrow, v_sh = vc & 3u;
-    const uint32_t stl = STEPTAB_OFF + lg * 32;
-    const uint32_t qbl = QB_OFF + lane * 16;
+    const uint32_t p_wr = pbuf + (uint32_t)lane * 4;                             // + head * 256
+    const uint32_t p_rd = pbuf + (uint32_t)(li & 7) * PROW + (uint32_t)lg * 16;    // + block * 64
+    const uint32_t p_shift = (li & 8) ? 16u : 0u;              // rows 8..15 carry the odd dims: P in the high half
 
-    float m_ref = -INFINITY;        // reference of head li, in exp2 units; never below a score seen
-    float l_part = 0.f;             // this lane's share of the softmax denominator
-    constexpr int NACC = DENSE ? 4 : 8;         // output accumulators (16 x 16 each)
-    float4v acc[NACC];
+    float m_ref[8], l_part[8];      // per head: reference in log2 units (never below a score seen), this lane's share of the denominator
 #pragma unroll
-    for (int e = 0; e < NACC; e++) acc[e] = (float4v){0, 0, 0, 0};
+    for (int hh = 0; hh < 8; hh++) { m_ref[hh] = -INFINITY; l_part[hh] = 0.f; }
+    float4v acc[4];                 // acc[jb][r] = out[head 4(lg & 1) + r][dim 8 li + 2 jb + (lg >> 1)]
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[e] = (float4v){0, 0, 0, 0};
 
     for (; tile < t1; tile += step_tiles) {
         const int nt = min(MT, t1 - tile);
         const bool more = tile + step_tiles < t1;
         wait_loads(v_loads);                                 // K records and norms of this tile are in LDS
         __builtin_amdgcn_wave_barrier();
-        // fp32 V norms of the tile (lane = token), 0 past the end
-        {
-            const uint16_t vraw = lds_at<uint16_t>(kbuf + tl.kt + tl.knr + vnph + lane * 2);
-            lds_put<float>(vnf + lane * 4, lane < nt ? bgtq_h2f(vraw) : 0.f);
-        }
+        const uint32_t vraw = lds_at<uint16_t>(vn_l);
 
-        // ---- scores ---------------------------------------------------------------
-        float4v S[4];
+        // ---- scores of this lane's token, 8 heads, in log2 units ----------------------------------------
+        float S[8];
 #pragma unroll
-        for (int k = 0; k < 4; k++) S[k] = (float4v){0, 0, 0, 0};
+        for (int hh = 0; hh < 8; hh++) S[hh] = 0.f;
         {
-            // Software pipeline over the packed steps.  The iteration that multiplies step m first
-            // forms the table addresses of step m+1 (from raw codes and parameters read one
-            // iteration earlier), multiplies step m, then fetches the parameters of step m+2, its raw
-            // codes and norms (through offsets read one iteration earlier still) and last the table
-            // words of step m+1.  Every LDS read is consumed one iteration after it was issued.
-            const int last = n_packed - 1;
-            uint4v e0, e1;                                  // parameters of the step whose addresses are formed next
-            uint32_t xo, no;                                // record and norm offsets of the step fetched next
-            uint32_t rlo[4], rhi[4], nrm[4], ncur[4];
-            uint32_t ad[4][4];
-            uint4v w[4];
-            half8 Q;
-            auto params = [&](int m) {
-                const uint32_t at = stl + (uint32_t)min(m, last) * 128;
-                e0 = lds_at<uint4v>(at);
-                e1 = lds_at<uint4v>(at + 16);
-            };
-            auto offsets = [&](int m) {
-                const uint32_t at = stl + (uint32_t)min(m, last) * 128;
-                xo = lds_at<uint32_t>(at);
-                no = lds_at<uint32_t>(at + 24);
-            };
-            auto raws = [&](uint32_t xoff, uint32_t noff) {
+            // One pointer walks this lane's struct: A rows and parameters of the unit.  The codes of a
+            // unit and its parameters are requested while the previous unit's table words are on their
+            // way (every parameter row names the byte offset of the unit after it).
+            uint32_t qp = qs_l;
+            uint32_t np = knrow_l;
+            uint32_t n16 = lds_at<uint16_t>(np);                           // norm of the current segment
+            float4v D1 = {0, 0, 0, 0}, D2 = {0, 0, 0, 0};                  // sums over the segment's units: heads 0..3, 4..7
+            uint4v pa = lds_at<uint4v>(qp + QS_PA), pb = lds_at<uint4v>(qp + QS_PB);
+            uint32_t xk = krow_l + kfirst;                                 // byte address of the unit whose codes are read next
+            uint2v r = {lds_codes4(xk), 0};
+            auto segment_done = [&]() {
+                const float n = bgtq_h2f((uint16_t)n16) * c2;
+                np += 2;
+                n16 = lds_at<uint16_t>(np);                                // (past the last segment: unused)
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const uint32_t at = krow0 + xoff + k * kstride;
-                    rlo[k] = lds_at<uint32_t>(at);
-                    rhi[k] = lds_at<uint32_t>(at + 4);
-                    nrm[k] = lds_at<uint16_t>(knrow0 + noff + k * (32u * kn_st));
+                for (int e = 0; e < 4; e++) S[e] = fmaf(n, D1[e], S[e]);
+                D1 = (float4v){0, 0, 0, 0};
+                if (two) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) S[4 + e] = fmaf(n, D2[e], S[4 + e]);
+                    D2 = (float4v){0, 0, 0, 0};
                 }
             };
-            auto addresses = [&]() {                        // bit fields -> table addresses
-                const uint32_t lb = (lane4 & e0.w) + e0.z;
-                const uint32_t pw = e1.x, pw2 = pw * 2, pw3 = pw * 3, tsh = e1.y;
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const uint32_t raw = __builtin_amdgcn_alignbyte(rhi[k], rlo[k], e0.y);
-                    ad[k][0] = (__builtin_amdgcn_ubfe(raw, 0, pw) << tsh) + lb;
-                    ad[k][1] = (__builtin_amdgcn_ubfe(raw, pw, pw) << tsh) + lb;
-                    ad[k][2] = (__builtin_amdgcn_ubfe(raw, pw2, pw) << tsh) + lb;
-                    ad[k][3] = (__builtin_amdgcn_ubfe(raw, pw3, pw) << tsh) + lb;
-                }
-            };
-            auto tables = [&](int m) {                      // table words and the query operand of step m
-                Q = lds_at<half8>(qbl + (uint32_t)m * 1024);
-#pragma unroll
-                for (int k = 0; k < 4; k++)
-                    w[k] = (uint4v){lds_at<uint32_t>(ad[k][0]), lds_at<uint32_t>(ad[k][1]),
-                                   lds_at<uint32_t>(ad[k][2]), lds_at<uint32_t>(ad[k][3])};
-            };
-            auto multiply = [&]() {                         // table words times their segment's norm, then the MFMAs
-                uint4v x[4], y[4];
-#pragma unroll
-                for (int k = 0; k < 4; k++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        uint32_t hi, lo;
-                        scale_pair(w[k][i], ncur[k], hi, lo);
-                        x[k][i] = hi;
-                        y[k][i] = lo;
-                    }
-#pragma unroll
-                for (int k = 0; k < 4; k++)
-                    S[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, x[k]), Q, S[k], 0, 0, 0);
-#pragma unroll
-                for (int k = 0; k < 4; k++)
-                    S[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, y[k]), Q, S[k], 0, 0, 0);
-            };
-            auto latch_norms = [&]() {
-#pragma unroll
-                for (int k = 0; k < 4; k++) ncur[k] = nrm[k];
-            };
-            if (n_packed > 0) {
-                params(0);
-                offsets(1);
-                const uint32_t x1 = xo, n1 = no;
-                offsets(2);
-                raws(e0.x, e1.z);                           // step 0
-                addresses();
-                latch_norms();
+            int u = 0;
+            for (; u < n_pair; u++) {
+                const uint32_t base = and_or_v(rep, pb.z, pb.y);
+                uint32_t ad0 = __builtin_amdgcn_alignbit(r.x, r.x, pa.x);
+                uint32_t ad1 = __builtin_amdgcn_alignbit(r.x, r.x, pa.y);
+                uint32_t ad2 = __builtin_amdgcn_alignbit(r.x, r.x, pa.z);
+                uint32_t ad3 = __builtin_amdgcn_alignbit(r.x, r.x, pa.w);
+                xk = krow_l + pb.w;
                 __builtin_amdgcn_sched_barrier(0);
-                params(1);
-                raws(x1, n1);                               // step 1
+                ad0 = and_or_v(ad0, pb.x, base);
+                ad1 = and_or_v(ad1, pb.x, base);
+                ad2 = and_or_v(ad2, pb.x, base);
+                ad3 = and_or_v(ad3, pb.x, base);
                 __builtin_amdgcn_sched_barrier(0);
-                tables(0);
-                for (int m = 0; m < last; m++) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    addresses();                            // step m+1
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply();                             // step m
-                    latch_norms();                          // norms of step m+1
-                    __builtin_amdgcn_sched_barrier(0);
-                    params(m + 2);
-                    raws(xo, no);                           // step m+2
-                    offsets(m + 3);
-                    __builtin_amdgcn_sched_barrier(0);
-                    tables(m + 1);
-                }
+                r.x = lds_codes4(xk);
+                pa = lds_at<uint4v>(qp + 16 + QS_PA);
+                pb = lds_at<uint4v>(qp + 16 + QS_PB);
+                uint4v W;
+                W[0] = lds_at<uint32_t>(ad0);
+                W[1] = lds_at<uint32_t>(ad1);
+                W[2] = lds_at<uint32_t>(ad2);
+                W[3] = lds_at<uint32_t>(ad3);
+                const half8 A1 = lds_at<half8>(qp);
+                half8 A2 = A1;
+                if (two) A2 = lds_at<half8>(qp + QS_A2);
                 __builtin_amdgcn_sched_barrier(0);
-                multiply();
+                const half8 Bk = __builtin_bit_cast(half8, W);
+                D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, Bk, D1, 0, 0, 0);
+                if (two) D2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, Bk, D2, 0, 0, 0);
+                qp += 16;
+                if ((kend >> u) & 1u) segment_done();
             }
-            // raw-byte steps (codes of 5..8 bits): one table read per code
-            for (int m = n_packed; m < n_steps; m++) {
-                const uint4v f0 = lds_at<uint4v>(stl + m * 128), f1 = lds_at<uint4v>(stl + m * 128 + 16);
-                const half8 Qr = lds_at<half8>(qbl + (uint32_t)m * 1024);
+            if (u < n_units) r = lds_codes8(xk);
+            for (; u < n_units; u++) {
+                // one byte and one table read per code
+                uint4v W;
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const uint32_t at = krow0 + f0.x + k * kstride;
-                    const uint32_t lo = lds_at<uint32_t>(at), hi = lds_at<uint32_t>(at + 4), hi2 = lds_at<uint32_t>(at + 8);
-                    const uint32_t n16 = lds_at<uint16_t>(knrow0 + f1.z + k * (16u * kn_st * 2));
-                    const uint32_t r0 = __builtin_amdgcn_alignbyte(hi, lo, f0.y);
-                    const uint32_t r1 = __builtin_amdgcn_alignbyte(hi2, hi, f0.y);
-                    uint4v x, y;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const uint32_t r = e < 2 ? r0 : r1;
-                        const uint32_t b0 = (r >> ((e & 1) * 16)) & 0xFF, b1 = (r >> ((e & 1) * 16 + 8)) & 0xFF;
-                        const uint32_t c0 = lds_at<uint16_t>(f0.z + b0 * 2), c1 = lds_at<uint16_t>(f0.z + b1 * 2);
-                        uint32_t hi, lo;
-                        scale_pair(c0 | (c1 << 16), n16, hi, lo);
-                        x[e] = hi;
-                        y[e] = lo;
-                    }
-                    S[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, x), Qr, S[k], 0, 0, 0);
-                    S[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, y), Qr, S[k], 0, 0, 0);
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t x = e < 2 ? r.x : r.y;
+                    const uint32_t c0 = pb.y + ((x >> ((e & 1) * 16)) & 0xFF) * 2;
+                    const uint32_t c1 = pb.y + ((x >> ((e & 1) * 16 + 8)) & 0xFF) * 2;
+                    W[e] = (uint32_t)lds_at<uint16_t>(c0) | ((uint32_t)lds_at<uint16_t>(c1) << 16);
                 }
+                const half8 A1 = lds_at<half8>(qp);
+                half8 A2 = A1;
+                if (two) A2 = lds_at<half8>(qp + QS_A2);
+                r = lds_codes8(krow_l + pb.w);
+                pb = lds_at<uint4v>(qp + 16 + QS_PB);
+                const half8 Bk = __builtin_bit_cast(half8, W);
+                D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, Bk, D1, 0, 0, 0);
+                if (two) D2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, Bk, D2, 0, 0, 0);
+                qp += 16;
+                if ((kend >> u) & 1u) segment_done();
             }
         }
         asm volatile("" ::: "memory");
@@ -479,88 +508,95 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         int k_loads = 0;
         if (more) k_loads = issue_k(tile + step_tiles);      // all reads of the K buffer are done
 
-        // ---- online softmax: lane (head li, group lg) holds tokens 16k + 4lg + r ------
-        if (nt < MT) {
+        // ---- online softmax: lane = token ----------------------------------------------------
+        const bool live = lane < nt;
+        float d[8];
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int tk = (r >> 2) * 16 + lg * 4 + (r & 3);
-                if (tk >= nt) S[r >> 2][r & 3] = -INFINITY;
+        for (int hh = 0; hh < 8; hh++) d[hh] = S[hh] - m_ref[hh];
+        float mx = fmaxf(fmaxf(fmaxf(d[0], d[1]), fmaxf(d[2], d[3])), fmaxf(fmaxf(d[4], d[5]), fmaxf(d[6], d[7])));
+        if (__builtin_amdgcn_ballot_w64(live && mx > 0.f)) {   // wave-uniform, rare after the first tiles
+            float alpha[8];
+#pragma unroll
+            for (int hh = 0; hh < 8; hh++) {
+                const float wm = wave_max(live ? S[hh] : -INFINITY);
+                const float m_new = wm > m_ref[hh] ? wm + REFRESH : m_ref[hh];
+                alpha[hh] = (m_ref[hh] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref[hh] - m_new);
+                l_part[hh] *= alpha[hh];
+                m_ref[hh] = m_new;
+                d[hh] = S[hh] - m_new;
+            }
+            // acc rows are heads 4(lg & 1) + r
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t pick = (lg & 1) ? 0xFFFFFFFFu : 0u;     // (bitwise: keeps the factors in registers)
+                const float al = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, alpha[4 + r]) & pick) |
+                                                           (__builtin_bit_cast(uint32_t, alpha[r]) & ~pick));
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[e][r] *= al;
             }
         }
-        float mx = S[0][0];
+        // P * v_norm, formed in fp32 and rounded to fp16 once, goes to LDS as [head][token]
+        {
+            const float vn = live ? bgtq_h2f((uint16_t)vraw) : 0.f;
 #pragma unroll
-        for (int r = 1; r < 16; r++) mx = fmaxf(mx, S[r >> 2][r & 3]);
-        mx *= c2;
-        if (__builtin_amdgcn_ballot_w64(mx > m_ref)) {    // wave-uniform, rare after the first tiles
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_ref, mx + REFRESH);
-            const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
-            // acc rows are columns 4lg+r (head (4lg + r) & 7 where columns 8..15 repeat heads 0..7), not
-            // this lane's: fetch their factors
-            float al[4];
-#pragma unroll
-            for (int r = 0; r < 4; r++) al[r] = __shfl(alpha, lg * 4 + r, 64);
-#pragma unroll
-            for (int e = 0; e < NACC; e++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) acc[e][r] *= al[r];
-            l_part *= alpha;
-            m_ref = m_new;
+            for (int hh = 0; hh < 8; hh++) {
+                const float pe = live ? __builtin_amdgcn_exp2f(d[hh]) : 0.f;
+                l_part[hh] += pe;
+                lds_put<uint16_t>(p_wr + hh * PROW, bgtq_f2h(pe * vn));
+            }
         }
         wait_loads(k_loads);                                 // the V records of this tile are in LDS
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();
 
-        if constexpr (DENSE) {
-            // values, at most 8 heads.  The product runs over (token, dim parity) pairs: A row
-            // (head h, parity e') holds P[h][t] in slot (t, e') and zero in slot (t, 1 - e'), B
-            // column c of accumulator jb holds the table word of token t = dims (8c + 2jb, + 1) in
-            // slots (t, 0), (t, 1).  D[(h, e')][c] is then out[h][8c + 2jb + e'], a table word
-            // is an MFMA operand as it comes, and the 8 head rows that would repeat rows 0..7
-            // carry the odd dims instead.  Lane (c = li, lg) decodes unit c of tokens 4lg .. 4lg+3
-            // of every 16-token block; raw codes are fetched one block ahead.
-            const uint32_t pmask = (li & 8) ? 0xFFFF0000u : 0x0000FFFFu;
+        {
+            // values.  The product runs over (token, dim parity) pairs: A row (head h, parity e')
+            // holds P[h][t] in slot (t, e') and zero in slot (t, 1 - e'), B column c of accumulator jb
+            // holds the table word of token t = dims (8c + 2jb, + 1) in slots (t, 0), (t, 1).
+            // D[(h, e')][c] is then out[h][8c + 2jb + e'], a table word is an MFMA operand as it
+            // comes, and the 8 head rows that would repeat rows 0..7 carry the odd dims instead.
+            // Lane (c = li, lg) decodes unit c of tokens 4lg .. 4lg+3 of every 16-token block; raw
+            // codes are fetched one block ahead.
             uint32_t vlo[4], vhi[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                vlo[i] = lds_at<uint32_t>(vbase + (uint32_t)i * vrow);
-                vhi[i] = lds_at<uint32_t>(vbase + (uint32_t)i * vrow + 4);
-            }
+            for (int i = 0; i < 4; i++) lds_read2(vbase + (uint32_t)i * vrow, vlo[i], vhi[i]);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const float4v vn4 = lds_at<float4v>(vnf + (k * 16 + lg * 4) * 4);
+                const uint4v pw = lds_at<uint4v>(p_rd + k * 64);
                 uint4v W[4];                                  // [pair of the unit][token]
+                // stage by stage, so that neighbouring instructions do not depend on each other
+                uint32_t raw[4], ad[4][4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint32_t raw = __builtin_amdgcn_alignbyte(vhi[i], vlo[i], v_sh);
+                for (int i = 0; i < 4; i++) raw[i] = __builtin_amdgcn_alignbyte(vhi[i], vlo[i], v_sh);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
                         const int fp = e * 2 * VBW;
-                        const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
-                        W[e][i] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
+                        ad[e][i] = fp <= vshift ? raw[i] << (vshift - fp) : raw[i] >> (fp - vshift);
                     }
-                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
+                        ad[e][i] = and_or(ad[e][i], fmask, vbank);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) W[e][i] = lds_at<uint32_t>(ad[e][i]);
                 __builtin_amdgcn_sched_barrier(0);
                 if (k + 1 < 4) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int tk = (k + 1) * 16 + i;
-                        vlo[i] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
-                        vhi[i] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
-                    }
+                    for (int i = 0; i < 4; i++) lds_read2(vbase + (uint32_t)((k + 1) * 16 + i) * vrow, vlo[i], vhi[i]);
                 }
-                // P * v_norm is formed in fp32, rounded to fp16 once and kept in the half of
-                // the word that belongs to this lane's parity
                 uint4v Pa;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float pe = __builtin_amdgcn_exp2f(fmaf(S[k][i], c2, -m_ref));
-                    l_part += pe;
-                    const float x = pe * vn4[i];
-                    const float2v xx = {x, x};
-                    Pa[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(xx, half2v)) & pmask;
-                }
+                for (int i = 0; i < 4; i++) Pa[i] = pw[i] << p_shift;
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int jb = 0; jb < 4; jb++)
@@ -568,121 +604,50 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                                                                      __builtin_bit_cast(half8, W[jb]), acc[jb], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
-        } else {
-            // values, 9..16 heads: lane (j = li, group lg) decodes unit j of its 8 tokens per half
-            // tile.  Raw codes are fetched one half ahead; the exponentials run while the table
-            // reads fly.
-            uint32_t vlo[8], vhi[8];
-#pragma unroll
-            for (int r = 0; r < 8; r++) {
-                const int tk = (r >> 2) * 16 + (r & 3);                       // + 4lg, folded into vbase
-                vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
-                vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
-            }
-#pragma unroll
-            for (int half = 0; half < 2; half++) {
-                const float4v vn_lo = lds_at<float4v>(vnf + (half * 32 + lg * 4) * 4);        // tokens 4lg .. 4lg+3
-                const float4v vn_hi = lds_at<float4v>(vnf + (half * 32 + 16 + lg * 4) * 4);   // tokens 16+4lg ..
-                uint32_t W[8][4];
-#pragma unroll
-                for (int r = 0; r < 8; r++) {
-                    const uint32_t raw = __builtin_amdgcn_alignbyte(vhi[r], vlo[r], v_sh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        constexpr uint32_t fmask = ((1u << (2 * VBW)) - 1u) << vshift;
-                        const int fp = e * 2 * VBW;
-                        const uint32_t sh = fp <= vshift ? raw << (vshift - fp) : raw >> (fp - vshift);
-                        W[r][e] = lds_at<uint32_t>(and_or(sh, fmask, vbank));
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                if (half + 1 < 2) {
-#pragma unroll
-                    for (int r = 0; r < 8; r++) {
-                        const int tk = (half + 1) * 32 + (r >> 2) * 16 + (r & 3);
-                        vlo[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow);
-                        vhi[r] = lds_at<uint32_t>(vbase + (uint32_t)tk * vrow + 4);
-                    }
-                }
-                // P * v_norm is formed in fp32 and rounded to fp16 once
-                half8 Pm;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int k = half * 2 + (e >> 1), r = (e & 1) * 2;
-                    const float p0 = __builtin_amdgcn_exp2f(fmaf(S[k][r], c2, -m_ref));
-                    const float p1 = __builtin_amdgcn_exp2f(fmaf(S[k][r + 1], c2, -m_ref));
-                    l_part += p0 + p1;
-                    const float4v vn4 = (e >> 1) ? vn_hi : vn_lo;
-                    const float2v pv = {p0 * vn4[r], p1 * vn4[r + 1]};
-                    const half2v ph = __builtin_convertvector(pv, half2v);
-                    Pm[2 * e] = ph[0];
-                    Pm[2 * e + 1] = ph[1];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    half8 Bv;
-                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;   // high or low halves
-#pragma unroll
-                    for (int p = 0; p < 4; p++) {
-                        uint32_t x = __builtin_amdgcn_perm(W[2 * p + 1][e >> 1], W[2 * p][e >> 1], sel);
-                        half2v hv = __builtin_bit_cast(half2v, x);
-                        Bv[2 * p] = hv[0];
-                        Bv[2 * p + 1] = hv[1];
-                    }
-                    acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Pm, Bv, acc[e], 0, 0, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
         }
         asm volatile("" ::: "memory");
-        __builtin_amdgcn_wave_barrier();     // V buffer and norm areas are rewritten from here on
+        __builtin_amdgcn_wave_barrier();     // V buffer, P buffer and norm areas are rewritten from here on
         v_loads = more ? issue_v(tile + step_tiles) : 0;
     }
 
     // ---- merge the waves -------------------------------------------------------------
-    float l_tot = l_part;
-    l_tot += __shfl_xor(l_tot, 16, 64);
-    l_tot += __shfl_xor(l_tot, 32, 64);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();                         // tables and tile buffers are dead from here
-    // Dim d of a row sits at (d & 7) * 16 + (d >> 3); with that column order and a row stride of
-    // MS floats the 64 lanes of every store below fall on 64 different banks.
-    constexpr int MS = DENSE ? MERGE_STRIDE : MERGE_STRIDE - 4;
-    float* mg_m = (float*)smem;              // [nw][16]
-    float* mg_l = mg_m + nw * 16;            // [nw][16]
-    float* mg_o = mg_l + nw * 16;            // [nw][16][MS]
-    if (lane < 16) { mg_m[wave * 16 + lane] = m_ref; mg_l[wave * 16 + lane] = l_tot; }
-    if constexpr (DENSE) {                   // acc[jb][r] = out[head 4(lg & 1) + r][dim 8li + 2jb + (lg >> 1)]
+    // Every wave leaves its reference, denominator and unnormalised sums in its own tile buffers
+    // (dead by now), in the order the merging threads read them: [m 8][l 8][head 8][li 16][lg >> 1][jb 4].
+    // After one barrier thread t of the first gqa * 32 owns head t / 32 and the four dims
+    // 8 li + (lg >> 1) + {0, 2, 4, 6} with (li, lg >> 1) = t % 32 and folds the waves in a fixed order.
+    {
+        float lt[8];
 #pragma unroll
-        for (int jb = 0; jb < 4; jb++)
+        for (int hh = 0; hh < 8; hh++) lt[hh] = wave_sum(l_part[hh]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (lane == 63) {
+            lds_put<float4v>(kbuf, (float4v){m_ref[0], m_ref[1], m_ref[2], m_ref[3]});
+            lds_put<float4v>(kbuf + 16, (float4v){m_ref[4], m_ref[5], m_ref[6], m_ref[7]});
+            lds_put<float4v>(kbuf + 32, (float4v){lt[0], lt[1], lt[2], lt[3]});
+            lds_put<float4v>(kbuf + 48, (float4v){lt[4], lt[5], lt[6], lt[7]});
+        }
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                mg_o[(wave * 16 + (lg & 1) * 4 + r) * MS + (2 * jb + (lg >> 1)) * 16 + li] = acc[jb][r];
-    } else {                                 // acc[e][r] = out[head 4lg + r][dim 8li + e]
-#pragma unroll
-        for (int e = 0; e < 8; e++)
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-                mg_o[(wave * 16 + lg * 4 + r) * MS + e * 16 + li] = acc[e][r];
+        for (int r = 0; r < 4; r++)
+            lds_put<float4v>(kbuf + 64 + ((((lg & 1) * 4 + r) * 16 + li) * 2 + (lg >> 1)) * 16,
+                             (float4v){acc[0][r], acc[1][r], acc[2][r], acc[3][r]});
     }
     __syncthreads();
-    for (int i = tid; i < gqa * D; i += nthr) {
-        const int hq = i / D, d = i - hq * D;
-        const int col = (d & 7) * 16 + (d >> 3);
-        // all reads of a batch go out before the first is used (one LDS round trip per batch)
-        float mw[MAX_WAVES], lw[MAX_WAVES], ow[MAX_WAVES];
+    for (int i = tid; i < gqa * 32; i += nthr) {
+        const int hq = i >> 5, idx = i & 31;
+        float mw[MAX_WAVES], lw[MAX_WAVES];
+        float4v ow[MAX_WAVES];
 #pragma unroll
-        for (int w = 0; w < MAX_WAVES; w++) {
-            const int ww = min(w, nw - 1);
-            mw[w] = mg_m[ww * 16 + hq];
-            lw[w] = mg_l[ww * 16 + hq];
-            ow[w] = mg_o[(ww * 16 + hq) * MS + col];
+        for (int w = 0; w < MAX_WAVES; w++) {                 // all reads go out before the first is used
+            const uint32_t wb = WAVES_OFF + (uint32_t)(min(w, nw - 1) * wave_bytes);
+            mw[w] = lds_at<float>(wb + hq * 4);
+            lw[w] = lds_at<float>(wb + 32 + hq * 4);
+            ow[w] = lds_at<float4v>(wb + 64 + (hq * 32 + idx) * 16);
         }
         float m = -INFINITY;
 #pragma unroll
         for (int w = 0; w < MAX_WAVES; w++) if (w < nw) m = fmaxf(m, mw[w]);
-        float den = 0.f, num = 0.f;
+        float den = 0.f;
+        float4v num = {0, 0, 0, 0};
 #pragma unroll
         for (int w = 0; w < MAX_WAVES; w++) {
             if (w < nw) {
@@ -691,20 +656,22 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                 num += f * ow[w];
             }
         }
-        size_t row = ((size_t)b * a.n_kv * gqa + (size_t)h * gqa + hq) * a.n_splits + c;
-        a.part_out[row * D + d] = (t1 > t0) ? num / den : 0.f;
-        if (d == 0) a.part_lse[row] = (t1 > t0) ? (m + log2f(den)) * 0.69314718055994530942f : -INFINITY;
+        const bool any = t1 > t0;
+        const float inv = any ? 1.f / den : 0.f;
+        const size_t row = ((size_t)b * a.n_kv * gqa + (size_t)h * gqa + hq) * a.n_splits + c;
+        float* dst = a.part_out + row * D + (idx >> 1) * 8 + (idx & 1);
+#pragma unroll
+        for (int jb = 0; jb < 4; jb++) dst[2 * jb] = num[jb] * inv;
+        if (idx == 0) a.part_lse[row] = any ? (m + log2f(den)) * 0.69314718055994530942f : -INFINITY;
     }
 }
 
 // LDS bytes of a work-group of nw waves
 size_t mfma_smem_bytes(const TileLayout& tl, int nw) {
-    size_t need = (size_t)WAVES_OFF + (size_t)nw * (tl.kbuf + tl.vt + VNF_BYTES);
-    size_t merge = (size_t)nw * (32 + 16 * MERGE_STRIDE) * 4;
-    return need > merge ? need : merge;
+    return (size_t)WAVES_OFF + (size_t)nw * wave_lds_bytes(tl);
 }
 
-template <int VBW, int VST, bool DENSE>
+template <int VBW, int VST, bool TWO>
 int launch_kernel(DecodeArgs a, hipStream_t st) {
     a.tl = tile_layout(a.k_row_width, VST, (int)a.kn_st);
     // no more waves than the longest partition has tiles
@@ -715,7 +682,7 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
     const size_t smem = mfma_smem_bytes(a.tl, nw);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
     a.nw = nw;
-    auto kern = decode_mfma_kernel<VBW, VST, DENSE>;
+    auto kern = decode_mfma_kernel<VBW, VST, TWO>;
     // 1: usable, -1: not usable.  Two threads racing through the first call both run the idempotent
     // set-up below and store the same value.
     static std::atomic<int> ready{0};
@@ -737,14 +704,15 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
 
 template <int VBW, int VST>
 int launch(const DecodeArgs& a, hipStream_t st) {
-    return a.gqa <= 8 ? launch_kernel<VBW, VST, true>(a, st) : launch_kernel<VBW, VST, false>(a, st);
+    return a.gqa > 4 ? launch_kernel<VBW, VST, true>(a, st) : launch_kernel<VBW, VST, false>(a, st);
 }
 
 }  // namespace
 
+
 int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     // layout requirements of the fast path; anything else takes the generic kernel
-    if (a.gqa > 16 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
+    if (a.gqa > 8 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
     if ((a.kp_st & 3) || (a.kp_sb & 3) || (a.kp_sh & 3) || ((uintptr_t)a.kp & 3)) return BGTQ_EUNSUPPORTED;
     if ((a.vp_st & 3) || (a.vp_sb & 3) || (a.vp_sh & 3) || ((uintptr_t)a.vp & 3)) return BGTQ_EUNSUPPORTED;
     if (a.kp_st != a.k_row_width) return BGTQ_EUNSUPPORTED;   // K records contiguous

@@ -12,7 +12,7 @@ HEAD_DIM = 128
 MAX_SEGMENTS = 8
 MAX_CENTROIDS = 256
 LUT_BINS = 256
-MAX_STEPS = 8
+MAX_UNITS = 24
 
 K_BITPACKED, K_MIXED = 0, 1
 V_BITPACKED, V_NIBBLE = 0, 1
@@ -36,13 +36,14 @@ PLAN_DTYPE = np.dtype([
     ('v_centroids', '<f4', (16,)), ('v_boundaries', '<f4', (16,)),
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
-    ('n_steps', '<i4', (2,)), ('n_packed_steps', '<i4', (2,)),
-    ('steptab', '<u4', (2, MAX_STEPS, 4, 8)),
+    ('n_units', '<i4', (2,)), ('n_pair_units', '<i4', (2,)),
+    ('kend', '<u4', (2,)), ('kfirst', '<u4', (2,)),
+    ('kprog', '<u4', (2, MAX_UNITS, 8)), ('kunit', '<u4', (2, MAX_UNITS)),
     ('lut_image', '<u4', (2, 13824 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
 ], align=True)
 
 # byte offsets inside lut_image[K_BITPACKED] / lut_image[K_MIXED] (BGTQ_LUT_* / BGTQ_LUTM_* of include/bgtq.h)
-LUT_K = {1: 0, 2: 512, 3: 2560, 4: 10752}
+LUT_K = {3: 0, 2: 8192, 4: 10240, 1: 11264}    # each on a multiple of its size once VLUT_BYTES is added
 LUT_KRAW, LUT_IMAGE_BYTES = 11776, 13824
 LUTM_KRAW = 4096
 VLUT_BYTES = 8192          # the kernel's table area starts with the V table; the K image follows it
@@ -89,58 +90,57 @@ def _raw_table(cb16: np.ndarray, bw: int) -> np.ndarray:
     return raw.view(np.uint32)
 
 
+
+
 def fill_decode_steps(p) -> None:
-    """Derive the MFMA step schedules of both K record layouts and the table images from the
+    """Derive the unit programs of both K record layouts and the table images from the
     segment table, codebooks and V LUT already stored in plan ``p`` (a 0-d structured array)."""
-    p['steptab'][...] = 0
-    p['n_steps'][...] = 0
-    p['n_packed_steps'][...] = 0
+    for f in ('kprog', 'kunit', 'n_units', 'n_pair_units', 'kend', 'kfirst'):
+        p[f][...] = 0
     for layout in (K_BITPACKED, K_MIXED):
         img = np.zeros(LUT_IMAGE_BYTES // 4, dtype=np.uint32)
-        packed, raw = [], []                      # unit rows (the eight words of a steptab entry)
-        n_ptab = 0
+        units, progs, offs = [], [], []     # per unit: dims, parameter row (without the next unit's offset), byte offset
+        n_ptab = n_pair = kend = 0
         for s in range(int(p['n_seg'])):
             bw, ln = int(p['seg_bw'][s]), int(p['seg_len'][s])
             start = int(p['seg_start'][s])
             cb = p['k_codebook_f16'][s]
+            seg_off = int(p['seg_pack_off' if layout == K_BITPACKED else 'seg_mixed_off'][s])
+            n_u = (ln + 7) // 8
             if bw <= 4:
+                if n_pair != len(units):
+                    raise ValueError("a pair-table segment follows a raw-byte segment")
                 if layout == K_BITPACKED:
                     table, unit_bytes, pw = LUT_K[bw], bw, 2 * bw
-                    mask, tsh = (31 * 4, 7) if bw <= 3 else (0, 2)
                     t = _pair_table(cb, bw)
-                    seg_off = int(p['seg_pack_off'][s])
+                    tsh, rep_mask = (7, 31 * 4) if bw <= 3 else (2, 0)
                 else:
-                    table, unit_bytes, pw, mask, tsh = n_ptab * 1024, 4, 8, 0, 2
+                    table, unit_bytes, pw, tsh, rep_mask = n_ptab * 1024, 4, 8, 2, 0
                     t = _byte_pair_table(cb, bw)
-                    seg_off = int(p['seg_mixed_off'][s])
                     n_ptab += 1
                 img[table // 4:table // 4 + t.size] = t
+                row = [(pw * i - tsh) % 32 for i in range(4)] + [((1 << pw) - 1) << tsh, VLUT_BYTES + table, rep_mask]
+                n_pair += n_u
             else:
                 table = (LUT_KRAW if layout == K_BITPACKED else LUTM_KRAW) + (bw - 5) * 512
-                unit_bytes, pw, mask, tsh = 8, 0, 0, 1
                 img[table // 4:table // 4 + 128] = _raw_table(cb, bw)
-                seg_off = int(p['seg_pack_off' if layout == K_BITPACKED else 'seg_mixed_off'][s])
-            for u in range((ln + 7) // 8):
-                off = seg_off + u * unit_bytes
+                unit_bytes = 8
+                row = [0, 0, 0, 0, 0, VLUT_BYTES + table, 0]
+            for u in range(n_u):
                 d0 = start + 8 * u
-                row = (off & ~3, off & 3, VLUT_BYTES + table, mask, pw, tsh, 2 * s, d0 | (min(8, start + ln - d0) << 8))
-                (packed if bw <= 4 else raw).append(row)
-        m = 0
-        for units in (packed, raw):
-            for u0 in range(0, len(units), 4):
-                if m >= MAX_STEPS:
-                    raise ValueError("segment table needs more MFMA steps than the plan holds")
-                for g in range(4):
-                    if u0 + g < len(units):
-                        p['steptab'][layout, m, g] = units[u0 + g]
-                    else:                          # repeat the last unit with an empty query range
-                        row = list(units[-1])
-                        row[7] &= 0xFF
-                        p['steptab'][layout, m, g] = row
-                m += 1
-            if units is packed:
-                p['n_packed_steps'][layout] = m
-        p['n_steps'][layout] = m
+                units.append(d0 | (min(8, start + ln - d0) << 8))
+                progs.append(row)
+                offs.append(seg_off + u * unit_bytes)
+            kend |= 1 << (len(units) - 1)
+        if len(units) > MAX_UNITS:
+            raise ValueError("segment table needs more units than the plan holds")
+        for u, row in enumerate(progs):
+            p['kprog'][layout, u] = row + [offs[u + 1] if u + 1 < len(units) else 0]
+        p['kunit'][layout, :len(units)] = units
+        p['n_units'][layout] = len(units)
+        p['n_pair_units'][layout] = n_pair
+        p['kend'][layout] = kend
+        p['kfirst'][layout] = offs[0] if offs else 0
         p['lut_image'][layout] = img
     vb = int(p['v_bits'])
     p['vlut_image'][...] = 0

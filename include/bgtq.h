@@ -29,12 +29,14 @@ extern "C" {
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
 #define BGTQ_STATIC_SCRATCH_BYTES (8u << 20)  /* partition results of bgtq_decode_attend_static */
-#define BGTQ_MAX_STEPS     8     /* MFMA steps of one K record, see bgtq_head_plan.steptab */
+#define BGTQ_MAX_UNITS     24    /* 8-dim units of one K record, see bgtq_head_plan.kunit */
 /* byte offsets inside bgtq_head_plan.lut_image[BGTQ_K_BITPACKED] (= offsets in the decode kernel's table area) */
-#define BGTQ_LUT_K1      0                       /* 4 entries   x 32 replicas */
-#define BGTQ_LUT_K2      512                     /* 16 entries  x 32 replicas */
-#define BGTQ_LUT_K3      2560                    /* 64 entries  x 32 replicas */
-#define BGTQ_LUT_K4      10752                   /* 256 entries, not replicated */
+/* (every pair table starts on a multiple of its own size in the kernel's table area, which puts the K image
+ * at offset BGTQ_VLUT_BYTES: an entry address is then the table offset OR-ed with the entry's index bits) */
+#define BGTQ_LUT_K3      0                       /* 64 entries  x 32 replicas */
+#define BGTQ_LUT_K2      8192                    /* 16 entries  x 32 replicas */
+#define BGTQ_LUT_K4      10240                   /* 256 entries, not replicated */
+#define BGTQ_LUT_K1      11264                   /* 4 entries   x 32 replicas */
 #define BGTQ_LUT_KRAW    11776                   /* 4 tables x 256 fp16       */
 #define BGTQ_LUT_KEND    13824                   /* end of the K tables       */
 /* the same for lut_image[BGTQ_K_MIXED]: up to 4 byte-indexed tables of 256 entries, then the raw tables */
@@ -101,27 +103,25 @@ typedef struct bgtq_head_plan {
     float    v_rot[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];    /* decode: out = acc @ v_rot */
     /*
      * Decode schedule of the K record for the MFMA attention kernel, one per K
-     * layout (index BGTQ_K_BITPACKED / BGTQ_K_MIXED), in the form the kernel
-     * copies into LDS.  A "unit" is 8 consecutive packed dims of one segment
-     * (zero padded at the segment's end); a step is one 16x16x32 MFMA whose four
-     * lane groups hold one unit each.  Units of segments with at most 4 bits per
-     * code ("packed" units: two codes select one pair-table entry) fill the first
-     * n_packed_steps steps four at a time in segment order, whatever segment
-     * they belong to; the raw-byte units (5..8 bits, one byte and one table read
-     * per code) fill the steps after them.  Every unit is scaled by its own
-     * segment's norm before the MFMA, so a step may mix segments freely.  Lane
-     * groups past the last unit of either kind repeat that unit with an empty
-     * query range.
-     * steptab[l][m][g] (layout l, step m, lane group g):
-     *   [0] byte offset of the unit in the record, rounded down to 4
-     *   [1] byte offset modulo 4
-     *   [2] byte offset of the unit's table from the start of the kernel's table
+     * layout (index BGTQ_K_BITPACKED / BGTQ_K_MIXED).  A "unit" is 8 consecutive
+     * packed dims of one segment (zero padded at the segment's end); the kernel
+     * walks the units in order, every lane decoding the unit of its own token,
+     * accumulates the units of a segment in the MFMA and scales the segment's sum
+     * by the token's norm of that segment.  Units of segments with codes of at most
+     * 4 bits (two codes select one pair-table entry) come first, n_pair_units[l] of
+     * them; the others take one byte and one table read per code.
+     * kprog[l][u] (32 bytes, read by every lane as it is):
+     *   [0..3] pair units: right-rotation that brings code pair 0..3 of the unit (8
+     *       codes, little-endian bit stream) to the bit position of the table's entry index
+     *   [4] mask of the entry index at that position
+     *   [5] byte offset of the segment's table from the start of the kernel's table
      *       area: BGTQ_VLUT_BYTES + offset inside lut_image[l]
-     *   [3] bank-replica mask (lane * 4 & mask selects the replica; 0: not replicated)
-     *   [4] bits per code pair (2 * bw; 8 in the mixed layout; 0 for raw-byte units)
-     *   [5] log2 of the table's entry stride in bytes
-     *   [6] byte offset of the segment's norm inside a token's norm row (2 * segment)
-     *   [7] first packed dim of the unit | number of real dims (0..8) << 8
+     *   [6] bank-replica mask (lane * 4 & mask selects the replica; 0: not replicated)
+     *   [7] byte offset in the record of the NEXT unit (0 after the last; unit 0 starts
+     *       at kfirst[l])
+     * kend[l]: bit u set = unit u is the last of its segment.
+     * kunit[l][u] = first packed dim of unit u | number of real dims (1..8) << 8, units
+     * numbered through the segments in order; 0 past the last unit.
      *
      * lut_image[l]: pair tables, entry (c0 | c1 << bw) = fp16 centroid pair (c0 in the
      * low half).  Bit-packed layout: bw 1..3 at BGTQ_LUT_K1/K2/K3 with every entry
@@ -136,9 +136,12 @@ typedef struct bgtq_head_plan {
      * v_bits), 32 replicas for v_bits <= 3, unreplicated for 4; BGTQ_V_NIBBLE: 256
      * byte-indexed entries, unreplicated).
      */
-    int32_t  n_steps[2];
-    int32_t  n_packed_steps[2];
-    uint32_t steptab[2][BGTQ_MAX_STEPS][4][8];
+    int32_t  n_units[2];
+    int32_t  n_pair_units[2];
+    uint32_t kend[2];
+    uint32_t kfirst[2];
+    uint32_t kprog[2][BGTQ_MAX_UNITS][8];
+    uint32_t kunit[2][BGTQ_MAX_UNITS];
     uint32_t lut_image[2][BGTQ_LUT_IMAGE_BYTES / 4];
     uint32_t vlut_image[2][BGTQ_VLUT_BYTES / 4];
 } bgtq_head_plan;

@@ -211,52 +211,69 @@ def test_plan_struct_mirrors_the_quantizer():
     assert np.allclose(p['v_rot'].reshape(128, 128), p['v_rot_T'].reshape(128, 128).T)
 
 
+def _unit_fields(row):
+    """Fields of a unit's parameter row (include/bgtq.h, bgtq_head_plan.kprog)."""
+    return dict(rot=[int(x) for x in row[0:4]], mask=int(row[4]), table=int(row[5]), rep_mask=int(row[6]),
+                next_off=int(row[7]))
+
+
 @pytest.mark.parametrize("seed,min_bits,max_bits,budget", [(9, 1, 7, 200), (4, 0, 4, 128), (5, 1, 5, 192)])
 def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, budget):
-    """The MFMA step schedules and the table images in the plan, checked against what they stand
-    for: every packed dim of every segment is read exactly once through a query range, unit byte
-    offsets walk each segment's stream, packed units come before raw-byte units, and a pair-table
-    entry (c0 | c1 << bw) holds the two fp16 centroids, in every bank replica."""
+    """The unit programs and the table images in the plan, checked against what they stand for:
+    every packed dim of every segment is read exactly once through a query range, unit byte offsets
+    walk each segment's stream (every row names the offset of the unit after it), the last unit of
+    every segment is flagged, pair-table units come before raw-byte units, the rotations bring every
+    code pair of a unit to the entry-index position of its table, and a pair-table entry
+    (c0 | c1 << bw) holds the two fp16 centroids, in every bank replica."""
     from blockgtq_amd import plan as P
     q, _ = make_quantizer(seed=seed, min_bits=min_bits, max_bits=max_bits, budget=budget)
     p = q.plan()[0]
     n_seg = int(p['n_seg'])
     for layout in (P.K_BITPACKED, P.K_MIXED):
-        n_steps, n_packed = int(p['n_steps'][layout]), int(p['n_packed_steps'][layout])
-        assert 0 <= n_packed <= n_steps <= P.MAX_STEPS and n_steps >= 1
+        n_units = int(p['n_units'][layout])
+        assert 1 <= n_units <= P.MAX_UNITS
+        assert not p['kunit'][layout, n_units:].any() and not p['kprog'][layout, n_units:].any()
         seen = np.zeros(128, dtype=int)
-        next_unit = {s: 0 for s in range(n_seg)}
-        n_ptab = {}
-        for m in range(n_steps):
-            for g in range(4):
-                lo, ph, table, mask, pw, tsh, noff, qd = (int(x) for x in p['steptab'][layout, m, g])
-                off, s, d0, ln = lo + ph, noff // 2, qd & 0xFF, qd >> 8
-                assert lo % 4 == 0 and 0 <= ph < 4 and noff % 2 == 0 and 0 <= s < n_seg
-                bw = int(p['seg_bw'][s])
-                assert (bw <= 4) == (m < n_packed)             # packed units first, raw-byte units after them
-                start, length = int(p['seg_start'][s]), int(p['seg_len'][s])
-                if ln == 0:                                     # a padding lane repeats a real unit
-                    assert (d0 - start) % 8 == 0 and start <= d0 < start + length
-                    continue
-                u = next_unit[s]
-                next_unit[s] += 1
-                assert d0 == start + 8 * u and ln == min(8, start + length - d0)
+        u, n_ptab, n_pair, kend = 0, 0, 0, 0
+        off = int(p['kfirst'][layout])
+        for s in range(n_seg):
+            bw = int(p['seg_bw'][s])
+            start, length = int(p['seg_start'][s]), int(p['seg_len'][s])
+            seg_off = int(p['seg_mixed_off' if layout else 'seg_pack_off'][s])
+            unit_bytes = 8 if bw > 4 else (bw if layout == P.K_BITPACKED else 4)
+            for i in range((length + 7) // 8):
+                f = _unit_fields(p['kprog'][layout, u])
+                d0, ln = int(p['kunit'][layout, u]) & 0xFF, int(p['kunit'][layout, u]) >> 8
+                assert d0 == start + 8 * i and ln == min(8, start + length - d0) and ln >= 1
+                assert off == seg_off + i * unit_bytes
+                off = f['next_off']
                 seen[d0:d0 + ln] += 1
-                seg_off = int(p['seg_mixed_off' if layout else 'seg_pack_off'][s])
                 if bw > 4:
-                    assert off == seg_off + 8 * u and pw == 0 and tsh == 1 and mask == 0
-                    assert table == P.VLUT_BYTES + (P.LUTM_KRAW if layout else P.LUT_KRAW) + (bw - 5) * 512
-                elif layout == P.K_BITPACKED:
-                    assert off == seg_off + bw * u and pw == 2 * bw
-                    assert table == P.VLUT_BYTES + P.LUT_K[bw]
-                    assert (mask, tsh) == ((124, 7) if bw <= 3 else (0, 2))
+                    assert f['rep_mask'] == 0 and f['mask'] == 0
+                    assert f['table'] == P.VLUT_BYTES + (P.LUTM_KRAW if layout else P.LUT_KRAW) + (bw - 5) * 512
                 else:
-                    assert off == seg_off + 4 * u and pw == 8 and (mask, tsh) == (0, 2)
-                    n_ptab.setdefault(s, len(n_ptab))
-                    assert table == P.VLUT_BYTES + 1024 * n_ptab[s]
+                    assert n_pair == u                    # no raw-byte unit so far
+                    n_pair += 1
+                    if layout == P.K_BITPACKED:
+                        pw, tsh = 2 * bw, (7 if bw <= 3 else 2)
+                        assert f['table'] == P.VLUT_BYTES + P.LUT_K[bw]
+                        assert f['rep_mask'] == (124 if bw <= 3 else 0)
+                    else:
+                        pw, tsh = 8, 2
+                        assert f['table'] == P.VLUT_BYTES + 1024 * n_ptab and f['rep_mask'] == 0
+                    assert f['mask'] == ((1 << pw) - 1) << tsh
+                    unit = 0x9E3779B9 & ((1 << (4 * pw)) - 1)            # any bit pattern of the unit's width
+                    for k in range(4):
+                        rot = ((unit >> f['rot'][k]) | (unit << (32 - f['rot'][k]))) & 0xFFFFFFFF
+                        assert (rot & f['mask']) >> tsh == (unit >> (pw * k)) & ((1 << pw) - 1)
+                u += 1
+            if bw <= 4 and layout == P.K_MIXED:
+                n_ptab += 1
+            kend |= 1 << (u - 1)
+        assert u == n_units and off == 0
+        assert int(p['n_pair_units'][layout]) == n_pair and int(p['kend'][layout]) == kend
         z = int(p['n_zero_dims'])
         assert (seen[z:] == 1).all() and (seen[:z] == 0).all()
-        assert all(next_unit[s] == (int(p['seg_len'][s]) + 7) // 8 for s in range(n_seg))
     img = p['lut_image'][P.K_BITPACKED]
     imgm = p['lut_image'][P.K_MIXED]
     i_ptab = 0
@@ -307,30 +324,35 @@ def test_v_packing_matches_a_plain_bit_stream(bits):
 
 # ---------------------------------------------------------------- library surface
 def _emulate_steps(p, rec, norms, qrot, layout):
-    """Scores of one token record computed the way the MFMA kernel walks the plan's step table:
-    per (step, lane group) one unit of 8 codes through the pair table (or the raw-byte table),
-    times the unit's query range, times the norm of the unit's segment."""
+    """Scores of one token record computed the way the MFMA kernel walks the plan: unit after unit,
+    8 codes through the unit's pair table (rotate, mask, read) or raw-byte table times the unit's
+    query range, summed over a segment (up to the unit flagged as its last), times the segment's norm."""
     from blockgtq_amd import plan as P
     img = p['lut_image'][layout].view(np.uint8)
-    ns, npk = int(p['n_steps'][layout]), int(p['n_packed_steps'][layout])
     out = np.zeros(qrot.shape[0])
     recp = np.concatenate([rec, np.zeros(16, np.uint8)])
-    for m in range(ns):
-        for g in range(4):
-            lo, ph, table, _mask, pw, tsh, noff, qd = (int(x) for x in p['steptab'][layout, m, g])
-            off, d0, ln = lo + ph, qd & 0xFF, qd >> 8
-            if ln == 0:
-                continue
-            table -= P.VLUT_BYTES
-            if m < npk:
-                raw = int.from_bytes(recp[off:off + 8].tobytes(), 'little')
-                vals = []
-                for i in range(4):
-                    a = table + (((raw >> (i * pw)) & ((1 << pw) - 1)) << tsh)
-                    vals += list(img[a:a + 4].view(np.float16))
-            else:
-                vals = [img[table + (int(recp[off + i]) << tsh):][:2].view(np.float16)[0] for i in range(8)]
-            out += (qrot[:, d0:d0 + ln].astype(np.float64) @ np.array(vals[:ln], np.float64)) * float(norms[noff // 2])
+    seg_sum = np.zeros(qrot.shape[0])
+    off, s = int(p['kfirst'][layout]), 0
+    for u in range(int(p['n_units'][layout])):
+        f = _unit_fields(p['kprog'][layout, u])
+        table = f['table'] - P.VLUT_BYTES
+        d0, ln = int(p['kunit'][layout, u]) & 0xFF, int(p['kunit'][layout, u]) >> 8
+        if u < int(p['n_pair_units'][layout]):
+            raw = int.from_bytes(recp[off:off + 4].tobytes(), 'little')
+            vals = []
+            for k in range(4):
+                rot = ((raw >> f['rot'][k]) | (raw << (32 - f['rot'][k]))) & 0xFFFFFFFF
+                a = table + (rot & f['mask'])
+                vals += list(img[a:a + 4].view(np.float16))
+        else:
+            vals = [img[table + 2 * int(recp[off + k]):][:2].view(np.float16)[0] for k in range(8)]
+        seg_sum += qrot[:, d0:d0 + ln].astype(np.float64) @ np.array(vals[:ln], np.float64)
+        off = f['next_off']
+        if (int(p['kend'][layout]) >> u) & 1:
+            out += seg_sum * float(norms[s])
+            seg_sum[:] = 0
+            s += 1
+    assert s == int(p['n_seg'])
     return out
 
 
