@@ -72,7 +72,7 @@ constexpr float REFRESH = 4.0f;
 // (query units are followed by the segment parameters)
 constexpr int VTAB_BYTES = BGTQ_VLUT_BYTES;
 constexpr int KTAB_BYTES = BGTQ_LUT_IMAGE_BYTES;
-constexpr int UROW = MAX_UNITS * 16;                            // one 16-byte slot per unit
+constexpr int UROW = (MAX_UNITS + 2) * 16;                      // one 16-byte slot per unit (+ 2: the look-ahead of the last units)
 // What a lane reads per unit sits behind one pointer: its A rows for both MFMAs and the unit's
 // parameters.  One struct per A row 0..3 (heads r and r + 4) and one whose A rows are zero (for the
 // lanes outside the unit's lane group); the parameters are repeated in each.  The stride puts the
@@ -82,7 +82,7 @@ constexpr int QSTRUCT = 4 * UROW + 16;
 constexpr int QS_OFF = VTAB_BYTES + KTAB_BYTES;
 constexpr int N_QJOBS = 8 * MAX_UNITS + 5 * 2 * MAX_UNITS + 2 * MAX_UNITS;   // query units, parameter halves, zero rows
 constexpr int WAVES_OFF = QS_OFF + 5 * QSTRUCT;
-constexpr int PROW = MT * 4 + 64;                                // bytes from one head's P row to the next: rows land 16 banks apart
+constexpr int PROW = MT * 4 + 32;                                // bytes from one head's P row to the next: rows land 8 banks apart
 constexpr int PBUF_BYTES = 8 * PROW;                          // P of a tile: [head][token], fp16 in the low half of a dword
 
 __host__ __device__ constexpr int kimg_bytes(int k_layout) { return k_layout == BGTQ_K_MIXED ? BGTQ_LUTM_KEND : BGTQ_LUT_KEND; }
@@ -219,31 +219,30 @@ __device__ __forceinline__ uint32_t and_or_v(uint32_t a, uint32_t mask, uint32_t
     return r;
 }
 
-// Wave-wide sum / maximum through the DPP lane crossbar (no LDS traffic): quads, half rows, rows of
-// 16, then the row results travel to the rows behind them; lane 63 ends up with the total (the
-// maximum is handed to every lane, the sum stays in lane 63).
-template <int CTRL, int ROWS>
-__device__ __forceinline__ float dpp_move(float keep, float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, x),
-                                                                 CTRL, ROWS, 0xF, false));
+// Wave-wide sums / maxima of 8 values at once through the DPP lane crossbar (no LDS traffic): quads,
+// half rows, rows of 16, then the row results travel to the rows behind them; lane 63 ends up with
+// the totals.  The 8 values go through every stage together, so that no instruction reads what the
+// one before it wrote (a DPP source needs two idle issue slots after its producer).
+#define BGTQ_DPP8(op, ctrl)                                                                       \
+    op " %0, %0, %0 " ctrl "\n\t" op " %1, %1, %1 " ctrl "\n\t" op " %2, %2, %2 " ctrl "\n\t"     \
+    op " %3, %3, %3 " ctrl "\n\t" op " %4, %4, %4 " ctrl "\n\t" op " %5, %5, %5 " ctrl "\n\t"     \
+    op " %6, %6, %6 " ctrl "\n\t" op " %7, %7, %7 " ctrl "\n\t"
+#define BGTQ_DPP_REDUCE8(op)                                                                      \
+    "s_nop 1\n\t"                                                                                 \
+    BGTQ_DPP8(op, "quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf")                               \
+    BGTQ_DPP8(op, "quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf")                               \
+    BGTQ_DPP8(op, "row_half_mirror row_mask:0xf bank_mask:0xf")                                   \
+    BGTQ_DPP8(op, "row_mirror row_mask:0xf bank_mask:0xf")                                        \
+    BGTQ_DPP8(op, "row_bcast:15 row_mask:0xa bank_mask:0xf")                                      \
+    BGTQ_DPP8(op, "row_bcast:31 row_mask:0xc bank_mask:0xf")                                      \
+    "s_nop 1\n\t"
+__device__ __forceinline__ void wave_sum8(float (&x)[8]) {            // totals in lane 63
+    asm volatile(BGTQ_DPP_REDUCE8("v_add_f32_dpp")
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]));
 }
-__device__ __forceinline__ float wave_sum(float x) {
-    x += dpp_move<0xB1, 0xF>(0.f, x);          // quad_perm [1,0,3,2]
-    x += dpp_move<0x4E, 0xF>(0.f, x);          // quad_perm [2,3,0,1]
-    x += dpp_move<0x141, 0xF>(0.f, x);         // row_half_mirror
-    x += dpp_move<0x140, 0xF>(0.f, x);         // row_mirror
-    x += dpp_move<0x142, 0xA>(0.f, x);         // row_bcast:15 into rows 1 and 3
-    x += dpp_move<0x143, 0xC>(0.f, x);         // row_bcast:31 into rows 2 and 3
-    return x;                                  // (the total is in lane 63 only)
-}
-__device__ __forceinline__ float wave_max(float x) {
-    x = fmaxf(x, dpp_move<0xB1, 0xF>(x, x));
-    x = fmaxf(x, dpp_move<0x4E, 0xF>(x, x));
-    x = fmaxf(x, dpp_move<0x141, 0xF>(x, x));
-    x = fmaxf(x, dpp_move<0x140, 0xF>(x, x));
-    x = fmaxf(x, dpp_move<0x142, 0xA>(x, x));
-    x = fmaxf(x, dpp_move<0x143, 0xC>(x, x));
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+__device__ __forceinline__ void wave_max8(float (&x)[8]) {            // maxima in lane 63
+    asm volatile(BGTQ_DPP_REDUCE8("v_max_f32_dpp")
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]));
 }
 
 // VBW: bits per V code; VST: bytes from one V record to the next (the record itself is
@@ -277,7 +276,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     const uint16_t* q_src = a.q + b * a.q_sb + (int64_t)h * gqa * a.q_sh;
     const int n_units = min(P.n_units[kl], MAX_UNITS);
     const int n_pair = min(P.n_pair_units[kl], n_units);
-    const uint32_t kend = P.kend[kl], kfirst = P.kfirst[kl];
+    const uint32_t kend = P.kend[kl], kfirst0 = P.kfirst[kl][0], kfirst1 = P.kfirst[kl][1];
     // Job j < N_QJOBS fills one 16-byte slot of the structs: a query unit (head j / MAX_UNITS), one half
     // of a unit's parameters for one struct, or a slot of the all-zero A rows.  The loads of a thread's
     // first job go out here, the slots are written once the streaming loads have been issued.
@@ -346,6 +345,15 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     // The shapes of a full tile are the same for every tile of the partition.
     const DmaShape full_k = dma_shape((int)kph + MT * krow, voff), full_kn = dma_shape((int)knph + MT * kn_st * 2, voff);
     const DmaShape full_vn = dma_shape((int)vnph + MT * 2, voff), full_v = dma_shape((int)vph + MT * vrow, voff);
+    // Sources of the wave's next tile (16-byte aligned: the phase stays in the LDS offset); they move on by
+    // the wave's tile stride after every issue.
+    const int step_tiles = nw * MT;
+    const int64_t first = t0 + wave * MT;
+    const uint8_t* k_src = kp_base - kph + first * krow;
+    const uint8_t* kn_src = kn_base - knph + first * kn_st * 2;
+    const uint8_t* vn_src = vn_base - vnph + first * 2;
+    const uint8_t* v_src = vp_base - vph + first * vrow;
+    const int k_step = step_tiles * krow, kn_step = step_tiles * kn_st * 2, vn_step = step_tiles * 2, v_step = step_tiles * vrow;
     // K records and both norm arrays of a tile go to the K buffer; returns the loads issued.
     auto issue_k = [&](int tile) -> int {
         const int nt = min(MT, t1 - tile);
@@ -355,19 +363,22 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             sn = dma_shape((int)knph + nt * kn_st * 2, voff);
             sv = dma_shape((int)vnph + nt * 2, voff);
         }
-        dma_region<9>(kp_base - kph + (int64_t)tile * krow, kbuf, sk, voff);
-        dma_region<2>(kn_base - knph + (int64_t)tile * kn_st * 2, kbuf + tl.kt, sn, voff);
-        dma_region<1>(vn_base - vnph + (int64_t)tile * 2, kbuf + tl.kt + tl.knr, sv, voff);
+        dma_region<9>(k_src, kbuf, sk, voff);
+        dma_region<2>(kn_src, kbuf + tl.kt, sn, voff);
+        dma_region<1>(vn_src, kbuf + tl.kt + tl.knr, sv, voff);
+        k_src += k_step;
+        kn_src += kn_step;
+        vn_src += vn_step;
         return sk.nfull + sn.nfull + sv.nfull + 3;
     };
     auto issue_v = [&](int tile) -> int {
         const int nt = min(MT, t1 - tile);
         DmaShape sv = full_v;
         if (nt < MT) sv = dma_shape((int)vph + nt * vrow, voff);
-        dma_region<5>(vp_base - vph + (int64_t)tile * vrow, vbuf, sv, voff);
+        dma_region<5>(v_src, vbuf, sv, voff);
+        v_src += v_step;
         return sv.nfull + 1;
     };
-    const int step_tiles = nw * MT;
     int tile = t0 + wave * MT;
     int v_loads = 0;                 // loads of the V tile issued after the current K tile
     if (tile < t1) issue_k(tile);
@@ -432,9 +443,6 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
             uint32_t np = knrow_l;
             uint32_t n16 = lds_at<uint16_t>(np);                           // norm of the current segment
             float4v D1 = {0, 0, 0, 0}, D2 = {0, 0, 0, 0};                  // sums over the segment's units: heads 0..3, 4..7
-            uint4v pa = lds_at<uint4v>(qp + QS_PA), pb = lds_at<uint4v>(qp + QS_PB);
-            uint32_t xk = krow_l + kfirst;                                 // byte address of the unit whose codes are read next
-            uint2v r = {lds_codes4(xk), 0};
             auto segment_done = [&]() {
                 const float n = bgtq_h2f((uint16_t)n16) * c2;
                 np += 2;
@@ -448,39 +456,59 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                     D2 = (float4v){0, 0, 0, 0};
                 }
             };
+            // Pair-table units, two at a time (their count is even): the table words and query rows of
+            // both are requested before the first is used, and so are the codes and parameters of the
+            // two units after them (every parameter row names the byte offset of the unit two on).
+            uint4v paA = lds_at<uint4v>(qp + QS_PA), pbA = lds_at<uint4v>(qp + QS_PB);
+            uint4v paB = lds_at<uint4v>(qp + 16 + QS_PA), pbB = lds_at<uint4v>(qp + 16 + QS_PB);
+            uint32_t xa = krow_l + kfirst0, xb = krow_l + kfirst1;         // byte addresses of the units whose codes are read next
+            uint32_t rA = lds_codes4(xa), rB = lds_codes4(xb);
             int u = 0;
-            for (; u < n_pair; u++) {
-                const uint32_t base = and_or_v(rep, pb.z, pb.y);
-                uint32_t ad0 = __builtin_amdgcn_alignbit(r.x, r.x, pa.x);
-                uint32_t ad1 = __builtin_amdgcn_alignbit(r.x, r.x, pa.y);
-                uint32_t ad2 = __builtin_amdgcn_alignbit(r.x, r.x, pa.z);
-                uint32_t ad3 = __builtin_amdgcn_alignbit(r.x, r.x, pa.w);
-                xk = krow_l + pb.w;
+            for (; u < n_pair; u += 2) {
+                const uint32_t baseA = and_or_v(rep, pbA.z, pbA.y), baseB = and_or_v(rep, pbB.z, pbB.y);
+                uint32_t a0 = __builtin_amdgcn_alignbit(rA, rA, paA.x), a1 = __builtin_amdgcn_alignbit(rA, rA, paA.y);
+                uint32_t a2 = __builtin_amdgcn_alignbit(rA, rA, paA.z), a3 = __builtin_amdgcn_alignbit(rA, rA, paA.w);
+                uint32_t b0 = __builtin_amdgcn_alignbit(rB, rB, paB.x), b1 = __builtin_amdgcn_alignbit(rB, rB, paB.y);
+                uint32_t b2 = __builtin_amdgcn_alignbit(rB, rB, paB.z), b3 = __builtin_amdgcn_alignbit(rB, rB, paB.w);
+                a0 = and_or_v(a0, pbA.x, baseA); a1 = and_or_v(a1, pbA.x, baseA);
+                a2 = and_or_v(a2, pbA.x, baseA); a3 = and_or_v(a3, pbA.x, baseA);
+                b0 = and_or_v(b0, pbB.x, baseB); b1 = and_or_v(b1, pbB.x, baseB);
+                b2 = and_or_v(b2, pbB.x, baseB); b3 = and_or_v(b3, pbB.x, baseB);
+                xa = krow_l + pbA.w;
+                xb = krow_l + pbB.w;
                 __builtin_amdgcn_sched_barrier(0);
-                ad0 = and_or_v(ad0, pb.x, base);
-                ad1 = and_or_v(ad1, pb.x, base);
-                ad2 = and_or_v(ad2, pb.x, base);
-                ad3 = and_or_v(ad3, pb.x, base);
+                uint4v WA, WB;
+                WA[0] = lds_at<uint32_t>(a0); WA[1] = lds_at<uint32_t>(a1);
+                WA[2] = lds_at<uint32_t>(a2); WA[3] = lds_at<uint32_t>(a3);
+                const half8 A1a = lds_at<half8>(qp);
+                half8 A2a = A1a;
+                if (two) A2a = lds_at<half8>(qp + QS_A2);
+                WB[0] = lds_at<uint32_t>(b0); WB[1] = lds_at<uint32_t>(b1);
+                WB[2] = lds_at<uint32_t>(b2); WB[3] = lds_at<uint32_t>(b3);
+                const half8 A1b = lds_at<half8>(qp + 16);
+                half8 A2b = A1b;
+                if (two) A2b = lds_at<half8>(qp + 16 + QS_A2);
+                rA = lds_codes4(xa);
+                rB = lds_codes4(xb);
+                paA = lds_at<uint4v>(qp + 32 + QS_PA);
+                pbA = lds_at<uint4v>(qp + 32 + QS_PB);
+                paB = lds_at<uint4v>(qp + 48 + QS_PA);
+                pbB = lds_at<uint4v>(qp + 48 + QS_PB);
                 __builtin_amdgcn_sched_barrier(0);
-                r.x = lds_codes4(xk);
-                pa = lds_at<uint4v>(qp + 16 + QS_PA);
-                pb = lds_at<uint4v>(qp + 16 + QS_PB);
-                uint4v W;
-                W[0] = lds_at<uint32_t>(ad0);
-                W[1] = lds_at<uint32_t>(ad1);
-                W[2] = lds_at<uint32_t>(ad2);
-                W[3] = lds_at<uint32_t>(ad3);
-                const half8 A1 = lds_at<half8>(qp);
-                half8 A2 = A1;
-                if (two) A2 = lds_at<half8>(qp + QS_A2);
-                __builtin_amdgcn_sched_barrier(0);
-                const half8 Bk = __builtin_bit_cast(half8, W);
-                D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, Bk, D1, 0, 0, 0);
-                if (two) D2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, Bk, D2, 0, 0, 0);
-                qp += 16;
+                const half8 BkA = __builtin_bit_cast(half8, WA);
+                D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1a, BkA, D1, 0, 0, 0);
+                if (two) D2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2a, BkA, D2, 0, 0, 0);
                 if ((kend >> u) & 1u) segment_done();
+                const half8 BkB = __builtin_bit_cast(half8, WB);
+                D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1b, BkB, D1, 0, 0, 0);
+                if (two) D2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2b, BkB, D2, 0, 0, 0);
+                if ((kend >> (u + 1)) & 1u) segment_done();
+                qp += 32;
             }
-            if (u < n_units) r = lds_codes8(xk);
+            // raw-byte units, one at a time: xa, xb are the addresses of the first two, pbA the first one's parameters
+            uint2v r = {0, 0};
+            uint4v pb = pbA;
+            if (u < n_units) r = lds_codes8(xa);
             for (; u < n_units; u++) {
                 // one byte and one table read per code
                 uint4v W;
@@ -494,7 +522,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
                 const half8 A1 = lds_at<half8>(qp);
                 half8 A2 = A1;
                 if (two) A2 = lds_at<half8>(qp + QS_A2);
-                r = lds_codes8(krow_l + pb.w);
+                r = lds_codes8(xb);
+                xb = krow_l + pb.w;
                 pb = lds_at<uint4v>(qp + 16 + QS_PB);
                 const half8 Bk = __builtin_bit_cast(half8, W);
                 D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, Bk, D1, 0, 0, 0);
@@ -515,11 +544,14 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
         for (int hh = 0; hh < 8; hh++) d[hh] = S[hh] - m_ref[hh];
         float mx = fmaxf(fmaxf(fmaxf(d[0], d[1]), fmaxf(d[2], d[3])), fmaxf(fmaxf(d[4], d[5]), fmaxf(d[6], d[7])));
         if (__builtin_amdgcn_ballot_w64(live && mx > 0.f)) {   // wave-uniform, rare after the first tiles
-            float alpha[8];
+            float alpha[8], wm[8];
+#pragma unroll
+            for (int hh = 0; hh < 8; hh++) wm[hh] = live ? S[hh] : -INFINITY;
+            wave_max8(wm);
 #pragma unroll
             for (int hh = 0; hh < 8; hh++) {
-                const float wm = wave_max(live ? S[hh] : -INFINITY);
-                const float m_new = wm > m_ref[hh] ? wm + REFRESH : m_ref[hh];
+                const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wm[hh]), 63));
+                const float m_new = top > m_ref[hh] ? top + REFRESH : m_ref[hh];
                 alpha[hh] = (m_ref[hh] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref[hh] - m_new);
                 l_part[hh] *= alpha[hh];
                 m_ref[hh] = m_new;
@@ -618,7 +650,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     {
         float lt[8];
 #pragma unroll
-        for (int hh = 0; hh < 8; hh++) lt[hh] = wave_sum(l_part[hh]);
+        for (int hh = 0; hh < 8; hh++) lt[hh] = l_part[hh];
+        wave_sum8(lt);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (lane == 63) {
             lds_put<float4v>(kbuf, (float4v){m_ref[0], m_ref[1], m_ref[2], m_ref[3]});

@@ -37,7 +37,7 @@ PLAN_DTYPE = np.dtype([
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
     ('n_units', '<i4', (2,)), ('n_pair_units', '<i4', (2,)),
-    ('kend', '<u4', (2,)), ('kfirst', '<u4', (2,)),
+    ('kend', '<u4', (2,)), ('kfirst', '<u4', (2, 2)), ('reserved1', '<u4', (2,)),
     ('kprog', '<u4', (2, MAX_UNITS, 8)), ('kunit', '<u4', (2, MAX_UNITS)),
     ('lut_image', '<u4', (2, 13824 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
 ], align=True)
@@ -126,21 +126,32 @@ def fill_decode_steps(p) -> None:
                 img[table // 4:table // 4 + 128] = _raw_table(cb, bw)
                 unit_bytes = 8
                 row = [0, 0, 0, 0, 0, VLUT_BYTES + table, 0]
+            if bw > 4 and len(units) % 2:
+                # the kernel takes pair-table units two at a time: an empty unit evens them out
+                units.append(0)
+                progs.append([0] * 7)
+                offs.append(0)
+                n_pair += 1
             for u in range(n_u):
                 d0 = start + 8 * u
                 units.append(d0 | (min(8, start + ln - d0) << 8))
                 progs.append(row)
                 offs.append(seg_off + u * unit_bytes)
             kend |= 1 << (len(units) - 1)
+        if n_pair == len(units) and n_pair % 2:
+            units.append(0)
+            progs.append([0] * 7)
+            offs.append(0)
+            n_pair += 1
         if len(units) > MAX_UNITS:
             raise ValueError("segment table needs more units than the plan holds")
         for u, row in enumerate(progs):
-            p['kprog'][layout, u] = row + [offs[u + 1] if u + 1 < len(units) else 0]
+            p['kprog'][layout, u] = row + [offs[u + 2] if u + 2 < len(units) else 0]
         p['kunit'][layout, :len(units)] = units
         p['n_units'][layout] = len(units)
         p['n_pair_units'][layout] = n_pair
         p['kend'][layout] = kend
-        p['kfirst'][layout] = offs[0] if offs else 0
+        p['kfirst'][layout] = (offs + [0, 0])[:2]
         p['lut_image'][layout] = img
     vb = int(p['v_bits'])
     p['vlut_image'][...] = 0

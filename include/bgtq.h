@@ -109,7 +109,8 @@ typedef struct bgtq_head_plan {
      * accumulates the units of a segment in the MFMA and scales the segment's sum
      * by the token's norm of that segment.  Units of segments with codes of at most
      * 4 bits (two codes select one pair-table entry) come first, n_pair_units[l] of
-     * them; the others take one byte and one table read per code.
+     * them, an even number: an empty unit (kunit 0, parameters 0) is inserted where the
+     * count would be odd; the others take one byte and one table read per code.
      * kprog[l][u] (32 bytes, read by every lane as it is):
      *   [0..3] pair units: right-rotation that brings code pair 0..3 of the unit (8
      *       codes, little-endian bit stream) to the bit position of the table's entry index
@@ -117,8 +118,8 @@ typedef struct bgtq_head_plan {
      *   [5] byte offset of the segment's table from the start of the kernel's table
      *       area: BGTQ_VLUT_BYTES + offset inside lut_image[l]
      *   [6] bank-replica mask (lane * 4 & mask selects the replica; 0: not replicated)
-     *   [7] byte offset in the record of the NEXT unit (0 after the last; unit 0 starts
-     *       at kfirst[l])
+     *   [7] byte offset in the record of the unit after the next (0 if there is none;
+     *       units 0 and 1 start at kfirst[l][0..1])
      * kend[l]: bit u set = unit u is the last of its segment.
      * kunit[l][u] = first packed dim of unit u | number of real dims (1..8) << 8, units
      * numbered through the segments in order; 0 past the last unit.
@@ -139,7 +140,8 @@ typedef struct bgtq_head_plan {
     int32_t  n_units[2];
     int32_t  n_pair_units[2];
     uint32_t kend[2];
-    uint32_t kfirst[2];
+    uint32_t kfirst[2][2];
+    uint32_t reserved1[2];
     uint32_t kprog[2][BGTQ_MAX_UNITS][8];
     uint32_t kunit[2][BGTQ_MAX_UNITS];
     uint32_t lut_image[2][BGTQ_LUT_IMAGE_BYTES / 4];

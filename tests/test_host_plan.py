@@ -212,7 +212,8 @@ def test_plan_struct_mirrors_the_quantizer():
 
 
 def _unit_fields(row):
-    """Fields of a unit's parameter row (include/bgtq.h, bgtq_head_plan.kprog)."""
+    """Fields of a unit's parameter row (include/bgtq.h, bgtq_head_plan.kprog); next_off is the byte
+    offset of the unit after the next."""
     return dict(rot=[int(x) for x in row[0:4]], mask=int(row[4]), table=int(row[5]), rep_mask=int(row[6]),
                 next_off=int(row[7]))
 
@@ -221,8 +222,8 @@ def _unit_fields(row):
 def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, budget):
     """The unit programs and the table images in the plan, checked against what they stand for:
     every packed dim of every segment is read exactly once through a query range, unit byte offsets
-    walk each segment's stream (every row names the offset of the unit after it), the last unit of
-    every segment is flagged, pair-table units come before raw-byte units, the rotations bring every
+    walk each segment's stream (every row names the offset of the unit two on), the last unit of
+    every segment is flagged, pair-table units come before raw-byte units and are an even number, the rotations bring every
     code pair of a unit to the entry-index position of its table, and a pair-table entry
     (c0 | c1 << bw) holds the two fp16 centroids, in every bank replica."""
     from blockgtq_amd import plan as P
@@ -235,18 +236,24 @@ def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, b
         assert not p['kunit'][layout, n_units:].any() and not p['kprog'][layout, n_units:].any()
         seen = np.zeros(128, dtype=int)
         u, n_ptab, n_pair, kend = 0, 0, 0, 0
-        off = int(p['kfirst'][layout])
+        offs = [int(x) for x in p['kfirst'][layout]]          # byte offsets of the units, as the rows chain them
         for s in range(n_seg):
             bw = int(p['seg_bw'][s])
             start, length = int(p['seg_start'][s]), int(p['seg_len'][s])
             seg_off = int(p['seg_mixed_off' if layout else 'seg_pack_off'][s])
             unit_bytes = 8 if bw > 4 else (bw if layout == P.K_BITPACKED else 4)
+            if bw > 4 and u % 2 and n_pair == u:
+                # the empty unit that makes the number of pair-table units even
+                assert int(p['kunit'][layout, u]) == 0 and not p['kprog'][layout, u, :7].any()
+                offs.append(int(p['kprog'][layout, u, 7]))
+                u += 1
+                n_pair += 1
             for i in range((length + 7) // 8):
                 f = _unit_fields(p['kprog'][layout, u])
                 d0, ln = int(p['kunit'][layout, u]) & 0xFF, int(p['kunit'][layout, u]) >> 8
                 assert d0 == start + 8 * i and ln == min(8, start + length - d0) and ln >= 1
-                assert off == seg_off + i * unit_bytes
-                off = f['next_off']
+                assert offs[u] == seg_off + i * unit_bytes
+                offs.append(f['next_off'])
                 seen[d0:d0 + ln] += 1
                 if bw > 4:
                     assert f['rep_mask'] == 0 and f['mask'] == 0
@@ -270,8 +277,13 @@ def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, b
             if bw <= 4 and layout == P.K_MIXED:
                 n_ptab += 1
             kend |= 1 << (u - 1)
-        assert u == n_units and off == 0
-        assert int(p['n_pair_units'][layout]) == n_pair and int(p['kend'][layout]) == kend
+        if n_pair == u and u % 2:                             # all units are pair-table units, an odd number
+            assert int(p['kunit'][layout, u]) == 0 and not p['kprog'][layout, u].any()
+            offs.append(0)
+            u += 1
+            n_pair += 1
+        assert u == n_units and offs[n_units:] == [0, 0]
+        assert int(p['n_pair_units'][layout]) == n_pair and n_pair % 2 == 0 and int(p['kend'][layout]) == kend
         z = int(p['n_zero_dims'])
         assert (seen[z:] == 1).all() and (seen[:z] == 0).all()
     img = p['lut_image'][P.K_BITPACKED]
@@ -332,8 +344,9 @@ def _emulate_steps(p, rec, norms, qrot, layout):
     out = np.zeros(qrot.shape[0])
     recp = np.concatenate([rec, np.zeros(16, np.uint8)])
     seg_sum = np.zeros(qrot.shape[0])
-    off, s = int(p['kfirst'][layout]), 0
+    offs, s = [int(x) for x in p['kfirst'][layout]], 0
     for u in range(int(p['n_units'][layout])):
+        off = offs[u]
         f = _unit_fields(p['kprog'][layout, u])
         table = f['table'] - P.VLUT_BYTES
         d0, ln = int(p['kunit'][layout, u]) & 0xFF, int(p['kunit'][layout, u]) >> 8
@@ -347,7 +360,7 @@ def _emulate_steps(p, rec, norms, qrot, layout):
         else:
             vals = [img[table + 2 * int(recp[off + k]):][:2].view(np.float16)[0] for k in range(8)]
         seg_sum += qrot[:, d0:d0 + ln].astype(np.float64) @ np.array(vals[:ln], np.float64)
-        off = f['next_off']
+        offs.append(f['next_off'])
         if (int(p['kend'][layout]) >> u) & 1:
             out += seg_sum * float(norms[s])
             seg_sum[:] = 0
