@@ -23,6 +23,7 @@ c_f = ctypes.c_float
 _SIGNATURES = {
     "bgtq_plan_sizeof": (ctypes.c_size_t, []),
     "bgtq_abi_version": (c_i, []),
+    "bgtq_decode_kernel_revision": (c_i, []),
     "bgtq_strerror": (ctypes.c_char_p, [c_i]),
     "bgtq_encode_k": (c_i, [c_p, c_p, c_i64, c_i64, c_i64, c_i, c_i, c_i,
                             c_p, c_i64, c_i64, c_i64, c_i,

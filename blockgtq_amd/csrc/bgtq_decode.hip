@@ -795,6 +795,7 @@ int bgtq_window_swap(void* kbuf, void* vbuf, int64_t w_sb, int64_t w_sh, int64_t
 
 size_t bgtq_plan_sizeof(void) { return sizeof(bgtq_head_plan); }
 int bgtq_abi_version(void) { return 3; }
+int bgtq_decode_kernel_revision(void) { return 3; }
 
 const char* bgtq_strerror(int code) {
     switch (code) {

@@ -149,16 +149,19 @@ def fill_cache(mgr: BlockGTQKVManager, w: Workload, energies, device, chunk: int
         mgr.seq_len = w.context
 
 
-def algorithmic_bytes_per_layer(mgr: BlockGTQKVManager, layer: int, seq_lens) -> int:
+def algorithmic_bytes_per_layer(mgr: BlockGTQKVManager, layer: int, seq_lens, nibble: bool = False) -> int:
     """Bytes one decode-attention launch must read/write by construction: every
     visible token's own K record, its fp16 group norms, V record and V norm,
-    plus the queries in and the outputs out."""
+    plus the queries in and the outputs out.  ``nibble``: the records of the
+    production cache's default layout (K as nibbles + raw bytes, V as nibbles)."""
     total = 0
-    vb = mgr._vpb
+    vb = mgr.hd // 2 if nibble else mgr._vpb
+    plans = mgr._batched_args[layer]['plans_np']
     for T_b in seq_lens:
         fp16_rows = min(T_b, mgr.n_sink + mgr.window) if mgr.buffered else 0
-        for q8 in mgr.quantizers[layer]:
-            total += (T_b - fp16_rows) * (q8._total_packed_bytes + 2 * q8._n_groups + vb + 2)
+        for hi, q8 in enumerate(mgr.quantizers[layer]):
+            kb = int(plans[hi]['k_mixed_bytes']) if nibble else q8._total_packed_bytes
+            total += (T_b - fp16_rows) * (kb + 2 * q8._n_groups + vb + 2)
             total += fp16_rows * mgr.hd * 2 * 2            # fp16 K and V rows of the buffer
     total += len(seq_lens) * mgr.n_q * mgr.hd * 2 * 2
     return total

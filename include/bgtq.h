@@ -154,6 +154,12 @@ size_t bgtq_plan_sizeof(void);
 /* Library/ABI version, bumped whenever a signature or the plan struct changes. */
 int bgtq_abi_version(void);
 
+/* Revision of the decode-attention kernels' memory access pattern (tile shapes, what
+ * is staged through LDS, partition scheme).  Figures measured on one revision, such as
+ * HBM traffic per launch, are only quoted while the library reports the same number.
+ * No counterpart in the reference. */
+int bgtq_decode_kernel_revision(void);
+
 /* Human-readable text for a return code of this library (static storage). */
 const char* bgtq_strerror(int code);
 

@@ -3,7 +3,6 @@ packed path's CPU checker and against what the mathematics fixes."""
 import numpy as np
 import pytest
 import torch
-import torch.nn as nn
 
 from blockgtq_amd import BlockGTQPipeline
 from blockgtq_amd.tq import TurboQuantMSE
@@ -68,29 +67,6 @@ def test_turboquant_round_trip(bits, nmse):
     assert abs(float(rel) / nmse - 1) < 0.1, float(rel)
 
 
-class _Attn(nn.Module):
-    def __init__(self, nkv):
-        super().__init__()
-        self.k_proj = nn.Linear(64, nkv * 128, bias=True)
-        self.v_proj = nn.Linear(64, nkv * 128, bias=False)
-
-
-class _Layer(nn.Module):
-    def __init__(self, nkv):
-        super().__init__()
-        self.self_attn = _Attn(nkv)
-
-
-class _Model(nn.Module):
-    def __init__(self, n_layers, nkv):
-        super().__init__()
-        self.model = nn.Module()
-        self.model.layers = nn.ModuleList([_Layer(nkv) for _ in range(n_layers)])
-
-    def forward(self, x, past_key_values=None):
-        return x
-
-
 def _quantizers(n_layers, nkv):
     gen = torch.Generator().manual_seed(2)
     data = {li: {'q': torch.randn(nkv, 512, 128, generator=gen) * torch.linspace(0.2, 3, 128),
@@ -99,59 +75,52 @@ def _quantizers(n_layers, nkv):
     return ua.build_unaccelerated_quantizers(data, n_layers, nkv, 128, device='cpu')
 
 
-def test_patch_wraps_projections_and_unpatch_restores():
-    torch.manual_seed(0)
-    m = _Model(2, 2)
+def test_round_trip_heads_is_the_per_head_reconstruction():
     kq, vq = _quantizers(2, 2)
     assert kq[0][0].rotation_threshold == 1 and vq[1][1].bit_width == 3
-    x = torch.randn(3, 7, 64)
-    attn = m.model.layers[1].self_attn
-    plain_k, plain_v = attn.k_proj(x), attn.v_proj(x)
-    handles = ua.patch_model_kv(m, kq, vq, 128, 2)
-    got_k, got_v = attn.k_proj(x), attn.v_proj(x)
-    assert got_k.shape == plain_k.shape and got_k.dtype == plain_k.dtype
+    g = torch.Generator().manual_seed(5)
+    k = (torch.randn(3, 2, 7, 128, generator=g) * torch.linspace(0.2, 3, 128)).half()
+    v = torch.randn(3, 2, 7, 128, generator=g).half()
+    k_hat, v_hat = ua.round_trip_heads(kq[1], vq[1], k, v)
+    assert k_hat.shape == k.shape and k_hat.dtype == torch.float32 and v_hat.dtype == torch.float32
     for h in range(2):
-        sl = slice(h * 128, (h + 1) * 128)
-        assert torch.allclose(got_k[..., sl], kq[1][h].compress_decompress(plain_k[..., sl].float()), atol=1e-6)
-        assert torch.allclose(got_v[..., sl], vq[1][h].compress_decompress(
-            plain_v[..., sl].reshape(-1, 128).float()).reshape(3, 7, 128), atol=1e-6)
-    cos = torch.nn.functional.cosine_similarity(got_k.flatten(), plain_k.flatten(), dim=0)
-    assert 0.9 < float(cos.detach()) < 1.0
-    ua.unpatch_model_kv(handles)
-    assert torch.equal(attn.k_proj(x), plain_k) and isinstance(attn.k_proj, nn.Linear)
+        for b in range(3):
+            assert torch.allclose(k_hat[b, h], kq[1][h].compress_decompress(k[b, h].float()), atol=1e-6)
+            assert torch.allclose(v_hat[b, h], vq[1][h].compress_decompress(v[b, h].float()), atol=1e-6)
+    cos = torch.nn.functional.cosine_similarity(k_hat.flatten(), k.float().flatten(), dim=0)
+    assert 0.9 < float(cos) < 1.0
+    # heads use their own quantizers: swapping them changes the result
+    swapped, _ = ua.round_trip_heads(kq[1][::-1], vq[1], k, v)
+    assert not torch.allclose(swapped, k_hat)
 
 
-class _Cache:
-    def __init__(self, n_layers, B, nkv, T):
-        g = torch.Generator().manual_seed(1)
-        self.key_cache = [torch.randn(B, nkv, T, 128, generator=g).half() for _ in range(n_layers)]
-        self.value_cache = [torch.randn(B, nkv, T, 128, generator=g).half() for _ in range(n_layers)]
+def test_quantizers_from_allocations_reproduce_calibrated_ones():
+    kq, vq = _quantizers(1, 2)
+    k2, v2 = ua.quantizers_from_allocations([q.bit_allocation for q in kq[0]], 128, 3,
+                                            [1000, 1001], rotation_threshold=1)
+    x = torch.randn(33, 128, generator=torch.Generator().manual_seed(8)) * torch.linspace(0.2, 3, 128)
+    for h in range(2):
+        assert torch.equal(k2[h].compress_decompress(x), kq[0][h].compress_decompress(x))
+        assert torch.equal(v2[h].compress_decompress(x), vq[0][h].compress_decompress(x))
 
 
-def test_buffered_patch_flushes_only_tokens_that_left_the_window():
-    m = _Model(2, 2)
-    kq, vq = _quantizers(2, 2)
-    patch = ua.patch_model_kv_buffered(m, kq, vq, 128, 2, 2, recent_window=16, n_sink_token=4)
-    cache = _Cache(2, 2, 2, 4 + 16 + 3)
-    before_k = [k.clone() for k in cache.key_cache]
-    before_v = [v.clone() for v in cache.value_cache]
-    m(torch.zeros(1), past_key_values=cache)
-    for li in range(2):
-        k, v = cache.key_cache[li], cache.value_cache[li]
-        changed = (k != before_k[li]).any(dim=-1).any(dim=0).any(dim=0)
-        assert changed.tolist() == [False] * 4 + [True] * 3 + [False] * 16
-        assert torch.equal(v[:, :, :4], before_v[li][:, :, :4]) and torch.equal(v[:, :, 7:], before_v[li][:, :, 7:])
-        ref = kq[li][1].compress_decompress(before_k[li][:, 1, 4:7].reshape(-1, 128).float())
-        assert torch.equal(k[:, 1, 4:7].reshape(-1, 128), ref.half())
-        assert patch.state[li]["n_flushed"] == 3
-    snap = [k.clone() for k in cache.key_cache]
-    m(torch.zeros(1), past_key_values=cache)               # nothing new left the window
-    assert all(torch.equal(a, b) for a, b in zip(snap, cache.key_cache))
-    patch.reset()
-    assert patch.state[0]["n_flushed"] == 0
-    patch.remove()
-    m(torch.zeros(1), past_key_values=cache)
-    assert all(torch.equal(a, b) for a, b in zip(snap, cache.key_cache))
+def test_decode_attention_expands_kv_heads_for_their_query_groups():
+    g = torch.Generator().manual_seed(9)
+    B, n_q, nkv, T = 2, 8, 2, 37
+    q = torch.randn(B, n_q, 128, generator=g).half()
+    k = torch.randn(B, nkv, T, 128, generator=g)
+    v = torch.randn(B, nkv, T, 128, generator=g)
+    out = ua.decode_attention(q, k, v)
+    assert out.shape == (B, n_q, 128) and out.dtype == torch.float32
+    assert torch.equal(out, ua.decode_attention(q.unsqueeze(2), k, v))
+    for b in range(B):
+        for hq in range(n_q):
+            h = hq // (n_q // nkv)
+            s = (q[b, hq].double() @ k[b, h].double().T) / 128 ** 0.5
+            ref = torch.softmax(s, -1) @ v[b, h].double()
+            assert torch.allclose(out[b, hq].double(), ref, atol=1e-5)
+    half_scale = ua.decode_attention(q, k, v, scale=0.5 / 128 ** 0.5)
+    assert not torch.allclose(half_scale, out)
 
 
 @pytest.mark.parametrize("k_layout,v_layout", [(0, 0), (1, 1)])
