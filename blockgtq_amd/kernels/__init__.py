@@ -15,17 +15,34 @@ import torch
 
 from .. import ops, plan as _plan
 
-# codebook_flat.data_ptr() -> quantizer that produced it via build_kernel_args()
-_QUANTIZER_OF_CODEBOOK = weakref.WeakValueDictionary()
+# id(codebook_flat tensor object) -> (weak reference to that tensor, weak reference to the quantizer
+# that produced it via build_kernel_args()).  The tensor OBJECT is the key, not its address: memory
+# of a freed codebook can be handed to another tensor, an id is only trusted while its object lives.
+_QUANTIZER_OF_CODEBOOK = {}
 
 
 def register_kernel_args(kernel_args: dict):
     """Remember which quantizer a ``build_kernel_args`` dict came from, so the
     fused entry can find that head's device plan from ``codebook_flat`` alone."""
     q = kernel_args.get('quantizer')
-    if q is not None and kernel_args['codebook_flat'].numel():
-        _QUANTIZER_OF_CODEBOOK[kernel_args['codebook_flat'].data_ptr()] = q
+    t = kernel_args['codebook_flat']
+    if q is not None and t.numel():
+        key = id(t)
+
+        def forget(ref, key=key):
+            if _QUANTIZER_OF_CODEBOOK.get(key, (None,))[0] is ref:
+                del _QUANTIZER_OF_CODEBOOK[key]
+
+        _QUANTIZER_OF_CODEBOOK[key] = (weakref.ref(t, forget), weakref.ref(q))
     return kernel_args
+
+
+def _quantizer_of(codebook_flat):
+    """The quantizer registered for exactly this tensor object, if it is still alive."""
+    entry = _QUANTIZER_OF_CODEBOOK.get(id(codebook_flat))
+    if entry is None or entry[0]() is not codebook_flat:
+        return None
+    return entry[1]()
 
 
 def _plan_from_args(codebook_flat, segments, v_lut, v_rotation, v_bits, device):
@@ -103,7 +120,7 @@ def fused_blockgtq_decode_attention(
     T = k_packed.shape[2]
     if q_pack_perm is not None:
         q = q[:, :, :, q_pack_perm]
-    quant = _QUANTIZER_OF_CODEBOOK.get(codebook_flat.data_ptr()) if codebook_flat.numel() else None
+    quant = _quantizer_of(codebook_flat)
     if quant is not None:
         plans = quant.device_plan()
     else:
@@ -152,7 +169,7 @@ def fused_blockgtq_prefill_attention(
     if k_packed.shape[1] != 1:
         raise NotImplementedError("pass one KV head per call (each head owns its plan)")
     T = k_packed.shape[2]
-    quant = _QUANTIZER_OF_CODEBOOK.get(codebook_flat.data_ptr()) if codebook_flat.numel() else None
+    quant = _quantizer_of(codebook_flat)
     if quant is not None:
         plans = quant.device_plan()
     else:

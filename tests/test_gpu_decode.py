@@ -78,6 +78,8 @@ CASES = [  # budget mn mx vb n_kv gqa B T k_layout v_layout
     (192, 1, 8, 3, 2, 8, 2, 777, 0, 0),
     (192, 1, 8, 3, 2, 8, 2, 777, 1, 1),
     (128, 0, 4, 2, 2, 4, 1, 1500, 0, 0),
+    (128, 0, 4, 2, 2, 4, 1, 700, 1, 1),        # 0-bit blocks in the nibble record
+    (160, 0, 8, 3, 2, 8, 2, 300, 1, 0),        # 0-bit blocks, nibbles and raw bytes
     (300, 2, 8, 4, 1, 16, 1, 300, 0, 0),
     (300, 2, 8, 4, 1, 16, 1, 300, 1, 0),
     (64, 1, 1, 1, 1, 1, 3, 64, 0, 1),
@@ -213,6 +215,16 @@ def test_production_cache_and_fused_entry(oracle_lib):
         assert o.shape == (1, 4, 1, 128)
         assert np.abs(o[0, :, 0].float().cpu().numpy() - ref[0, hi * 4:(hi + 1) * 4]).max() < TOL
         assert np.abs(lse[0].cpu().numpy() - ref_lse[0, hi * 4:(hi + 1) * 4]).max() < LSE_TOL
+        # the same call with tensors this package has never seen (copies of the codebook, the V table
+        # and the V rotation): the entry must assemble the head's plan from its arguments alone
+        o2, lse2 = fused_blockgtq_decode_attention(
+            q_h, cache.k_packed[0, :, hi:hi + 1, :Tn], cache.k_norms[0, :, hi:hi + 1, :Tn],
+            a['codebook_flat'].clone(), a['lut_offset'], a['norm_group'], list(a['segments_b']),
+            cache.v_packed[0, :, hi:hi + 1, :Tn], cache.v_norms[0, :, hi:hi + 1, :Tn], q8.v_lut.clone(),
+            scale=cache.scale, t_splits=8, v_bits=3, v_rotation=q8._v_rot.clone(),
+            k_nibble=True, v_nibble=True, return_lse=True)
+        assert np.abs(o2[0, :, 0].float().cpu().numpy() - ref[0, hi * 4:(hi + 1) * 4]).max() < TOL
+        assert np.abs(lse2[0].cpu().numpy() - ref_lse[0, hi * 4:(hi + 1) * 4]).max() < LSE_TOL
 
 
 def test_full_size_properties_config1():
@@ -373,6 +385,66 @@ def test_with_buffer_manager_keeps_sink_and_window_in_fp16(oracle_lib):
                 ref = p @ np.concatenate([vd, hist_v[b, h, fp].astype(np.float64)], 0)
                 got = out[b, h * gqa:(h + 1) * gqa]
                 assert np.abs(got - ref).max() < TOL, (step, b, h, np.abs(got - ref).max())
+
+
+def test_with_buffer_manager_at_the_full_ragged_shape(oracle_lib, decode_path):
+    """The ragged with-buffer workload at its stated shape, one layer: 32 sequences of 1024..16384
+    tokens, 32 query / 8 KV heads, 4 fp16 sink tokens, 128-token fp16 window, two appends through
+    the manager.  Three (row, head) pairs are checked against one fp64 softmax over
+    [sink | dequantised middle | window] built from the checker's records; all rows and heads
+    must agree between two managers that partition the context differently."""
+    if decode_path == "generic":
+        pytest.skip("the layout-agnostic kernel is covered at this shape's reduced size above")
+    w = wl.WORKLOADS["qwen3_8b_b32_ragged_buffered"]
+    lens = list(w.seq_lens)
+    Tmax, steps, ns, win, gqa = max(lens), 2, w.n_sink, w.window, w.n_q // w.n_kv
+    assert w.batch == 32 and w.n_kv == 8 and min(lens) >= 1024 and Tmax <= 16384 and (ns, win) == (4, 128)
+    mgrs = []
+    for n_splits in (0, 5):
+        mgr, energies = wl.build_manager(w, DEV, max_T=Tmax + steps + 8, n_layers=1)
+        mgr.n_splits = n_splits
+        mgrs.append(mgr)
+    hist_k, hist_v = wl.draw_kv(w, energies[0], Tmax + steps, 0, DEV)
+    for mgr in mgrs:
+        mgr.fill_buffered(0, hist_k[:, :, :Tmax], hist_v[:, :, :Tmax], lens)
+        mgr.set_seq_lens(lens)
+    plans_np = mgrs[0]._batched_args[0]['plans_np']
+    rows = [int(np.argmin(lens)), int(np.argmax(lens)), 7]
+    pairs = list(zip(rows, (0, 7, 3)))
+    ar = torch.arange(w.batch, device=DEV)
+    gen = torch.Generator().manual_seed(31)
+    for step in range(steps):
+        q = torch.randn(w.batch, w.n_q, 1, 128, generator=gen).half().to(DEV)
+        at = torch.tensor(lens, device=DEV)
+        k1 = hist_k[ar, :, at].unsqueeze(2).contiguous()
+        v1 = hist_v[ar, :, at].unsqueeze(2).contiguous()
+        outs = [mgr.append_and_attend(0, q, k1, v1)[:, :, 0].float() for mgr in mgrs]
+        for mgr in mgrs:
+            mgr.increment_seq_len()
+        lens = [t + 1 for t in lens]
+        assert torch.isfinite(outs[0]).all()
+        assert (outs[0] - outs[1]).abs().max() < 1e-3
+        got_all = outs[0].cpu().numpy()
+        for b, h in pairs:
+            T = lens[b]
+            hk = hist_k[b, h, :T].cpu().numpy()
+            hv = hist_v[b, h, :T].cpu().numpy()
+            pl = plans_np[h:h + 1]
+            mid = slice(ns, T - win)
+            codes, raw, _ = oracle_lib.encode_k(pl, hk[mid])
+            kd = oracle_lib.dequant_k(pl, codes, oracle_lib.f2h(raw[:, :max(int(pl['n_seg'][0]), 1)]))
+            vc, vn = oracle_lib.encode_v(pl, hv[mid])
+            vd = oracle_lib.dequant_v(pl, vc, vn).astype(np.float64) @ pl['v_rot'][0].reshape(128, 128).astype(np.float64)
+            fp = np.r_[0:ns, T - win:T]
+            qh = q[b, h * gqa:(h + 1) * gqa, 0].cpu().numpy()
+            q_rot = oracle_lib.rotate_q(pl, qh).astype(np.float64)
+            logits = np.concatenate([q_rot @ kd.astype(np.float64).T,
+                                     qh.astype(np.float64) @ hk[fp].astype(np.float64).T], 1) / np.sqrt(128)
+            p = np.exp(logits - logits.max(1, keepdims=True))
+            p /= p.sum(1, keepdims=True)
+            ref = p @ np.concatenate([vd, hv[fp].astype(np.float64)], 0)
+            got = got_all[b, h * gqa:(h + 1) * gqa]
+            assert np.abs(got - ref).max() < TOL, (step, b, h, np.abs(got - ref).max())
 
 
 @pytest.mark.parametrize("k_layout,v_layout,vb", [(0, 0, 3), (1, 1, 3), (1, 0, 4), (0, 1, 2), (1, 1, 4)])

@@ -492,3 +492,29 @@ def test_baked_q_proj_equals_rotation_of_the_projection(oracle_lib, seed, with_b
             y16 = y[:, lo:lo + 128].half().numpy()
             ref = oracle_lib.rotate_q(q.plan(), y16).astype(np.float64)
             assert np.abs(got - ref).max() < 2e-2 * max(1.0, np.abs(want).max())     # fp16 in and out
+
+
+def test_bench_allocations_follow_calibration_on_drawn_tensors():
+    """The headline workload takes its per-head bit allocations from the closed-form block
+    energies of the synthetic distribution.  Calibrating on 2048 drawn tokens of that
+    distribution (queries and keys share the per-block scaling; every query head of the group
+    is a sample) through ``BlockGTQQuantizer.calibrate`` reproduces them up to the sampling
+    noise of the block energies: the same bit budget, most heads identical, and where a head
+    differs it is one bit moved between two blocks whose scores are nearly tied."""
+    from blockgtq_amd import synthetic as syn, workloads as wl
+    w = wl.WORKLOADS["qwen3b_b8_32k_k3v3"]
+    gqa = w.n_q // w.n_kv
+    identical = total = 0
+    for layer in (0, 1, 9, 18, 27, 35):
+        qs, energies = wl.calibrate_layer(w, layer, 'cpu')
+        for h in range(w.n_kv):
+            gen = torch.Generator().manual_seed(w.seed * 31 + layer * 7 + h)
+            k = syn.make_keys(1, 2048, 128, energies[h:h + 1], w.rope_theta, gen)[0]
+            q = syn.make_keys(1, 2048 * gqa, 128, energies[h:h + 1], w.rope_theta, gen)[0]
+            drawn = BlockGTQQuantizer(128, avg_bits=w.k_bits, min_bits=w.min_bits, max_bits=w.max_bits, device='cpu')
+            drawn.calibrate(q, k)
+            diff = drawn.bit_allocation - qs[h].bit_allocation
+            assert int(diff.sum()) == 0 and int(diff.abs().max()) <= 1 and int((diff != 0).sum()) <= 4, (layer, h, diff)
+            identical += int((diff == 0).all())
+            total += 1
+    assert identical >= total * 2 // 3, (identical, total)

@@ -59,15 +59,26 @@ def test_k_bit_packed_record_is_a_per_segment_bit_stream(head):
     assert np.array_equal(orc.unpack_k(plan, rec, 0), codes)
 
 
-def test_k_mixed_record_layout(head):
+@pytest.mark.parametrize("with_zero_bit_blocks", [False, True])
+def test_k_mixed_record_layout(head, with_zero_bit_blocks):
+    """Nibbles of the <= 4-bit dims (two per byte, low nibble first), then one byte per wider code;
+    dims of 0-bit blocks come first in packed order and take no room in the record."""
     orc, q, plan, k, v, qq = head
+    if with_zero_bit_blocks:
+        q, en = make_quantizer(seed=1, min_bits=0, max_bits=8, budget=160)
+        plan = q.plan()
+        k, _, _ = make_kv(en, 200)
     codes, _, _ = orc.encode_k(plan, k)
     rec = orc.pack_k(plan, codes, 1)
+    z = int(plan[0]['n_zero_dims'])
     ns, nl = int(plan[0]['nopack_start']), int(plan[0]['nopack_len'])
-    assert rec.shape[1] == ns // 2 + nl
-    assert np.array_equal(rec[:, :ns // 2], (codes[:, 0:ns:2] & 15) | ((codes[:, 1:ns:2] & 15) << 4))
-    assert np.array_equal(rec[:, ns // 2:], codes[:, ns:ns + nl])
-    assert np.array_equal(orc.unpack_k(plan, rec, 1), codes)
+    assert (z > 0) == with_zero_bit_blocks and z % 2 == 0 and nl > 0
+    nib = (ns - z) // 2
+    assert rec.shape[1] == nib + nl == int(plan[0]['k_mixed_bytes'])
+    assert np.array_equal(rec[:, :nib], (codes[:, z:ns:2] & 15) | ((codes[:, z + 1:ns:2] & 15) << 4))
+    assert np.array_equal(rec[:, nib:], codes[:, ns:ns + nl])
+    back = orc.unpack_k(plan, rec, 1)
+    assert np.array_equal(back[:, z:], codes[:, z:]) and not back[:, :z].any()
 
 
 @pytest.mark.parametrize("bits,nibble", [(1, False), (2, False), (3, False), (4, False), (2, True), (3, True)])
