@@ -72,6 +72,15 @@ _SIGNATURES = {
                               c_i, c_i, c_i, c_i, c_i,
                               c_p, c_i64, c_i64, c_i64,
                               c_p, c_i64, c_i64, c_i64, c_p]),
+    "bgtq_prefill_attn": (c_i, [c_p,
+                                c_p, c_i64, c_i64, c_i64,
+                                c_p, c_i64, c_i64, c_i64, c_i,
+                                c_p, c_i64, c_i64, c_i64,
+                                c_p, c_i64, c_i64, c_i64, c_i,
+                                c_p, c_i64, c_i64, c_i64,
+                                c_i, c_i, c_i, c_i, c_i, c_i, c_i,
+                                c_i, c_i, ctypes.c_float, c_i,
+                                c_p, c_i64, c_i64, c_i64, c_p]),
     "bgtq_lse_reduce": (c_i, [c_p, c_p, c_p, c_i, c_p, c_p, c_i,
                               c_i, c_i, c_i, c_i, c_p, c_i64, c_i64, c_p, c_p]),
 }

@@ -25,6 +25,7 @@ SOURCES = {
     # LDS tiles are written as 128-bit / 16-bit words and read back as 32-bit words
     "bgtq_decode_mfma.hip": ["-fno-strict-aliasing"],
     "bgtq_dequant.hip": [],
+    "bgtq_prefill.hip": ["-fno-strict-aliasing"],
 }
 
 

@@ -1,0 +1,438 @@
+// Prompt-phase (many query tokens) attention over packed K and V records (gfx950).
+//
+// One work-group of 4 waves owns 128 query rows of one (batch row, KV head): BQ = 128 / gqa
+// consecutive query tokens of every query head of the group, 32 rows per wave.  It walks the
+// 64-token tiles its rows can see.  Per tile the raw records come from HBM straight into LDS
+// (global_load_lds_dwordx4), all four waves dequantise them once through the plan's pair tables
+// into an fp16 K tile [token][dim] (packed-dim order, fp16(centroid * group norm): what
+// bgtq_dequant_kv writes) and a transposed fp16 V tile [dim][token], and then every wave runs
+// both products on v_mfma_f32_32x32x16_f16 for its own rows:
+//
+//   S^T = K Q^T   A = K tile rows (tokens), B = the wave's rotated queries (kept in registers).
+//                 In the result a lane holds one query (column) and 16 tokens of each 32-token
+//                 block, so the softmax statistics of a query are in-lane up to one exchange
+//                 between the two halves of the wave.
+//   O^T = V^T P^T A = transposed V tile rows (dims), B = P straight from the score registers:
+//                 the token order of a lane's score registers is a fixed permutation of the
+//                 contraction index, and the V reads follow the same permutation.
+//
+// The exponentials are taken relative to a per-query reference that is only moved when a score
+// exceeds it (to the maximum + 4 in log2 units), so the accumulators are rescaled rarely.  At the
+// end O is normalised, un-rotated on v_mfma_f32_32x32x2_f32 against the plan's fp32 V rotation
+// (operands again taken from the accumulator registers under a permutation of the contraction
+// index) and stored as fp16.  No fp16 K/V tensor of the layer is written.
+//
+// Reference behaviour: blockgtq/kernels/fused_packed_attention.py:1876-2594 (prefill kernel),
+// driver blockgtq/prefill.py:66-101.
+#include <atomic>
+
+#include "bgtq_lds.h"
+
+namespace {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int D = BGTQ_D;
+constexpr int MT = 64;                       // tokens per tile
+constexpr int ROWS = 128;                    // query rows per work-group (4 waves x 32)
+constexpr int NTHR = 256;
+constexpr int MAX_UNITS = BGTQ_MAX_UNITS;
+constexpr int MAX_KN = 8;
+constexpr float REFRESH = 4.0f;
+constexpr int KROW = D * 2 + 16;             // bytes of a K tile row: rows 4 banks apart
+constexpr int VTROW = MT * 2 + 16;           // bytes of a transposed V tile row (one dim, 64 tokens)
+
+// LDS layout (bytes): [V table | K tables | unit programs | unit dims | raw K | K norms | V norms | raw V | K tile | V^T tile]
+constexpr int VTAB_OFF = 0;
+constexpr int KTAB_OFF = BGTQ_VLUT_BYTES;
+constexpr int PROG_OFF = KTAB_OFF + BGTQ_LUT_IMAGE_BYTES;            // [MAX_UNITS][8] dwords
+constexpr int UNIT_OFF = PROG_OFF + MAX_UNITS * 32;                  // [MAX_UNITS] dwords
+constexpr int RAW_OFF = UNIT_OFF + MAX_UNITS * 4;
+
+struct PrefillArgs {
+    const bgtq_head_plan* plans;
+    const uint16_t* q;  int64_t q_sb, q_sh, q_ss;
+    const uint8_t* kp;  int64_t kp_sb, kp_sh, kp_st;
+    const uint16_t* kn; int64_t kn_sb, kn_sh, kn_st;
+    const uint8_t* vp;  int64_t vp_sb, vp_sh, vp_st;
+    const uint16_t* vn; int64_t vn_sb, vn_sh;
+    int B, n_kv, gqa, S, T, q_pos_offset, causal;
+    int k_layout, v_layout;
+    float scale;
+    int unrotate;
+    uint16_t* out; int64_t o_sb, o_sh, o_ss;
+    int k_row_width, v_row_width, v_stride;
+    int kt, knr, vnr, vt;      // raw tile areas
+};
+
+__host__ __device__ inline int raw_bytes(int krow, int vstride, int kn_st, int& kt, int& knr, int& vnr, int& vt) {
+    kt = (MT * krow + 32 + 15) & ~15;
+    knr = (MT * kn_st * 2 + 16 + 15) & ~15;
+    vnr = MT * 2 + 16;
+    vt = (MT * vstride + 32 + 15) & ~15;
+    return kt + knr + vnr + vt;
+}
+
+__device__ __forceinline__ uint32_t pk_mul_f16(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("v_pk_mul_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ uint32_t cvt_pk_f16(float lo, float hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 r = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+__global__ __launch_bounds__(NTHR, 2) void prefill_mfma_kernel(PrefillArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = blockIdx.y, b = blockIdx.z;
+    const bgtq_head_plan& P = a.plans[h];
+    const int gqa = a.gqa, kl = a.k_layout;
+    const bool vnib = a.v_layout == BGTQ_V_NIBBLE;
+    const int BQ = ROWS / gqa;                                   // query tokens per work-group
+    const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;         // the blocks that see most tokens start first
+    const int s0 = qb * BQ;
+    const int krow = a.k_row_width, vrow = a.v_stride, kn_st = (int)a.kn_st;
+    const int vbw = vnib ? 4 : (int)P.v_bits;                    // bits of a V code as stored
+    const bool vrep = !vnib && vbw <= 3;                         // V pair table replicated over the banks
+
+    // ---- the tiles this work-group walks
+    const int s_last = min(s0 + BQ, a.S) - 1;
+    const int t_end = a.causal ? min(a.T, a.q_pos_offset + s_last + 1) : a.T;
+    const int n_tiles = (t_end + MT - 1) / MT;
+
+    // ---- this lane's query row: row r = wave * 32 + (lane & 31); head r / BQ, token s0 + r % BQ
+    const int li = lane & 31, lg = lane >> 5;
+    const int row = wave * 32 + li;
+    const int hq = row / BQ, sq = s0 + row - hq * BQ;
+    const bool row_ok = hq < gqa && sq < a.S;
+    // tokens t < lim are visible to this row
+    const int lim = !row_ok ? 0 : a.causal ? min(a.T, a.q_pos_offset + sq + 1) : a.T;
+
+    // ---- LDS areas
+    const uint32_t kraw = RAW_OFF, knraw = kraw + a.kt, vnraw = knraw + a.knr, vraw = vnraw + a.vnr;
+    const uint32_t ktile = vraw + a.vt, vtile = ktile + MT * KROW;
+
+    // ---- tables, unit programs and unit dims into LDS
+    const uint32_t voff = (uint32_t)lane * 16;
+    {
+        const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
+        const uint8_t* kimg = (const uint8_t*)P.lut_image[kl];
+        const int vbytes = (vnib || vbw == 4) ? 1024 : (1 << (2 * vbw)) * 128;
+        const int kbytes = kl == BGTQ_K_MIXED ? BGTQ_LUTM_KEND : BGTQ_LUT_KEND;
+        const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
+        for (int cc = wave; cc < vch + kch; cc += NTHR / 64) {
+            const uint8_t* src;
+            uint32_t dst;
+            int left;
+            if (cc < vch) { src = vimg + cc * 1024; dst = VTAB_OFF + cc * 1024; left = vbytes - cc * 1024; }
+            else { src = kimg + (cc - vch) * 1024; dst = KTAB_OFF + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
+            dma16(voff, src, __builtin_amdgcn_readfirstlane(dst), __builtin_amdgcn_ballot_w64((int)voff < left));
+        }
+        if (tid < MAX_UNITS * 8) lds_put<uint32_t>(PROG_OFF + tid * 4, P.kprog[kl][tid >> 3][tid & 7]);
+        if (tid < MAX_UNITS) lds_put<uint32_t>(UNIT_OFF + tid * 4, P.kunit[kl][tid]);
+    }
+    const int n_units = min(P.n_units[kl], MAX_UNITS), n_pair = min(P.n_pair_units[kl], n_units);
+    const uint32_t kend = P.kend[kl], kfirst0 = P.kfirst[kl][0], kfirst1 = P.kfirst[kl][1];
+    const int n_zero = min(max(P.n_zero_dims, 0), D);
+
+    // ---- the wave's queries as B operands: lane (query li, half lg) holds dims 16 kk + 8 lg .. + 7 of step kk
+    half8 Qb[8];
+    {
+        const uint16_t* qrow = a.q + b * a.q_sb + ((int64_t)h * gqa + (row_ok ? hq : 0)) * a.q_sh + (int64_t)(row_ok ? sq : 0) * a.q_ss;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+            uint4v w = {0, 0, 0, 0};
+            if (row_ok) w = *(const uint4v*)(qrow + 16 * kk + 8 * lg);
+            Qb[kk] = __builtin_bit_cast(half8, w);
+        }
+    }
+
+    // ---- streaming sources
+    const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
+    const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
+    const uint8_t* kn_base = (const uint8_t*)(a.kn + b * a.kn_sb + h * a.kn_sh);
+    const uint8_t* vn_base = (const uint8_t*)(a.vn + b * a.vn_sb + h * a.vn_sh);
+    const uint32_t kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
+    const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
+    // wave 0 fetches the K records, wave 1 the V records, wave 2 both norm arrays
+    auto issue_tile = [&](int tile) {
+        const int t = tile * MT, nt = min(MT, t_end - t);
+        if (wave == 0) {
+            dma_region<9>(kp_base - kph + (int64_t)t * krow, kraw, dma_shape((int)kph + nt * krow, voff), voff);
+        } else if (wave == 1) {
+            dma_region<9>(vp_base - vph + (int64_t)t * vrow, vraw, dma_shape((int)vph + nt * vrow, voff), voff);
+        } else if (wave == 2) {
+            dma_region<2>(kn_base - knph + (int64_t)t * kn_st * 2, knraw, dma_shape((int)knph + nt * kn_st * 2, voff), voff);
+            dma_region<1>(vn_base - vnph + (int64_t)t * 2, vnraw, dma_shape((int)vnph + nt * 2, voff), voff);
+        }
+    };
+    if (n_tiles > 0) issue_tile(0);
+
+    // the K tile's columns of 0-bit dims are never written: zero them once
+    for (int i = tid; i < MT * (n_zero / 2); i += NTHR) {
+        const int t = i / (n_zero / 2), c = i - t * (n_zero / 2);
+        lds_put<uint32_t>(ktile + t * KROW + c * 4, 0u);
+    }
+
+    const float c2 = a.scale * 1.44269504088896340736f;        // scores in log2 units
+    const uint32_t rep = ((uint32_t)lane & 31u) * 4u;
+    float16v O[4];                                              // O^T: block db = dims 32 db .., reg r -> dim 32 db + 8 (r / 4) + 4 lg + r % 4
+#pragma unroll
+    for (int db = 0; db < 4; db++) O[db] = (float16v){0};
+    float m_ref = -INFINITY, l_part = 0.f;                       // per query (this half's share of the denominator)
+
+    // K dequantisation: lane = token, wave w takes units w, w + 4, ...
+    const uint32_t krow_l = kraw + kph + (uint32_t)lane * krow;
+    const uint32_t knrow_l = knraw + knph + (uint32_t)lane * kn_st * 2;
+    // V dequantisation: thread (token pair tp, unit pair up); code pair e of a unit's raw word is brought to
+    // the table-index position by a rotation (the V table sits at LDS address 0)
+    const int tp = tid & 31, up = tid >> 5;
+    const int vtsh = vrep ? 7 : 2;
+    uint32_t vrot[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) vrot[e] = (uint32_t)(2 * vbw * e - vtsh) & 31u;
+    const uint32_t vfmask = ((1u << (2 * vbw)) - 1u) << vtsh, vbase = vrep ? rep : 0u;
+
+    for (int tile = 0; tile < n_tiles; tile++) {
+        const int t0 = tile * MT;
+        const int nt = min(MT, t_end - t0);                      // records of this tile; the rows behind them hold stale bytes
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wave's share of the raw tile (and, first time, of the tables)
+        __syncthreads();                                         // raw tile complete; the previous tile's products are done
+
+        // ---- K tile: fp16(centroid * norm), packed-dim order
+        for (int u = wave; u < n_units; u += NTHR / 64) {
+            const uint4v pa = lds_at<uint4v>(PROG_OFF + u * 32), pb = lds_at<uint4v>(PROG_OFF + u * 32 + 16);
+            const uint32_t dsc = lds_at<uint32_t>(UNIT_OFF + u * 4);
+            const int d0 = (int)(dsc & 0xFF), len = (int)(dsc >> 8) & 0xFF;
+            if (len == 0) continue;                              // (wave-uniform) the empty unit that evens out the pair units
+            const uint32_t off = u == 0 ? kfirst0 : u == 1 ? kfirst1 : lds_at<uint32_t>(PROG_OFF + (u - 2) * 32 + 28);
+            const int seg = __builtin_popcount(kend & ((1u << u) - 1u));
+            // rows past the tile's last record get norm 0: their products must stay finite (P is 0 there)
+            const uint32_t n16 = lane < nt ? (uint32_t)lds_at<uint16_t>(knrow_l + seg * 2) : 0u;
+            const uint32_t nn = n16 | (n16 << 16);
+            uint32_t w[4];
+            if (u < n_pair) {
+                const uint32_t r = lds_codes4(krow_l + off);
+                const uint32_t base = and_or_v(rep, pb.z, pb.y);
+                w[0] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.x), pb.x, base));
+                w[1] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.y), pb.x, base));
+                w[2] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.z), pb.x, base));
+                w[3] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.w), pb.x, base));
+            } else {
+                const uint2v r = lds_codes8(krow_l + off);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t x = e < 2 ? r.x : r.y;
+                    const uint32_t c0 = pb.y + ((x >> ((e & 1) * 16)) & 0xFF) * 2;
+                    const uint32_t c1 = pb.y + ((x >> ((e & 1) * 16 + 8)) & 0xFF) * 2;
+                    w[e] = (uint32_t)lds_at<uint16_t>(c0) | ((uint32_t)lds_at<uint16_t>(c1) << 16);
+                }
+            }
+            const uint32_t dst = ktile + (uint32_t)lane * KROW + (uint32_t)d0 * 2;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (2 * e < len) lds_put<uint32_t>(dst + e * 4, pk_mul_f16(w[e], nn));
+        }
+
+        // ---- V^T tile: fp16(centroid * norm), [dim][token]; thread = tokens 2 tp, 2 tp + 1, units 2 up, 2 up + 1
+        {
+            uint32_t nrm[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const uint32_t n16 = 2 * tp + j < nt ? (uint32_t)lds_at<uint16_t>(vnraw + vnph + (uint32_t)(2 * tp + j) * 2) : 0u;
+                nrm[j] = n16 | (n16 << 16);
+            }
+#pragma unroll
+            for (int uu = 0; uu < 2; uu++) {
+                const int u = 2 * up + uu;
+                uint32_t w[2][4];
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const uint32_t r = lds_codes4(vraw + vph + (uint32_t)(2 * tp + j) * vrow + (uint32_t)(u * vbw));
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        w[j][e] = pk_mul_f16(lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, vrot[e]), vfmask, vbase)), nrm[j]);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    // (dim 8u + 2e of both tokens), (dim 8u + 2e + 1 of both tokens)
+                    const uint32_t lo = __builtin_amdgcn_perm(w[1][e], w[0][e], 0x05040100u);
+                    const uint32_t hi = __builtin_amdgcn_perm(w[1][e], w[0][e], 0x07060302u);
+                    lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e) * VTROW + (uint32_t)tp * 4, lo);
+                    lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e + 1) * VTROW + (uint32_t)tp * 4, hi);
+                }
+            }
+        }
+        __syncthreads();                                         // tiles complete; the raw buffers are free
+        if (tile + 1 < n_tiles) issue_tile(tile + 1);
+
+        // ---- S^T = K Q^T for the wave's 32 queries: 2 token blocks x 8 steps of 16 dims
+        float16v Sc[2];
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++) {
+            Sc[tb] = (float16v){0};
+            const uint32_t arow = ktile + (uint32_t)(32 * tb + li) * KROW + (uint32_t)lg * 16;
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) {
+                const half8 A = lds_at<half8>(arow + kk * 32);
+                Sc[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A, Qb[kk], Sc[tb], 0, 0, 0);
+            }
+        }
+        // ---- softmax, lane = query; reg r of block tb is token t0 + 32 tb + 8 (r / 4) + 4 lg + r % 4
+        float mx = -INFINITY;
+        if (__builtin_amdgcn_ballot_w64(t0 + MT > lim)) {        // (wave-uniform) some row of the wave has masked tokens in this tile
+#pragma unroll
+            for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float s = Sc[tb][r] * c2;
+                    if (t0 + 32 * tb + 8 * (r >> 2) + 4 * lg + (r & 3) >= lim) s = -INFINITY;
+                    Sc[tb][r] = s;
+                    mx = fmaxf(mx, s);
+                }
+        } else {
+#pragma unroll
+            for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    Sc[tb][r] *= c2;
+                    mx = fmaxf(mx, Sc[tb][r]);
+                }
+        }
+        if (__builtin_amdgcn_ballot_w64(mx > m_ref)) {           // wave-uniform, rare after the first tiles
+            const float other = __shfl_xor(mx, 32, 64);
+            const float top = fmaxf(mx, other);
+            const float m_new = top > m_ref ? top + REFRESH : m_ref;
+            const float alpha = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+            l_part *= alpha;
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) O[db][r] *= alpha;
+            m_ref = m_new;
+        }
+        uint32_t Pw[2][8];                                        // fp16 pairs: Pw[tb][j] = regs 2j, 2j + 1
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float p0 = __builtin_amdgcn_exp2f(Sc[tb][2 * j] - m_ref);
+                const float p1 = __builtin_amdgcn_exp2f(Sc[tb][2 * j + 1] - m_ref);
+                l_part += p0 + p1;
+                Pw[tb][j] = cvt_pk_f16(p0, p1);
+            }
+        // ---- O^T += V^T P^T: step (tb, hf) contracts the 16 tokens 32 tb + 16 hf + {4 lg + i, 8 + 4 lg + i}
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                const uint4v pw = {Pw[tb][4 * hf], Pw[tb][4 * hf + 1], Pw[tb][4 * hf + 2], Pw[tb][4 * hf + 3]};
+                const half8 Bp = __builtin_bit_cast(half8, pw);
+                const uint32_t col = (uint32_t)(32 * tb + 16 * hf + 4 * lg) * 2;
+#pragma unroll
+                for (int db = 0; db < 4; db++) {
+                    const uint32_t vr = vtile + (uint32_t)(32 * db + li) * VTROW + col;
+                    const uint2v x0 = lds_at<uint2v>(vr), x1 = lds_at<uint2v>(vr + 16);
+                    const uint4v av = {x0.x, x0.y, x1.x, x1.y};
+                    O[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, av), Bp, O[db], 0, 0, 0);
+                }
+            }
+    }
+
+    // ---- normalise; un-rotate: out^T = R^T O^T, contraction slot g of step (db, r) is dim 32 db + 8 (r / 4) + 4 g + r % 4
+    const float l_tot = l_part + __shfl_xor(l_part, 32, 64);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) O[db][r] *= inv;
+    float16v R[4];
+    if (a.unrotate) {
+        const float* rot = P.v_rot;
+#pragma unroll
+        for (int ob = 0; ob < 4; ob++) R[ob] = (float16v){0};
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int d = 32 * db + 8 * (r >> 2) + 4 * lg + (r & 3);
+#pragma unroll
+                for (int ob = 0; ob < 4; ob++)
+                    R[ob] = __builtin_amdgcn_mfma_f32_32x32x2f32(rot[d * D + 32 * ob + li], O[db][r], R[ob], 0, 0, 0);
+            }
+    } else {
+#pragma unroll
+        for (int ob = 0; ob < 4; ob++) R[ob] = O[ob];
+    }
+    if (row_ok) {
+        uint16_t* orow = a.out + b * a.o_sb + ((int64_t)h * gqa + hq) * a.o_sh + (int64_t)sq * a.o_ss;
+#pragma unroll
+        for (int ob = 0; ob < 4; ob++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                uint2v w = {cvt_pk_f16(R[ob][4 * j], R[ob][4 * j + 1]), cvt_pk_f16(R[ob][4 * j + 2], R[ob][4 * j + 3])};
+                *(uint2v*)(orow + 32 * ob + 8 * j + 4 * lg) = w;
+            }
+    }
+}
+
+}  // namespace
+
+extern "C" int bgtq_prefill_attn(const bgtq_head_plan* plans,
+                                 const void* q_rot, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                 const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                                 const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                                 const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                                 const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                                 int B, int n_kv, int gqa, int S, int T, int q_pos_offset, int is_causal,
+                                 int k_layout, int v_layout, float scale, int unrotate,
+                                 void* out, int64_t o_sb, int64_t o_sh, int64_t o_ss, void* stream) {
+    BGTQ_CHECK_ARG(plans && q_rot && k_packed && k_norms && v_packed && v_norms && out);
+    BGTQ_CHECK_ARG(B > 0 && n_kv > 0 && gqa > 0 && S > 0 && T >= 0 && q_pos_offset >= 0);
+    BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
+    BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
+    // layout requirements of this kernel; callers fall back to bgtq_dequant_kv + their own attention
+    if (gqa > ROWS || !(scale > 0.f)) return BGTQ_EUNSUPPORTED;
+    if ((kp_st & 3) || (kp_sb & 3) || (kp_sh & 3) || ((uintptr_t)k_packed & 3)) return BGTQ_EUNSUPPORTED;
+    if ((vp_st & 3) || (vp_sb & 3) || (vp_sh & 3) || ((uintptr_t)v_packed & 3)) return BGTQ_EUNSUPPORTED;
+    if (kp_st != k_row_width || k_row_width < 4 || k_row_width > 128) return BGTQ_EUNSUPPORTED;
+    if (vn_st != 1 || kn_st < 1 || kn_st > MAX_KN) return BGTQ_EUNSUPPORTED;
+    if (v_row_width != 16 && v_row_width != 32 && v_row_width != 48 && v_row_width != 64) return BGTQ_EUNSUPPORTED;
+    if (vp_st < v_row_width || vp_st > v_row_width + 4) return BGTQ_EUNSUPPORTED;
+    if (v_layout == BGTQ_V_NIBBLE && v_row_width != 64) return BGTQ_EUNSUPPORTED;
+    if ((q_ss & 7) || (q_sh & 7) || (q_sb & 7) || ((uintptr_t)q_rot & 15)) return BGTQ_EUNSUPPORTED;   // 16-byte query loads
+    if ((o_ss & 3) || (o_sh & 3) || (o_sb & 3) || ((uintptr_t)out & 7)) return BGTQ_EUNSUPPORTED;      // 8-byte output stores
+    if (T == 0) return BGTQ_EUNSUPPORTED;
+    PrefillArgs a;
+    a.plans = plans;
+    a.q = (const uint16_t*)q_rot; a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss;
+    a.kp = (const uint8_t*)k_packed; a.kp_sb = kp_sb; a.kp_sh = kp_sh; a.kp_st = kp_st;
+    a.kn = (const uint16_t*)k_norms; a.kn_sb = kn_sb; a.kn_sh = kn_sh; a.kn_st = kn_st;
+    a.vp = (const uint8_t*)v_packed; a.vp_sb = vp_sb; a.vp_sh = vp_sh; a.vp_st = vp_st;
+    a.vn = (const uint16_t*)v_norms; a.vn_sb = vn_sb; a.vn_sh = vn_sh;
+    a.B = B; a.n_kv = n_kv; a.gqa = gqa; a.S = S; a.T = T; a.q_pos_offset = q_pos_offset; a.causal = is_causal != 0;
+    a.k_layout = k_layout; a.v_layout = v_layout; a.scale = scale; a.unrotate = unrotate != 0;
+    a.out = (uint16_t*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
+    a.k_row_width = k_row_width; a.v_row_width = v_row_width; a.v_stride = (int)vp_st;
+    const int raw = raw_bytes(k_row_width, (int)vp_st, (int)kn_st, a.kt, a.knr, a.vnr, a.vt);
+    const size_t smem = (size_t)RAW_OFF + raw + (size_t)MT * KROW + (size_t)D * VTROW;
+    static std::atomic<int> ready{0};
+    if (ready.load(std::memory_order_acquire) == 0) {
+        // offsets into the dynamic LDS block are used as LDS addresses: holds only without static LDS
+        hipFuncAttributes fa;
+        hipError_t e = hipFuncGetAttributes(&fa, (const void*)prefill_mfma_kernel);
+        if (e != hipSuccess) return (int)e;
+        e = hipFuncSetAttribute((const void*)prefill_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return (int)e;
+        ready.store(fa.sharedSizeBytes == 0 ? 1 : -1, std::memory_order_release);
+    }
+    if (ready.load(std::memory_order_acquire) < 0 || smem > 160 * 1024) return BGTQ_EUNSUPPORTED;
+    const int BQ = ROWS / gqa;
+    dim3 grid((unsigned)((S + BQ - 1) / BQ), (unsigned)n_kv, (unsigned)B);
+    hipLaunchKernelGGL(prefill_mfma_kernel, grid, dim3(NTHR), smem, (hipStream_t)stream, a);
+    return bgtq_launch_status();
+}

@@ -244,6 +244,49 @@ def dequant_kv(plans: torch.Tensor, k_packed: torch.Tensor, k_norms: torch.Tenso
     return ko, vo
 
 
+UNSUPPORTED = -2          # BGTQ_EUNSUPPORTED: the fast kernel does not take this argument set
+
+
+@torch.no_grad()
+def prefill_attention_packed(plans: torch.Tensor, q_rot: torch.Tensor, k_packed: torch.Tensor,
+                             k_norms: torch.Tensor, v_packed: torch.Tensor, v_norms: torch.Tensor,
+                             T: int, *, k_layout: int = _plan.K_BITPACKED, v_layout: int = _plan.V_BITPACKED,
+                             scale: Optional[float] = None, is_causal: bool = True, q_pos_offset: int = 0,
+                             unrotate: bool = True, k_row_width: Optional[int] = None,
+                             v_row_width: Optional[int] = None) -> Optional[torch.Tensor]:
+    """Attention of many query tokens straight over the packed cache (``bgtq_prefill_attn``).
+
+    q_rot (B, n_q, S, D) fp16 rotated queries; cache tensors as for ``decode_attention``.
+    Query token s sees records ``t <= q_pos_offset + s`` when ``is_causal``.  Returns
+    (B, n_q, S, D) fp16, or ``None`` when the kernel does not take this argument set
+    (the caller then dequantises with ``dequant_kv`` and uses ``prefill_attention``)."""
+    _capi.require_cuda(k_packed, "k_packed")
+    assert q_rot.dtype == torch.float16 and q_rot.dim() == 4 and q_rot.stride(-1) == 1
+    assert k_packed.dtype == torch.uint8 and k_packed.stride(-1) == 1
+    assert v_packed.dtype == torch.uint8 and v_packed.stride(-1) == 1
+    assert k_norms.dtype == torch.float16 and v_norms.dtype == torch.float16
+    B, n_q, S, D = q_rot.shape
+    n_kv = k_packed.shape[1]
+    assert D == _plan.HEAD_DIM and n_q % n_kv == 0 and k_packed.shape[2] >= T
+    k_row_width = k_packed.shape[-1] if k_row_width is None else k_row_width
+    v_row_width = v_packed.shape[-1] if v_row_width is None else v_row_width
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    out = torch.empty((B, n_q, S, D), dtype=torch.float16, device=q_rot.device)
+    code = _capi.lib().bgtq_prefill_attn(
+        _capi.ptr(plans), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1), q_rot.stride(2),
+        _capi.ptr(k_packed), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2), k_row_width,
+        _capi.ptr(k_norms), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2),
+        _capi.ptr(v_packed), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2), v_row_width,
+        _capi.ptr(v_norms), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
+        B, n_kv, n_q // n_kv, S, T, int(q_pos_offset), int(bool(is_causal)),
+        k_layout, v_layout, scale, int(bool(unrotate)),
+        _capi.ptr(out), out.stride(0), out.stride(1), out.stride(2), _capi.stream_ptr(q_rot.device))
+    if code == UNSUPPORTED:
+        return None
+    _capi.check(code, "bgtq_prefill_attn")
+    return out
+
+
 @torch.no_grad()
 def prefill_attention(q_rot: torch.Tensor, k_hat: torch.Tensor, v_hat: torch.Tensor,
                       v_rot: Optional[torch.Tensor] = None, scale: Optional[float] = None,

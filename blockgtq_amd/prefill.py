@@ -7,10 +7,11 @@ ever materialised.  Reference behaviour: blockgtq/prefill.py:24-111.
 
 As in the reference, attention inside the prompt sees the *quantised* keys and
 values (what later decode steps will see), not the layer's fp16 K/V: the
-records of the layer are dequantised in one pass for all KV heads
-(``bgtq_dequant_kv``), the queries are permuted + rotated into each head's
-packed space with one batched GEMM, and the score/value GEMMs run in the
-library's fused causal attention.
+queries are permuted + rotated into each head's packed space with one batched
+GEMM and ``bgtq_prefill_attn`` attends straight over the records (tiles are
+dequantised inside the kernel; no fp16 K/V of the layer is written).  Argument
+sets that kernel does not take go through one dequantisation pass
+(``bgtq_dequant_kv``) and the library's fused causal attention.
 """
 import torch
 
@@ -44,9 +45,16 @@ def packed_prefill_attention(cache, li, q, T, q_pos_offset=0):
     else:
         qg = q.reshape(B, cache.nkv, cache.gqa * S, D).float()
         q_rot = (qg @ q_mat.unsqueeze(0)).to(torch.float16).reshape(B, n_q, S, D)
+    plans = cache.batched_args[li]['plans']
+    out = ops.prefill_attention_packed(
+        plans, q_rot.contiguous(), cache.k_packed[li], cache.k_norms[li], cache.v_packed[li], cache.v_norms[li], T,
+        k_layout=cache._k_layout, v_layout=cache._v_layout, scale=cache.scale, is_causal=True,
+        q_pos_offset=q_pos_offset, k_row_width=cache.k_bytes_per_tok, v_row_width=cache.vpb)
+    if out is not None:
+        return out
+    # argument sets the fused kernel does not take: one dequantisation pass + the library's attention
     k_hat, v_hat = ops.dequant_kv(
-        cache.batched_args[li]['plans'], cache.k_packed[li], cache.k_norms[li],
-        cache.v_packed[li], cache.v_norms[li], T,
+        plans, cache.k_packed[li], cache.k_norms[li], cache.v_packed[li], cache.v_norms[li], T,
         k_layout=cache._k_layout, v_layout=cache._v_layout,
         k_row_width=cache.k_bytes_per_tok, v_row_width=cache.vpb)
     return ops.prefill_attention(q_rot, k_hat, v_hat, v_rot, cache.scale, True, q_pos_offset)

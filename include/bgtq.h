@@ -423,6 +423,34 @@ int bgtq_dequant_kv(const bgtq_head_plan* plans,
                     void* v_out, int64_t vo_sb, int64_t vo_sh, int64_t vo_st,
                     void* stream);
 
+/*
+ * Prompt-phase attention straight over the packed cache: S query tokens per
+ * sequence attend to records [0, T), query token s seeing t <= q_pos_offset + s
+ * when is_causal.  Every 64-token tile of records is dequantised once per block of
+ * 128 query rows inside the kernel (same values as bgtq_dequant_kv writes), both
+ * products run on matrix cores, the V un-rotation (when unrotate != 0) is applied
+ * before the fp16 store; no fp16 K/V tensor of the layer exists.  Replaces
+ * _packed_prefill_kernel as driven by fused_blockgtq_prefill_attention
+ * (blockgtq/kernels/fused_packed_attention.py:1876-2594, :2597-2760), for all KV
+ * heads of a layer in one launch.
+ *   q_rot      fp16 [B][n_kv*gqa][S][128], already permuted + rotated
+ *              (bgtq_rotate_q semantics), strides q_sb/q_sh/q_ss in halves, rows 16-byte aligned
+ *   cache      as for bgtq_decode_attn (same strides, layouts and row widths)
+ *   out        fp16 [B][n_kv*gqa][S][128], strides o_sb/o_sh/o_ss in halves
+ * Returns BGTQ_EUNSUPPORTED for argument sets outside the kernel's layout requirements
+ * (those of bgtq_decode_attn's fast path, any gqa <= 128); callers then use
+ * bgtq_dequant_kv and an attention of their own.
+ */
+int bgtq_prefill_attn(const bgtq_head_plan* plans,
+                      const void* q_rot, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                      const void* k_packed, int64_t kp_sb, int64_t kp_sh, int64_t kp_st, int k_row_width,
+                      const void* k_norms, int64_t kn_sb, int64_t kn_sh, int64_t kn_st,
+                      const void* v_packed, int64_t vp_sb, int64_t vp_sh, int64_t vp_st, int v_row_width,
+                      const void* v_norms, int64_t vn_sb, int64_t vn_sh, int64_t vn_st,
+                      int B, int n_kv, int gqa, int S, int T, int q_pos_offset, int is_causal,
+                      int k_layout, int v_layout, float scale, int unrotate,
+                      void* out, int64_t o_sb, int64_t o_sh, int64_t o_ss, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

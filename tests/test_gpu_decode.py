@@ -600,6 +600,55 @@ def test_prompt_attention_rows_equal_decode_steps():
         assert (full[:, :, s].float() - dec.float()).abs().max() < TOL
 
 
+@pytest.mark.parametrize("gqa,n_kv,B,T,S,kl,vl,vb,mn,mx,causal", [
+    (8, 2, 2, 333, 333, 0, 0, 3, 1, 6, True),      # whole prompt, two tiles and a tail per late block
+    (4, 2, 1, 500, 77, 1, 1, 3, 1, 8, True),       # a later chunk of queries, nibble records, raw-byte units
+    (1, 3, 1, 200, 200, 0, 0, 2, 0, 4, True),      # one query head per KV head, 0-bit blocks, 2-bit V
+    (3, 1, 2, 190, 190, 0, 1, 4, 1, 5, True),      # query groups that do not divide the 128 rows of a work-group
+    (16, 1, 1, 130, 130, 1, 0, 4, 2, 8, True),
+    (8, 1, 1, 150, 40, 0, 0, 3, 1, 5, False),      # no mask: every query sees all records
+])
+def test_prompt_kernel_all_heads_in_one_launch(oracle_lib, decode_path, gqa, n_kv, B, T, S, kl, vl, vb, mn, mx, causal):
+    """``bgtq_prefill_attn`` (every KV head and batch row in one launch) against fp64 attention over the
+    checker's dequantised records, row s seeing records t <= T - S + s."""
+    if decode_path == "generic":
+        pytest.skip("one kernel serves this entry point")
+    args, qs, _, kp, kn, vp, vn = _build(192 if mx > 4 else 128, mn, mx, vb, n_kv, gqa, B, T, seed=70 + gqa + kl,
+                                         k_layout=kl, v_layout=vl)
+    gen = torch.Generator().manual_seed(gqa)
+    q = (torch.randn(B, n_kv * gqa, S, 128, generator=gen) * 0.6).half().to(DEV)
+    q_rot = torch.stack([ops.rotate_q(args['plans'], q[:, :, s].contiguous(), n_kv) for s in range(S)], 2)
+    off = T - S
+    out = ops.prefill_attention_packed(args['plans'], q_rot.contiguous(), kp, kn, vp, vn, T, k_layout=kl, v_layout=vl,
+                                       is_causal=causal, q_pos_offset=off)
+    assert out is not None, "the kernel refused a layout it is meant to take"
+    assert out.shape == (B, n_kv * gqa, S, 128) and out.dtype == torch.float16
+    got = out.float().cpu().numpy()
+    for b in range(B):
+        for h in range(n_kv):
+            ref = _causal_reference(oracle_lib, args['plans_np'][h:h + 1], q_rot[b, h * gqa:(h + 1) * gqa].cpu().numpy(),
+                                    kp[b, h, :T].cpu().numpy(), kn[b, h, :T].cpu().numpy(), vp[b, h, :T].cpu().numpy(),
+                                    vn[b, h, :T].cpu().numpy(), kl, vl, vb, off if causal else T)
+            assert np.abs(got[b, h * gqa:(h + 1) * gqa] - ref).max() < TOL
+    # without the un-rotation the kernel's output times the V rotation is the same thing
+    raw = ops.prefill_attention_packed(args['plans'], q_rot.contiguous(), kp, kn, vp, vn, T, k_layout=kl, v_layout=vl,
+                                       is_causal=causal, q_pos_offset=off, unrotate=False)
+    v_rot = torch.stack([q8._v_rot.float() for q8 in qs]).to(DEV)
+    back = (raw.float().reshape(B, n_kv, gqa * S, 128) @ v_rot.unsqueeze(0)).reshape(B, n_kv * gqa, S, 128)
+    assert (back - out.float()).abs().max() < TOL
+
+
+def test_prompt_kernel_refuses_layouts_it_cannot_take():
+    """Strided K records or misaligned query rows come back as 'unsupported' (None here), so that callers
+    can take the dequantise-then-attend route; nothing is launched."""
+    args, qs, q_rot1, kp, kn, vp, vn = _build(192, 1, 5, 3, 1, 4, 1, 100, seed=5)
+    q = torch.zeros(1, 4, 8, 128, dtype=torch.float16, device=DEV)
+    wide = torch.zeros(1, 1, 102, kp.shape[-1] + 4, dtype=torch.uint8, device=DEV)
+    wide[..., :kp.shape[-1]] = kp
+    assert ops.prefill_attention_packed(args['plans'], q, wide[..., :kp.shape[-1]], kn, vp, vn, 100) is None
+    assert ops.prefill_attention_packed(args['plans'], q, kp, kn, vp, vn, 100) is not None
+
+
 def test_merge_entry_point_refuses_what_its_kernel_cannot_take():
     """Misaligned partial vectors and more partitions than the kernel's table holds come back
     as error codes from the C-ABI, before anything is launched."""
