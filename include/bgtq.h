@@ -427,7 +427,7 @@ int bgtq_dequant_kv(const bgtq_head_plan* plans,
  * Prompt-phase attention straight over the packed cache: S query tokens per
  * sequence attend to records [0, T), query token s seeing t <= q_pos_offset + s
  * when is_causal.  Every 64-token tile of records is dequantised once per block of
- * 128 query rows inside the kernel (same values as bgtq_dequant_kv writes), both
+ * 256 query rows inside the kernel (same values as bgtq_dequant_kv writes), both
  * products run on matrix cores, the V un-rotation (when unrotate != 0) is applied
  * before the fp16 store; no fp16 K/V tensor of the layer exists.  Replaces
  * _packed_prefill_kernel as driven by fused_blockgtq_prefill_attention
@@ -438,7 +438,7 @@ int bgtq_dequant_kv(const bgtq_head_plan* plans,
  *   cache      as for bgtq_decode_attn (same strides, layouts and row widths)
  *   out        fp16 [B][n_kv*gqa][S][128], strides o_sb/o_sh/o_ss in halves
  * Returns BGTQ_EUNSUPPORTED for argument sets outside the kernel's layout requirements
- * (those of bgtq_decode_attn's fast path, any gqa <= 128); callers then use
+ * (those of bgtq_decode_attn's fast path, any gqa <= 256); callers then use
  * bgtq_dequant_kv and an attention of their own.
  */
 int bgtq_prefill_attn(const bgtq_head_plan* plans,
