@@ -44,7 +44,7 @@ constexpr float REFRESH = 4.0f;
 constexpr int KROW = D * 2 + 16;             // bytes of a K tile row: rows 4 banks apart
 constexpr int VTROW = MT * 2 + 16;           // bytes of a transposed V tile row (one dim, 64 tokens)
 
-// LDS layout (bytes): [V table | K tables | unit programs | unit dims | raw K | K norms | V norms | raw V | K tile | V^T tile]
+// LDS layout (bytes): [V table | K tables | unit programs | unit dims | 2 x (raw K | K norms | V norms | raw V) | 2 x (K tile | V^T tile)]
 constexpr int VTAB_OFF = 0;
 constexpr int KTAB_OFF = BGTQ_VLUT_BYTES;
 constexpr int PROG_OFF = KTAB_OFF + BGTQ_LUT_IMAGE_BYTES;            // [MAX_UNITS][8] dwords
@@ -115,8 +115,10 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     const int lim = !row_ok ? 0 : a.causal ? min(a.T, a.q_pos_offset + sq + 1) : a.T;
 
     // ---- LDS areas
-    const uint32_t kraw = RAW_OFF, knraw = kraw + a.kt, vnraw = knraw + a.knr, vraw = vnraw + a.vnr;
-    const uint32_t ktile = vraw + a.vt, vtile = ktile + MT * KROW;
+    // two sets of raw buffers and two sets of dequantised tiles: set (tile & 1)
+    const uint32_t raw_set = (uint32_t)(a.kt + a.knr + a.vnr + a.vt);
+    const uint32_t tile_set = MT * KROW + D * VTROW;
+    const uint32_t tiles0 = RAW_OFF + 2 * raw_set;
 
     // ---- tables, unit programs and unit dims into LDS
     const uint32_t voff = (uint32_t)lane * 16;
@@ -163,6 +165,7 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     // wave 0 fetches the K records, wave 1 the V records, wave 2 both norm arrays
     auto issue_tile = [&](int tile) {
         const int t = tile * MT, nt = min(MT, t_end - t);
+        const uint32_t kraw = RAW_OFF + (uint32_t)(tile & 1) * raw_set, knraw = kraw + a.kt, vnraw = knraw + a.knr, vraw = vnraw + a.vnr;
         if (wave == 0) {
             dma_region<9>(kp_base - kph + (int64_t)t * krow, kraw, dma_shape((int)kph + nt * krow, voff), voff);
         } else if (wave == 1) {
@@ -175,9 +178,9 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     if (n_tiles > 0) issue_tile(0);
 
     // the K tile's columns of 0-bit dims are never written: zero them once
-    for (int i = tid; i < MT * (n_zero / 2); i += NTHR) {
-        const int t = i / (n_zero / 2), c = i - t * (n_zero / 2);
-        lds_put<uint32_t>(ktile + t * KROW + c * 4, 0u);
+    for (int i = tid; i < 2 * MT * (n_zero / 2); i += NTHR) {
+        const int t = i / (n_zero / 2), c = i - t * (n_zero / 2);        // t: row of set t / MT
+        lds_put<uint32_t>(tiles0 + (uint32_t)(t / MT) * tile_set + (uint32_t)(t % MT) * KROW + c * 4, 0u);
     }
 
     const float c2 = a.scale * 1.44269504088896340736f;        // scores in log2 units
@@ -188,8 +191,8 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     float m_ref = -INFINITY, l_part = 0.f;                       // per query (this half's share of the denominator)
 
     // K dequantisation: lane = token, wave w takes units w, w + NWAVES, ...
-    const uint32_t krow_l = kraw + kph + (uint32_t)lane * krow;
-    const uint32_t knrow_l = knraw + knph + (uint32_t)lane * kn_st * 2;
+    const uint32_t krow_l0 = RAW_OFF + kph + (uint32_t)lane * krow;                    // set 0; + raw_set for set 1
+    const uint32_t knrow_l0 = RAW_OFF + a.kt + knph + (uint32_t)lane * kn_st * 2;
     // V dequantisation: thread (token pair tp, unit pair up); code pair e of a unit's raw word is brought to
     // the table-index position by a rotation (the V table sits at LDS address 0)
     const int tp = tid & 31, up = tid >> 5;
@@ -199,12 +202,13 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     for (int e = 0; e < 4; e++) vrot[e] = (uint32_t)(2 * vbw * e - vtsh) & 31u;
     const uint32_t vfmask = ((1u << (2 * vbw)) - 1u) << vtsh, vbase = vrep ? rep : 0u;
 
-    for (int tile = 0; tile < n_tiles; tile++) {
-        const int t0 = tile * MT;
-        const int nt = min(MT, t_end - t0);                      // records of this tile; the rows behind them hold stale bytes
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wave's share of the raw tile (and, first time, of the tables)
-        __syncthreads();                                         // raw tile complete; the previous tile's products are done
-
+    // Dequantise raw tile `tile` (set tile & 1) into the K and V^T tiles of the same set.
+    auto dequant_tile = [&](int tile) {
+        const int nt = min(MT, t_end - tile * MT);               // records of this tile; the rows behind them hold stale bytes
+        const uint32_t set = (uint32_t)(tile & 1);
+        const uint32_t krow_l = krow_l0 + set * raw_set, knrow_l = knrow_l0 + set * raw_set;
+        const uint32_t vnraw = RAW_OFF + set * raw_set + a.kt + a.knr, vraw = vnraw + a.vnr;
+        const uint32_t ktile = tiles0 + set * tile_set, vtile = ktile + MT * KROW;
         // ---- K tile: fp16(centroid * norm), packed-dim order
         for (int u = wave; u < n_units; u += NTHR / 64) {
             const uint4v pa = lds_at<uint4v>(PROG_OFF + u * 32), pb = lds_at<uint4v>(PROG_OFF + u * 32 + 16);
@@ -269,8 +273,23 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
                 }
             }
         }
-        __syncthreads();                                         // tiles complete; the raw buffers are free
-        if (tile + 1 < n_tiles) issue_tile(tile + 1);
+    };
+
+    // Pipeline: while the products of tile i run, tile i + 1 is dequantised into the other set of tiles and the
+    // raw records of tile i + 2 stream into the set tile i's came from; one barrier per tile.
+    if (n_tiles > 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wave's share of raw tile 0 and of the tables
+        __syncthreads();
+        dequant_tile(0);
+        if (n_tiles > 1) issue_tile(1);
+    }
+    for (int tile = 0; tile < n_tiles; tile++) {
+        const int t0 = tile * MT;
+        const uint32_t ktile = tiles0 + (uint32_t)(tile & 1) * tile_set, vtile = ktile + MT * KROW;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wave's share of raw tile + 1
+        __syncthreads();    // raw tile + 1 and tiles `tile` complete; everyone is done with the products of tile - 1
+        if (tile + 1 < n_tiles) dequant_tile(tile + 1);
+        if (tile + 2 < n_tiles) issue_tile(tile + 2);           // (its raw set was last read before this barrier)
 
         // ---- S^T = K Q^T for the wave's 32 queries: 2 token blocks x 8 steps of 16 dims
         float16v Sc[2];
@@ -420,7 +439,7 @@ extern "C" int bgtq_prefill_attn(const bgtq_head_plan* plans,
     a.out = (uint16_t*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
     a.k_row_width = k_row_width; a.v_row_width = v_row_width; a.v_stride = (int)vp_st;
     const int raw = raw_bytes(k_row_width, (int)vp_st, (int)kn_st, a.kt, a.knr, a.vnr, a.vt);
-    const size_t smem = (size_t)RAW_OFF + raw + (size_t)MT * KROW + (size_t)D * VTROW;
+    const size_t smem = (size_t)RAW_OFF + 2 * ((size_t)raw + (size_t)MT * KROW + (size_t)D * VTROW);
     static std::atomic<int> ready{0};
     if (ready.load(std::memory_order_acquire) == 0) {
         // offsets into the dynamic LDS block are used as LDS addresses: holds only without static LDS
