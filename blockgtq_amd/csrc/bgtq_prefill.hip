@@ -18,9 +18,14 @@
 //
 // The exponentials are taken relative to a per-query reference that is only moved when a score
 // exceeds it (to the maximum + 4 in log2 units), so the accumulators are rescaled rarely.  At the
-// end O is normalised, un-rotated on v_mfma_f32_32x32x2_f32 against the plan's fp32 V rotation
-// (operands again taken from the accumulator registers under a permutation of the contraction
-// index) and stored as fp16.  No fp16 K/V tensor of the layer is written.
+// end O is normalised and un-rotated against the plan's fp32 V rotation, again on the fp16 matrix
+// cores: both factors are split into an fp16 head and an fp16 remainder and three of the four
+// products are summed in fp32 (operands once more taken from the accumulator registers under a
+// permutation of the contraction index), then stored as fp16.  No fp16 K/V tensor of the layer
+// is written.
+//
+// Work-groups are numbered so that every (batch row, KV head) pair of the query block that sees
+// most tokens starts first and the short blocks fill the tail of the launch.
 //
 // Reference behaviour: blockgtq/kernels/fused_packed_attention.py:1876-2594 (prefill kernel),
 // driver blockgtq/prefill.py:66-101.
@@ -40,16 +45,15 @@ constexpr int NTHR = 64 * NWAVES;
 constexpr int V_UNITS_PER_THREAD = 16 * 32 / NTHR;   // V tile: 32 token pairs x 16 units over the threads
 constexpr int MAX_UNITS = BGTQ_MAX_UNITS;
 constexpr int MAX_KN = 8;
+constexpr int UPW = (MAX_UNITS + NWAVES - 1) / NWAVES;   // K units per wave
 constexpr float REFRESH = 4.0f;
 constexpr int KROW = D * 2 + 16;             // bytes of a K tile row: rows 4 banks apart
 constexpr int VTROW = MT * 2 + 16;           // bytes of a transposed V tile row (one dim, 64 tokens)
 
-// LDS layout (bytes): [V table | K tables | unit programs | unit dims | 2 x (raw K | K norms | V norms | raw V) | 2 x (K tile | V^T tile)]
+// LDS layout (bytes): [V table | K tables | 2 x (raw K | K norms | V norms | raw V) | 2 x (K tile | V^T tile)]
 constexpr int VTAB_OFF = 0;
 constexpr int KTAB_OFF = BGTQ_VLUT_BYTES;
-constexpr int PROG_OFF = KTAB_OFF + BGTQ_LUT_IMAGE_BYTES;            // [MAX_UNITS][8] dwords
-constexpr int UNIT_OFF = PROG_OFF + MAX_UNITS * 32;                  // [MAX_UNITS] dwords
-constexpr int RAW_OFF = UNIT_OFF + MAX_UNITS * 4;
+constexpr int RAW_OFF = KTAB_OFF + BGTQ_LUT_IMAGE_BYTES;
 
 struct PrefillArgs {
     const bgtq_head_plan* plans;
@@ -90,12 +94,14 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int h = blockIdx.y, b = blockIdx.z;
+    const int h = blockIdx.x, b = blockIdx.y;
     const bgtq_head_plan& P = a.plans[h];
     const int gqa = a.gqa, kl = a.k_layout;
     const bool vnib = a.v_layout == BGTQ_V_NIBBLE;
     const int BQ = ROWS / gqa;                                   // query tokens per work-group
-    const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;         // the blocks that see most tokens start first
+    // work-groups start in the order of their index, x fastest: every (batch row, KV head) pair of the query
+    // block that sees most tokens first, so that the short blocks fill the tail of the launch
+    const int qb = (int)gridDim.z - 1 - (int)blockIdx.z;
     const int s0 = qb * BQ;
     const int krow = a.k_row_width, vrow = a.v_stride, kn_st = (int)a.kn_st;
     const int vbw = vnib ? 4 : (int)P.v_bits;                    // bits of a V code as stored
@@ -120,7 +126,7 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     const uint32_t tile_set = MT * KROW + D * VTROW;
     const uint32_t tiles0 = RAW_OFF + 2 * raw_set;
 
-    // ---- tables, unit programs and unit dims into LDS
+    // ---- tables into LDS
     const uint32_t voff = (uint32_t)lane * 16;
     {
         const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
@@ -136,8 +142,6 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
             else { src = kimg + (cc - vch) * 1024; dst = KTAB_OFF + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
             dma16(voff, src, __builtin_amdgcn_readfirstlane(dst), __builtin_amdgcn_ballot_w64((int)voff < left));
         }
-        if (tid < MAX_UNITS * 8) lds_put<uint32_t>(PROG_OFF + tid * 4, P.kprog[kl][tid >> 3][tid & 7]);
-        if (tid < MAX_UNITS) lds_put<uint32_t>(UNIT_OFF + tid * 4, P.kunit[kl][tid]);
     }
     const int n_units = min(P.n_units[kl], MAX_UNITS), n_pair = min(P.n_pair_units[kl], n_units);
     const uint32_t kend = P.kend[kl], kfirst0 = P.kfirst[kl][0], kfirst1 = P.kfirst[kl][1];
@@ -190,7 +194,7 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     for (int db = 0; db < 4; db++) O[db] = (float16v){0};
     float m_ref = -INFINITY, l_part = 0.f;                       // per query (this half's share of the denominator)
 
-    // K dequantisation: lane = token, wave w takes units w, w + NWAVES, ...
+    // K dequantisation: lane = token, wave w takes units w, w + NWAVES, ... (parameters: ku[] below)
     const uint32_t krow_l0 = RAW_OFF + kph + (uint32_t)lane * krow;                    // set 0; + raw_set for set 1
     const uint32_t knrow_l0 = RAW_OFF + a.kt + knph + (uint32_t)lane * kn_st * 2;
     // V dequantisation: thread (token pair tp, unit pair up); code pair e of a unit's raw word is brought to
@@ -202,6 +206,29 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     for (int e = 0; e < 4; e++) vrot[e] = (uint32_t)(2 * vbw * e - vtsh) & 31u;
     const uint32_t vfmask = ((1u << (2 * vbw)) - 1u) << vtsh, vbase = vrep ? rep : 0u;
 
+    // The K units of this wave (w, w + NWAVES, ...): their parameters stay in scalar registers for the
+    // whole walk.  A unit the wave does not have reads valid addresses and stores nothing (len 0).
+    struct KUnit { uint32_t rot[4], mask, tab, repm, off, d0x2, seg2; int len; bool raw; };
+    KUnit ku[UPW];
+#pragma unroll
+    for (int i = 0; i < UPW; i++) {
+        const int u = wave + i * NWAVES;
+        const bool have = u < n_units;
+        const int uu = have ? u : 0;
+        const uint32_t dsc = P.kunit[kl][uu];
+        ku[i].len = have ? (int)(dsc >> 8) & 0xFF : 0;
+        ku[i].d0x2 = (dsc & 0xFF) * 2;
+        ku[i].raw = have && ku[i].len > 0 && u >= n_pair;
+        const bool pair = have && ku[i].len > 0 && u < n_pair;
+#pragma unroll
+        for (int e = 0; e < 4; e++) ku[i].rot[e] = pair ? P.kprog[kl][uu][e] : 0u;
+        ku[i].mask = pair ? P.kprog[kl][uu][4] : 0u;
+        ku[i].tab = ku[i].len > 0 ? P.kprog[kl][uu][5] : (uint32_t)KTAB_OFF;
+        ku[i].repm = pair ? P.kprog[kl][uu][6] : 0u;
+        ku[i].off = ku[i].len == 0 ? 0u : uu == 0 ? kfirst0 : uu == 1 ? kfirst1 : P.kprog[kl][uu - 2][7];
+        ku[i].seg2 = ku[i].len == 0 ? 0u : 2u * (uint32_t)__builtin_popcount(kend & ((1u << uu) - 1u));
+    }
+
     // Dequantise raw tile `tile` (set tile & 1) into the K and V^T tiles of the same set.
     auto dequant_tile = [&](int tile) {
         const int nt = min(MT, t_end - tile * MT);               // records of this tile; the rows behind them hold stale bytes
@@ -209,39 +236,48 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
         const uint32_t krow_l = krow_l0 + set * raw_set, knrow_l = knrow_l0 + set * raw_set;
         const uint32_t vnraw = RAW_OFF + set * raw_set + a.kt + a.knr, vraw = vnraw + a.vnr;
         const uint32_t ktile = tiles0 + set * tile_set, vtile = ktile + MT * KROW;
-        // ---- K tile: fp16(centroid * norm), packed-dim order
-        for (int u = wave; u < n_units; u += NTHR / 64) {
-            const uint4v pa = lds_at<uint4v>(PROG_OFF + u * 32), pb = lds_at<uint4v>(PROG_OFF + u * 32 + 16);
-            const uint32_t dsc = lds_at<uint32_t>(UNIT_OFF + u * 4);
-            const int d0 = (int)(dsc & 0xFF), len = (int)(dsc >> 8) & 0xFF;
-            if (len == 0) continue;                              // (wave-uniform) the empty unit that evens out the pair units
-            const uint32_t off = u == 0 ? kfirst0 : u == 1 ? kfirst1 : lds_at<uint32_t>(PROG_OFF + (u - 2) * 32 + 28);
-            const int seg = __builtin_popcount(kend & ((1u << u) - 1u));
-            // rows past the tile's last record get norm 0: their products must stay finite (P is 0 there)
-            const uint32_t n16 = lane < nt ? (uint32_t)lds_at<uint16_t>(knrow_l + seg * 2) : 0u;
-            const uint32_t nn = n16 | (n16 << 16);
-            uint32_t w[4];
-            if (u < n_pair) {
-                const uint32_t r = lds_codes4(krow_l + off);
-                const uint32_t base = and_or_v(rep, pb.z, pb.y);
-                w[0] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.x), pb.x, base));
-                w[1] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.y), pb.x, base));
-                w[2] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.z), pb.x, base));
-                w[3] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, pa.w), pb.x, base));
-            } else {
-                const uint2v r = lds_codes8(krow_l + off);
+        // ---- K tile: fp16(centroid * norm), packed-dim order.  The wave's units go through three
+        // branch-free stages (codes and norms, table lookups, products and stores), so that the LDS
+        // round trips of all its units overlap.
+        {
+            uint32_t nn[UPW];
+            uint2v rr[UPW];
+            uint32_t w[UPW][4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const uint32_t x = e < 2 ? r.x : r.y;
-                    const uint32_t c0 = pb.y + ((x >> ((e & 1) * 16)) & 0xFF) * 2;
-                    const uint32_t c1 = pb.y + ((x >> ((e & 1) * 16 + 8)) & 0xFF) * 2;
-                    w[e] = (uint32_t)lds_at<uint16_t>(c0) | ((uint32_t)lds_at<uint16_t>(c1) << 16);
+            for (int i = 0; i < UPW; i++) {
+                // rows past the tile's last record get norm 0: their products must stay finite (P is 0 there)
+                const uint32_t n16 = lane < nt ? (uint32_t)lds_at<uint16_t>(knrow_l + ku[i].seg2) : 0u;
+                nn[i] = n16 | (n16 << 16);
+                rr[i] = lds_codes8(krow_l + ku[i].off);
+            }
+#pragma unroll
+            for (int i = 0; i < UPW; i++) {
+                const uint32_t r = rr[i].x;
+                const uint32_t base = and_or(rep, ku[i].repm, ku[i].tab);
+                w[i][0] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[0]), ku[i].mask, base));
+                w[i][1] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[1]), ku[i].mask, base));
+                w[i][2] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[2]), ku[i].mask, base));
+                w[i][3] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[3]), ku[i].mask, base));
+            }
+#pragma unroll
+            for (int i = 0; i < UPW; i++) {
+                if (ku[i].raw) {                                 // (wave-uniform) one byte per code, one fp16 per table entry
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t x = e < 2 ? rr[i].x : rr[i].y;
+                        const uint32_t c0 = ku[i].tab + ((x >> ((e & 1) * 16)) & 0xFF) * 2;
+                        const uint32_t c1 = ku[i].tab + ((x >> ((e & 1) * 16 + 8)) & 0xFF) * 2;
+                        w[i][e] = (uint32_t)lds_at<uint16_t>(c0) | ((uint32_t)lds_at<uint16_t>(c1) << 16);
+                    }
                 }
             }
-            const uint32_t dst = ktile + (uint32_t)lane * KROW + (uint32_t)d0 * 2;
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (2 * e < len) lds_put<uint32_t>(dst + e * 4, pk_mul_f16(w[e], nn));
+            for (int i = 0; i < UPW; i++) {
+                const uint32_t dst = ktile + (uint32_t)lane * KROW + ku[i].d0x2;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (2 * e < ku[i].len) lds_put<uint32_t>(dst + e * 4, pk_mul_f16(w[i][e], nn[i]));
+            }
         }
 
         // ---- V^T tile: fp16(centroid * norm), [dim][token]; thread = tokens 2 tp, 2 tp + 1 of V_UNITS_PER_THREAD units
@@ -363,7 +399,8 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
             }
     }
 
-    // ---- normalise; un-rotate: out^T = R^T O^T, contraction slot g of step (db, r) is dim 32 db + 8 (r / 4) + 4 g + r % 4
+    // ---- normalise; un-rotate: out^T = R^T O^T on the fp16 matrix cores with both factors split into an
+    // fp16 head and an fp16 remainder (x = hi + lo up to 2^-22 |x|; the lo * lo product is dropped), fp32 sums
     const float l_tot = l_part + __shfl_xor(l_part, 32, 64);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
 #pragma unroll
@@ -372,18 +409,71 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
         for (int r = 0; r < 16; r++) O[db][r] *= inv;
     float16v R[4];
     if (a.unrotate) {
+        // R^T goes through LDS (the tiles are dead): row o = output dim, 128 fp16 heads in the order the MFMA
+        // wants its contraction slots, position 32 db + 16 s + 8 g + e <-> dim 32 db + 16 s + 8 (e / 4) + 4 g + e % 4
+        // (what register 8 s + e of accumulator block db holds in half-wave g); the remainders follow at RT_LO.
+        constexpr uint32_t RT_ROW = D * 2 + 16, RT_LO = D * RT_ROW;
+        static_assert(2 * RT_LO <= 2 * (MT * KROW + D * VTROW), "both halves of R^T fit into the tile sets");
+        __syncthreads();                                        // every wave is done with the tiles
         const float* rot = P.v_rot;
+        for (int idx = tid; idx < D * 4; idx += NTHR) {
+            const int o = idx & (D - 1), dq = idx >> 7;         // this thread: column o of rows 32 dq .. 32 dq + 31
+            float x[32];
 #pragma unroll
-        for (int ob = 0; ob < 4; ob++) R[ob] = (float16v){0};
+            for (int i = 0; i < 32; i++) x[i] = rot[(32 * dq + i) * D + o];
+#pragma unroll
+            for (int g8 = 0; g8 < 4; g8++) {                    // positions 8 g8 .. 8 g8 + 7 of the block: s = g8 / 2, g = g8 % 2
+                uint32_t hi[4], lo[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int e0 = 2 * j, e1 = 2 * j + 1;
+                    const float x0 = x[16 * (g8 >> 1) + 8 * (e0 >> 2) + 4 * (g8 & 1) + (e0 & 3)];
+                    const float x1 = x[16 * (g8 >> 1) + 8 * (e1 >> 2) + 4 * (g8 & 1) + (e1 & 3)];
+                    const _Float16 h0 = (_Float16)x0, h1 = (_Float16)x1;
+                    hi[j] = cvt_pk_f16((float)h0, (float)h1);
+                    lo[j] = cvt_pk_f16(x0 - (float)h0, x1 - (float)h1);
+                }
+                const uint32_t dst = (uint32_t)o * RT_ROW + (uint32_t)(32 * dq + 8 * g8) * 2;
+                lds_put<uint4v>(dst, (uint4v){hi[0], hi[1], hi[2], hi[3]});
+                lds_put<uint4v>(RT_LO + dst, (uint4v){lo[0], lo[1], lo[2], lo[3]});
+            }
+        }
+        // the wave's O^T as B operands: step (db, s) takes registers 8 s .. 8 s + 7 of block db
+        half8 Bh[8], Bl[8];
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int d = 32 * db + 8 * (r >> 2) + 4 * lg + (r & 3);
+            for (int sst = 0; sst < 2; sst++) {
+                uint32_t hi[4], lo[4];
 #pragma unroll
-                for (int ob = 0; ob < 4; ob++)
-                    R[ob] = __builtin_amdgcn_mfma_f32_32x32x2f32(rot[d * D + 32 * ob + li], O[db][r], R[ob], 0, 0, 0);
+                for (int j = 0; j < 4; j++) {
+                    const float x0 = O[db][8 * sst + 2 * j], x1 = O[db][8 * sst + 2 * j + 1];
+                    const _Float16 h0 = (_Float16)x0, h1 = (_Float16)x1;
+                    hi[j] = cvt_pk_f16((float)h0, (float)h1);
+                    lo[j] = cvt_pk_f16(x0 - (float)h0, x1 - (float)h1);
+                }
+                Bh[2 * db + sst] = __builtin_bit_cast(half8, (uint4v){hi[0], hi[1], hi[2], hi[3]});
+                Bl[2 * db + sst] = __builtin_bit_cast(half8, (uint4v){lo[0], lo[1], lo[2], lo[3]});
             }
+        __syncthreads();
+#pragma unroll
+        for (int ob = 0; ob < 4; ob++) R[ob] = (float16v){0};
+#pragma unroll
+        for (int st = 0; st < 8; st++) {                        // four independent accumulators per pass
+            half8 Ah[4], Al[4];
+#pragma unroll
+            for (int ob = 0; ob < 4; ob++) {
+                const uint32_t arow = (uint32_t)(32 * ob + li) * RT_ROW + (uint32_t)lg * 16 + st * 32;
+                Ah[ob] = lds_at<half8>(arow);
+                Al[ob] = lds_at<half8>(RT_LO + arow);
+            }
+#pragma unroll
+            for (int ob = 0; ob < 4; ob++) R[ob] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Ah[ob], Bh[st], R[ob], 0, 0, 0);
+#pragma unroll
+            for (int ob = 0; ob < 4; ob++) R[ob] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Al[ob], Bh[st], R[ob], 0, 0, 0);
+#pragma unroll
+            for (int ob = 0; ob < 4; ob++) R[ob] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Ah[ob], Bl[st], R[ob], 0, 0, 0);
+        }
     } else {
 #pragma unroll
         for (int ob = 0; ob < 4; ob++) R[ob] = O[ob];
@@ -452,7 +542,8 @@ extern "C" int bgtq_prefill_attn(const bgtq_head_plan* plans,
     }
     if (ready.load(std::memory_order_acquire) < 0 || smem > 160 * 1024) return BGTQ_EUNSUPPORTED;
     const int BQ = ROWS / gqa;
-    dim3 grid((unsigned)((S + BQ - 1) / BQ), (unsigned)n_kv, (unsigned)B);
+    if ((S + BQ - 1) / BQ > 65535 || B > 65535) return BGTQ_EUNSUPPORTED;
+    dim3 grid((unsigned)n_kv, (unsigned)B, (unsigned)((S + BQ - 1) / BQ));
     hipLaunchKernelGGL(prefill_mfma_kernel, grid, dim3(NTHR), smem, (hipStream_t)stream, a);
     return bgtq_launch_status();
 }
