@@ -236,77 +236,78 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
         const uint32_t krow_l = krow_l0 + set * raw_set, knrow_l = knrow_l0 + set * raw_set;
         const uint32_t vnraw = RAW_OFF + set * raw_set + a.kt + a.knr, vraw = vnraw + a.vnr;
         const uint32_t ktile = tiles0 + set * tile_set, vtile = ktile + MT * KROW;
-        // ---- K tile: fp16(centroid * norm), packed-dim order.  The wave's units go through three
-        // branch-free stages (codes and norms, table lookups, products and stores), so that the LDS
-        // round trips of all its units overlap.
-        {
-            uint32_t nn[UPW];
-            uint2v rr[UPW];
-            uint32_t w[UPW][4];
+        // K tile [token][dim] (packed-dim order) and V^T tile [dim][token], both fp16(centroid * norm).  K: lane =
+        // token, the wave's own units; V: thread = tokens 2 tp, 2 tp + 1 of V_UNITS_PER_THREAD units.  Both go
+        // through the same three stages together, without a branch between them, so that all LDS round trips
+        // of a stage overlap: codes and norms, table lookups, products and stores.
+        uint32_t nn[UPW], kw[UPW][4];
+        uint2v rr[UPW];
+        uint32_t nrm[2], vr[V_UNITS_PER_THREAD][2], vw[V_UNITS_PER_THREAD][2][4];
+        // ---- stage 1
 #pragma unroll
-            for (int i = 0; i < UPW; i++) {
-                // rows past the tile's last record get norm 0: their products must stay finite (P is 0 there)
-                const uint32_t n16 = lane < nt ? (uint32_t)lds_at<uint16_t>(knrow_l + ku[i].seg2) : 0u;
-                nn[i] = n16 | (n16 << 16);
-                rr[i] = lds_codes8(krow_l + ku[i].off);
-            }
+        for (int i = 0; i < UPW; i++) {
+            // rows past the tile's last record get norm 0: their products must stay finite (P is 0 there)
+            const uint32_t n16 = lds_at<uint16_t>(knrow_l + ku[i].seg2);
+            nn[i] = lane < nt ? n16 | (n16 << 16) : 0u;
+            rr[i] = lds_codes8(krow_l + ku[i].off);
+        }
 #pragma unroll
-            for (int i = 0; i < UPW; i++) {
-                const uint32_t r = rr[i].x;
-                const uint32_t base = and_or(rep, ku[i].repm, ku[i].tab);
-                w[i][0] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[0]), ku[i].mask, base));
-                w[i][1] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[1]), ku[i].mask, base));
-                w[i][2] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[2]), ku[i].mask, base));
-                w[i][3] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[3]), ku[i].mask, base));
-            }
+        for (int j = 0; j < 2; j++) {
+            const uint32_t n16 = lds_at<uint16_t>(vnraw + vnph + (uint32_t)(2 * tp + j) * 2);
+            nrm[j] = 2 * tp + j < nt ? n16 | (n16 << 16) : 0u;
+        }
 #pragma unroll
-            for (int i = 0; i < UPW; i++) {
-                if (ku[i].raw) {                                 // (wave-uniform) one byte per code, one fp16 per table entry
+        for (int uu = 0; uu < V_UNITS_PER_THREAD; uu++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const uint32_t x = e < 2 ? rr[i].x : rr[i].y;
-                        const uint32_t c0 = ku[i].tab + ((x >> ((e & 1) * 16)) & 0xFF) * 2;
-                        const uint32_t c1 = ku[i].tab + ((x >> ((e & 1) * 16 + 8)) & 0xFF) * 2;
-                        w[i][e] = (uint32_t)lds_at<uint16_t>(c0) | ((uint32_t)lds_at<uint16_t>(c1) << 16);
-                    }
-                }
-            }
+            for (int j = 0; j < 2; j++)
+                vr[uu][j] = lds_codes4(vraw + vph + (uint32_t)(2 * tp + j) * vrow + (uint32_t)((V_UNITS_PER_THREAD * up + uu) * vbw));
+        // ---- stage 2
 #pragma unroll
-            for (int i = 0; i < UPW; i++) {
-                const uint32_t dst = ktile + (uint32_t)lane * KROW + ku[i].d0x2;
+        for (int i = 0; i < UPW; i++) {
+            const uint32_t r = rr[i].x;
+            const uint32_t base = and_or(rep, ku[i].repm, ku[i].tab);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                kw[i][e] = lds_at<uint32_t>(and_or(__builtin_amdgcn_alignbit(r, r, ku[i].rot[e]), ku[i].mask, base));
+        }
+#pragma unroll
+        for (int uu = 0; uu < V_UNITS_PER_THREAD; uu++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    if (2 * e < ku[i].len) lds_put<uint32_t>(dst + e * 4, pk_mul_f16(w[i][e], nn[i]));
-            }
-        }
-
-        // ---- V^T tile: fp16(centroid * norm), [dim][token]; thread = tokens 2 tp, 2 tp + 1 of V_UNITS_PER_THREAD units
-        {
-            uint32_t nrm[2];
+                    vw[uu][j][e] = lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(vr[uu][j], vr[uu][j], vrot[e]), vfmask, vbase));
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const uint32_t n16 = 2 * tp + j < nt ? (uint32_t)lds_at<uint16_t>(vnraw + vnph + (uint32_t)(2 * tp + j) * 2) : 0u;
-                nrm[j] = n16 | (n16 << 16);
-            }
-#pragma unroll
-            for (int uu = 0; uu < V_UNITS_PER_THREAD; uu++) {
-                const int u = V_UNITS_PER_THREAD * up + uu;
-                uint32_t w[2][4];
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const uint32_t r = lds_codes4(vraw + vph + (uint32_t)(2 * tp + j) * vrow + (uint32_t)(u * vbw));
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        w[j][e] = pk_mul_f16(lds_at<uint32_t>(and_or_v(__builtin_amdgcn_alignbit(r, r, vrot[e]), vfmask, vbase)), nrm[j]);
-                }
+        for (int i = 0; i < UPW; i++) {
+            if (ku[i].raw) {                                     // (wave-uniform) one byte per code, one fp16 per table entry
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    // (dim 8u + 2e of both tokens), (dim 8u + 2e + 1 of both tokens)
-                    const uint32_t lo = __builtin_amdgcn_perm(w[1][e], w[0][e], 0x05040100u);
-                    const uint32_t hi = __builtin_amdgcn_perm(w[1][e], w[0][e], 0x07060302u);
-                    lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e) * VTROW + (uint32_t)tp * 4, lo);
-                    lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e + 1) * VTROW + (uint32_t)tp * 4, hi);
+                    const uint32_t x = e < 2 ? rr[i].x : rr[i].y;
+                    const uint32_t c0 = ku[i].tab + ((x >> ((e & 1) * 16)) & 0xFF) * 2;
+                    const uint32_t c1 = ku[i].tab + ((x >> ((e & 1) * 16 + 8)) & 0xFF) * 2;
+                    kw[i][e] = (uint32_t)lds_at<uint16_t>(c0) | ((uint32_t)lds_at<uint16_t>(c1) << 16);
                 }
+            }
+        }
+        // ---- stage 3.  A dim pair past the unit's last dim goes to the 16 spare bytes at the end of the lane's
+        // K tile row, which nothing reads.
+        const uint32_t krow_t = ktile + (uint32_t)lane * KROW;
+#pragma unroll
+        for (int i = 0; i < UPW; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                lds_put<uint32_t>(krow_t + (2 * e < ku[i].len ? ku[i].d0x2 + e * 4 : (uint32_t)(D * 2)), pk_mul_f16(kw[i][e], nn[i]));
+#pragma unroll
+        for (int uu = 0; uu < V_UNITS_PER_THREAD; uu++) {
+            const int u = V_UNITS_PER_THREAD * up + uu;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t w0 = pk_mul_f16(vw[uu][0][e], nrm[0]), w1 = pk_mul_f16(vw[uu][1][e], nrm[1]);
+                // (dim 8u + 2e of both tokens), (dim 8u + 2e + 1 of both tokens)
+                const uint32_t lo = __builtin_amdgcn_perm(w1, w0, 0x05040100u);
+                const uint32_t hi = __builtin_amdgcn_perm(w1, w0, 0x07060302u);
+                lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e) * VTROW + (uint32_t)tp * 4, lo);
+                lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e + 1) * VTROW + (uint32_t)tp * 4, hi);
             }
         }
     };
