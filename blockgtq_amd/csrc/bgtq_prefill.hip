@@ -200,19 +200,24 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     // V dequantisation: thread (token pair tp, unit pair up); code pair e of a unit's raw word is brought to
     // the table-index position by a rotation (the V table sits at LDS address 0)
     const int tp = tid & 31, up = tid >> 5;
+    // Column order of the V^T tile: inside every group of 16 tokens, token x sits at position
+    // 8 ((x >> 2) & 1) + 4 (x >> 3) + (x & 3), so that the 8 tokens {4 g + i, 8 + 4 g + i} a half-wave g contracts in
+    // one MFMA step are 16 contiguous bytes.  Tokens 2 tp and 2 tp + 1 stay neighbours: byte offset of their dword
+    const uint32_t vcol = (uint32_t)(8 * (tp >> 3) + 4 * ((tp >> 1) & 1) + 2 * ((tp >> 2) & 1) + (tp & 1)) * 4;
     const int vtsh = vrep ? 7 : 2;
     uint32_t vrot[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) vrot[e] = (uint32_t)(2 * vbw * e - vtsh) & 31u;
     const uint32_t vfmask = ((1u << (2 * vbw)) - 1u) << vtsh, vbase = vrep ? rep : 0u;
 
-    // The K units of this wave (w, w + NWAVES, ...): their parameters stay in scalar registers for the
+    // The K units of this wave (w, w + NWAVES, then the third round shifted by half): their parameters stay in scalar registers for the
     // whole walk.  A unit the wave does not have reads valid addresses and stores nothing (len 0).
     struct KUnit { uint32_t rot[4], mask, tab, repm, off, d0x2, seg2; int len; bool raw; };
     KUnit ku[UPW];
 #pragma unroll
     for (int i = 0; i < UPW; i++) {
-        const int u = wave + i * NWAVES;
+        // the third round starts at wave NWAVES / 2: the first waves also issue the tile loads
+        const int u = i < 2 ? wave + i * NWAVES : i * NWAVES + (wave + NWAVES / 2) % NWAVES;
         const bool have = u < n_units;
         const int uu = have ? u : 0;
         const uint32_t dsc = P.kunit[kl][uu];
@@ -306,8 +311,8 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
                 // (dim 8u + 2e of both tokens), (dim 8u + 2e + 1 of both tokens)
                 const uint32_t lo = __builtin_amdgcn_perm(w1, w0, 0x05040100u);
                 const uint32_t hi = __builtin_amdgcn_perm(w1, w0, 0x07060302u);
-                lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e) * VTROW + (uint32_t)tp * 4, lo);
-                lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e + 1) * VTROW + (uint32_t)tp * 4, hi);
+                lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e) * VTROW + vcol, lo);
+                lds_put<uint32_t>(vtile + (uint32_t)(8 * u + 2 * e + 1) * VTROW + vcol, hi);
             }
         }
     };
@@ -389,13 +394,11 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
             for (int hf = 0; hf < 2; hf++) {
                 const uint4v pw = {Pw[tb][4 * hf], Pw[tb][4 * hf + 1], Pw[tb][4 * hf + 2], Pw[tb][4 * hf + 3]};
                 const half8 Bp = __builtin_bit_cast(half8, pw);
-                const uint32_t col = (uint32_t)(32 * tb + 16 * hf + 4 * lg) * 2;
+                const uint32_t col = (uint32_t)(32 * tb + 16 * hf + 8 * lg) * 2;
 #pragma unroll
                 for (int db = 0; db < 4; db++) {
-                    const uint32_t vr = vtile + (uint32_t)(32 * db + li) * VTROW + col;
-                    const uint2v x0 = lds_at<uint2v>(vr), x1 = lds_at<uint2v>(vr + 16);
-                    const uint4v av = {x0.x, x0.y, x1.x, x1.y};
-                    O[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, av), Bp, O[db], 0, 0, 0);
+                    const half8 av = lds_at<half8>(vtile + (uint32_t)(32 * db + li) * VTROW + col);
+                    O[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, Bp, O[db], 0, 0, 0);
                 }
             }
     }
