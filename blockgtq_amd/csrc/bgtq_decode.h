@@ -23,6 +23,8 @@ struct DecodeArgs {
     int v_row_width;
     int nw;                // MFMA kernel: waves per work-group
     TileLayout tl;
+    int wave_bytes;        // MFMA kernel: LDS bytes of one wave's buffers
+    int per_tiles, rem_tiles;   // MFMA kernel, equal row lengths: tiles per partition, partitions with one more
 };
 
 // Fast path: MFMA kernel for bit-packed K and V records (bgtq_decode_mfma.hip).

@@ -151,9 +151,13 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
 
     // ---- this partition's tiles: the tiles of the row are dealt to the partitions as evenly as
     // whole tiles allow (partition sizes differ by at most one tile)
-    const int T = a.seq_lens ? a.seq_lens[b] : a.T;
-    const int n_tiles = (T + MT - 1) / MT;
-    const int per = n_tiles / a.n_splits, rem = n_tiles - per * a.n_splits;
+    int T = a.T, per = a.per_tiles, rem = a.rem_tiles;        // (the launcher divides when every row has T records)
+    if (a.seq_lens) {
+        T = a.seq_lens[b];
+        const int n_tiles = (T + MT - 1) / MT;
+        per = n_tiles / a.n_splits;
+        rem = n_tiles - per * a.n_splits;
+    }
     const int tile_lo = c * per + min(c, rem), tile_hi = tile_lo + per + (c < rem ? 1 : 0);
     const int t0 = tile_lo * MT, t1 = min(tile_hi * MT, T);
 
@@ -161,7 +165,12 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     constexpr int vrow = VST;
     const int kn_st = (int)a.kn_st;
     const TileLayout tl = a.tl;
-    const uint16_t* q_src = a.q + b * a.q_sb + (int64_t)h * gqa * a.q_sh;
+    // byte offset of (row b, KV head h) of a tensor whose strides (in elements of `elem` bytes) the launcher
+    // has checked to fit 32 bits
+    auto at_bh = [&](int64_t sb, int64_t sh, int elem) -> uint64_t {
+        return ((uint64_t)(uint32_t)b * (uint32_t)sb + (uint64_t)(uint32_t)h * (uint32_t)sh) * (uint32_t)elem;
+    };
+    const uint16_t* q_src = (const uint16_t*)((const uint8_t*)a.q + ((uint64_t)(uint32_t)b * (uint32_t)a.q_sb + (uint64_t)(uint32_t)(h * gqa) * (uint32_t)a.q_sh) * 2u);
     const int n_units = min(P.n_units[kl], MAX_UNITS);
     const int n_pair = min(P.n_pair_units[kl], n_units);
     const uint32_t kend = P.kend[kl], kfirst0 = P.kfirst[kl][0], kfirst1 = P.kfirst[kl][1];
@@ -220,14 +229,14 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     }
 
     // ---- per-wave buffers and streaming sources: 16-byte aligned bases and phases (constant per tile) ----
-    const int wave_bytes = wave_lds_bytes(tl);
+    const int wave_bytes = a.wave_bytes;
     const uint32_t kbuf = WAVES_OFF + wave * wave_bytes;                       // K records, K norms, V norms
     const uint32_t vbuf = kbuf + tl.kbuf;                                     // V records
     const uint32_t pbuf = vbuf + tl.vt;                                       // P * v_norm of the tile
-    const uint8_t* kp_base = a.kp + b * a.kp_sb + h * a.kp_sh;
-    const uint8_t* vp_base = a.vp + b * a.vp_sb + h * a.vp_sh;
-    const uint8_t* kn_base = (const uint8_t*)(a.kn + b * a.kn_sb + h * a.kn_sh);
-    const uint8_t* vn_base = (const uint8_t*)(a.vn + b * a.vn_sb + h * a.vn_sh);
+    const uint8_t* kp_base = a.kp + at_bh(a.kp_sb, a.kp_sh, 1);
+    const uint8_t* vp_base = a.vp + at_bh(a.vp_sb, a.vp_sh, 1);
+    const uint8_t* kn_base = (const uint8_t*)a.kn + at_bh(a.kn_sb, a.kn_sh, 2);
+    const uint8_t* vn_base = (const uint8_t*)a.vn + at_bh(a.vn_sb, a.vn_sh, 2);
     const uint32_t kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
     const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
     // The shapes of a full tile are the same for every tile of the partition.
@@ -236,11 +245,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     // Sources of the wave's next tile (16-byte aligned: the phase stays in the LDS offset); they move on by
     // the wave's tile stride after every issue.
     const int step_tiles = nw * MT;
-    const int64_t first = t0 + wave * MT;
-    const uint8_t* k_src = kp_base - kph + first * krow;
-    const uint8_t* kn_src = kn_base - knph + first * kn_st * 2;
-    const uint8_t* vn_src = vn_base - vnph + first * 2;
-    const uint8_t* v_src = vp_base - vph + first * vrow;
+    const uint32_t first = (uint32_t)(t0 + wave * MT);          // (a (row, head) slice is below 4 GB: checked by the launcher)
+    const uint8_t* k_src = kp_base - kph + first * (uint32_t)krow;
+    const uint8_t* kn_src = kn_base - knph + first * (uint32_t)(kn_st * 2);
+    const uint8_t* vn_src = vn_base - vnph + first * 2u;
+    const uint8_t* v_src = vp_base - vph + first * (uint32_t)vrow;
     const int k_step = step_tiles * krow, kn_step = step_tiles * kn_st * 2, vn_step = step_tiles * 2, v_step = step_tiles * vrow;
     // K records and both norm arrays of a tile go to the K buffer; returns the loads issued.
     auto issue_k = [&](int tile) -> int {
@@ -275,7 +284,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_mfma_kernel(DecodeArgs 
     // tables and the first K tile: all are needed now)
     {
         if (tid < N_QJOBS) lds_put<uint4v>(job_slot(tid), job0);
-        for (int j = tid + nthr; j < N_QJOBS; j += nthr) lds_put<uint4v>(job_slot(j), job_load(j));
+        if (nthr < N_QJOBS)                                   // (uniform) small work-groups only
+            for (int j = tid + nthr; j < N_QJOBS; j += nthr) lds_put<uint4v>(job_slot(j), job_load(j));
 #pragma unroll
         for (int i = 0; i < PBUF_BYTES; i += 1024)
             if (i + 1024 <= PBUF_BYTES || lane * 16 < PBUF_BYTES - i) lds_put<uint4v>(pbuf + i + lane * 16, (uint4v){0, 0, 0, 0});
@@ -603,6 +613,9 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
     const size_t smem = mfma_smem_bytes(a.tl, nw);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
     a.nw = nw;
+    a.wave_bytes = wave_lds_bytes(a.tl);
+    a.per_tiles = tiles / a.n_splits;
+    a.rem_tiles = tiles - a.per_tiles * a.n_splits;
     auto kern = decode_mfma_kernel<VBW, VST, TWO>;
     // 1: usable, -1: not usable.  Two threads racing through the first call both run the idempotent
     // set-up below and store the same value.
@@ -634,6 +647,15 @@ int launch(const DecodeArgs& a, hipStream_t st) {
 int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream) {
     // layout requirements of the fast path; anything else takes the generic kernel
     if (a.gqa > 8 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
+    // the kernel forms its addresses from 32-bit factors: batch and head strides, and the bytes of one
+    // (row, head) slice, must fit
+    {
+        const int64_t lim = (int64_t)1 << 32;
+        const int64_t strides[] = {a.q_sb, a.q_sh, a.kp_sb, a.kp_sh, a.kn_sb, a.kn_sh, a.vp_sb, a.vp_sh, a.vn_sb, a.vn_sh};
+        for (int64_t st : strides) if (st < 0 || st >= lim) return BGTQ_EUNSUPPORTED;
+        const int64_t rows = (int64_t)a.T + MT;
+        if (rows * a.kp_st >= lim || rows * a.vp_st >= lim || rows * a.kn_st * 2 >= lim) return BGTQ_EUNSUPPORTED;
+    }
     if ((a.kp_st & 3) || (a.kp_sb & 3) || (a.kp_sh & 3) || ((uintptr_t)a.kp & 3)) return BGTQ_EUNSUPPORTED;
     if ((a.vp_st & 3) || (a.vp_sb & 3) || (a.vp_sh & 3) || ((uintptr_t)a.vp & 3)) return BGTQ_EUNSUPPORTED;
     if (a.kp_st != a.k_row_width) return BGTQ_EUNSUPPORTED;   // K records contiguous
