@@ -197,9 +197,11 @@ __global__ __launch_bounds__(NTHR, 8 / NWAVES) void prefill_mfma_kernel(PrefillA
     // K dequantisation: lane = token, wave w takes units w, w + NWAVES, ... (parameters: ku[] below)
     const uint32_t krow_l0 = RAW_OFF + kph + (uint32_t)lane * krow;                    // set 0; + raw_set for set 1
     const uint32_t knrow_l0 = RAW_OFF + a.kt + knph + (uint32_t)lane * kn_st * 2;
-    // V dequantisation: thread (token pair tp, unit pair up); code pair e of a unit's raw word is brought to
-    // the table-index position by a rotation (the V table sits at LDS address 0)
-    const int tp = tid & 31, up = tid >> 5;
+    // V dequantisation: thread (token pair tp, unit up); code pair e of a unit's raw word is brought to
+    // the table-index position by a rotation (the V table sits at LDS address 0).  Neighbouring lanes take
+    // neighbouring units of one token pair: a half-wave then reads 16 token pairs (records 96 bytes apart fall on
+    // 8 banks) instead of 32
+    const int tp = (tid >> 1) & 31, up = 2 * (tid >> 6) + (tid & 1);
     // Column order of the V^T tile: inside every group of 16 tokens, token x sits at position
     // 8 ((x >> 2) & 1) + 4 (x >> 3) + (x & 3), so that the 8 tokens {4 g + i, 8 + 4 g + i} a half-wave g contracts in
     // one MFMA step are 16 contiguous bytes.  Tokens 2 tp and 2 tp + 1 stay neighbours: byte offset of their dword
