@@ -31,3 +31,6 @@ struct DecodeArgs {
 // Returns BGTQ_EUNSUPPORTED when the arguments do not meet its layout
 // requirements, in which case the caller takes the layout-agnostic kernel.
 int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream);
+
+// Segment-loop MFMA kernel (bgtq_decode_seg.hip): same contract, same layout requirements.
+int bgtq_launch_decode_seg(const DecodeArgs& a, hipStream_t stream);

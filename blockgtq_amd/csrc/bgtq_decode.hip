@@ -624,7 +624,7 @@ int scratch_of_current_device(void** out) {
 extern "C" {
 
 int bgtq_set_decode_path(int path) {
-    if (path < 0 || path > 2) return BGTQ_EINVAL;
+    if (path < 0 || path > 3) return BGTQ_EINVAL;
     g_decode_path = path;
     return BGTQ_OK;
 }
@@ -681,6 +681,11 @@ int bgtq_decode_attn(const bgtq_head_plan* plans,
     BGTQ_CHECK_ARG(v_row_width >= 1 && v_row_width <= BGTQ_D / 2);
     a.k_row_width = k_row_width; a.v_row_width = v_row_width;
     hipStream_t st = (hipStream_t)stream;
+    if (g_decode_path == 0 || g_decode_path == 3) {
+        int rc = bgtq_launch_decode_seg(a, st);
+        if (rc != BGTQ_EUNSUPPORTED) return rc;
+        if (g_decode_path == 3) return rc;
+    }
     if (g_decode_path != 1) {
         int rc = bgtq_launch_decode_mfma(a, st);
         if (rc != BGTQ_EUNSUPPORTED) return rc;

@@ -448,7 +448,8 @@ def test_with_buffer_manager_at_the_full_ragged_shape(oracle_lib, decode_path):
 
 
 @pytest.mark.parametrize("k_layout,v_layout,vb", [(0, 0, 3), (1, 1, 3), (1, 0, 4), (0, 1, 2), (1, 1, 4)])
-def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, vb):
+@pytest.mark.parametrize("forced", [3, 2])
+def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, vb, forced):
     """With the layout-agnostic kernel switched off, the MFMA kernel must accept bit-packed
     and mixed K records and bit-packed and nibble V records in any combination."""
     from blockgtq_amd import _capi
@@ -462,7 +463,7 @@ def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, v
     vw = vp.shape[-1]
     vp_wide = torch.full((*vp.shape[:-1], P.cache_row_bytes(vw)), 0xA5, dtype=torch.uint8, device=DEV)[..., :vw]
     vp_wide.copy_(vp)
-    assert lib.bgtq_set_decode_path(2) == 0
+    assert lib.bgtq_set_decode_path(forced) == 0
     try:
         for ns in (1, 4):
             for vrec in (vp, vp_wide):
