@@ -53,12 +53,11 @@ constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score 
 typedef float float16v __attribute__((ext_vector_type(16)));
 
 // ---- LDS layout (bytes) -----------------------------------------------------------
-// [ V pair table | K tables of the record layout in use | segment words | query rows | per wave:
+// [ V pair table | K tables of the record layout in use | query rows | per wave:
 //   K tile + K norms + V norms, V tile, P ]
 constexpr int VTAB_BYTES = BGTQ_VLUT_BYTES;
 constexpr int KTAB_BYTES = BGTQ_LUT_IMAGE_BYTES;
-constexpr int SEG_OFF = VTAB_BYTES + KTAB_BYTES;                // 8 segments x 16 bytes
-constexpr int QS_OFF = SEG_OFF + 128;
+constexpr int QS_OFF = VTAB_BYTES + KTAB_BYTES;
 // Query rows: one struct per head and one of zeros (for the lanes outside a unit's lane group), a
 // 16-byte slot per unit.  An odd number of slots per struct puts the structs a lane group reads
 // together on different banks.
@@ -148,7 +147,7 @@ template <> struct ScoreAcc<8> {
 
 // ---- unit decoders ----------------------------------------------------------------------------
 // Code paths of a segment (word 0 of its LDS parameters, bits 0..3)
-enum { PATH_B1 = 1, PATH_B2 = 2, PATH_B3 = 3, PATH_BYTE = 4, PATH_RAW = 5 };
+enum { PATH_B1 = BGTQ_PATH_B1, PATH_B2 = BGTQ_PATH_B2, PATH_B3 = BGTQ_PATH_B3, PATH_BYTE = BGTQ_PATH_BYTE, PATH_RAW = BGTQ_PATH_RAW };
 
 // bytes of one unit in the record
 template <int PATH> __host__ __device__ constexpr int unit_bytes() { return PATH <= 3 ? PATH : PATH == PATH_BYTE ? 4 : 8; }
@@ -300,57 +299,33 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const int n_seg = min(P.n_seg, BGTQ_MAX_SEGMENTS);
 
     // ---- set-up jobs: job j < (HEADS + 1) * MAX_UNITS fills one 16-byte query slot (head j / MAX_UNITS, the
-    // last struct is the zero row), the next n_seg jobs write the segment words.  The loads of a
-    // thread's first job go out here, the LDS slots are written once the streaming loads have been issued.
+    // last struct is the zero row) from the plan's unit map.  The loads of a thread's first job go out
+    // here, the LDS slots are written once the streaming loads have been issued.
     constexpr int N_QJOBS = (HEADS + 1) * MAX_UNITS;
-    const int n_jobs = N_QJOBS + n_seg;
     auto job_load = [&](int j, uint32_t& slot) -> uint4v {
         uint4v w = {0, 0, 0, 0};
-        if (j < N_QJOBS) {
-            const int jh = j / MAX_UNITS, ju = j - jh * MAX_UNITS;
-            slot = QS_OFF + jh * QSTRUCT + ju * 16;
-            // unit ju of the record: the segment it falls in, its first dim and its length
-            int first = 0, d0 = 0, len = 0;
-            for (int s = 0; s < n_seg; s++) {
-                const int nu = (P.seg_len[s] + 7) >> 3;
-                if (ju >= first && ju < first + nu) {
-                    d0 = P.seg_start[s] + 8 * (ju - first);
-                    len = min(8, P.seg_start[s] + P.seg_len[s] - d0);
-                }
-                first += nu;
-            }
-            if (jh < gqa && jh < HEADS && len > 0) {
-                const uint32_t* row = (const uint32_t*)(q_src + jh * a.q_sh + d0);        // d0 is even
+        const int jh = j / MAX_UNITS, ju = j - jh * MAX_UNITS;
+        slot = QS_OFF + jh * QSTRUCT + ju * 16;
+        const uint32_t dsc = P.sunit[kl][ju];
+        const int d0 = (int)(dsc & 0xFF), len = (int)(dsc >> 8);
+        if (jh < gqa && jh < HEADS && len > 0) {
+            const uint32_t* row = (const uint32_t*)(q_src + jh * a.q_sh + d0);        // d0 is even
 #pragma unroll
-                for (int pp = 0; pp < 4; pp++)
-                    w[pp] = row[min(pp, (D - d0) / 2 - 1)] &
-                            ((2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u));
-            }
-        } else {
-            const int s = j - N_QJOBS;
-            const int bw = P.seg_bw[s], nu = (P.seg_len[s] + 7) >> 3;
-            int path, table, off;
-            if (kl == BGTQ_K_MIXED) {
-                int n_ptab = 0;
-                for (int s2 = 0; s2 < s; s2++) n_ptab += P.seg_bw[s2] <= 4 ? 1 : 0;
-                off = P.seg_mixed_off[s];
-                path = bw <= 4 ? PATH_BYTE : PATH_RAW;
-                table = bw <= 4 ? BGTQ_LUTM_K0 + n_ptab * 1024 : BGTQ_LUTM_KRAW + (bw - 5) * 512;
-            } else {
-                off = P.seg_pack_off[s];
-                path = bw <= 3 ? bw : bw == 4 ? PATH_BYTE : PATH_RAW;
-                table = bw == 1 ? BGTQ_LUT_K1 : bw == 2 ? BGTQ_LUT_K2 : bw == 3 ? BGTQ_LUT_K3 : bw == 4 ? BGTQ_LUT_K4
-                                                                                                     : BGTQ_LUT_KRAW + (bw - 5) * 512;
-            }
-            slot = SEG_OFF + s * 16;
-            w[0] = (uint32_t)path | ((uint32_t)nu << 4) | ((uint32_t)off << 12);
-            w[1] = (uint32_t)(VTAB_BYTES + table);
+            for (int pp = 0; pp < 4; pp++)
+                w[pp] = row[min(pp, (D - d0) / 2 - 1)] &
+                        ((2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u));
         }
         return w;
     };
     uint4v job0 = {0, 0, 0, 0};
     uint32_t job0_slot = 0;
-    if (tid < n_jobs) job0 = job_load(tid, job0_slot);
+    if (tid < N_QJOBS) job0 = job_load(tid, job0_slot);
+    // segment words: lane s of every wave keeps the two words of segment s (read back with v_readlane)
+    uint32_t seg_w0 = 0, seg_w1 = 0;
+    if (lane < n_seg) {
+        seg_w0 = P.sseg[kl][lane][0];
+        seg_w1 = P.sseg[kl][lane][1];
+    }
 
     // ---- tables by DMA: V table at LDS offset 0, K tables behind it; the chunks are dealt round-robin
     // to the waves
@@ -381,8 +356,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const uint8_t* vn_base = (const uint8_t*)a.vn + at_bh(a.vn_sb, a.vn_sh, 2);
     const uint32_t kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
     const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
-    const DmaShape full_k = dma_shape((int)kph + MT * krow, voff), full_kn = dma_shape((int)knph + MT * kn_st * 2, voff);
-    const DmaShape full_vn = dma_shape((int)vnph + MT * 2, voff), full_v = dma_shape((int)vph + MT * vrow, voff);
+    const DmaShape full_k = dma_shape_uniform((int)kph + MT * krow), full_kn = dma_shape_uniform((int)knph + MT * kn_st * 2);
+    const DmaShape full_vn = dma_shape_uniform((int)vnph + MT * 2), full_v = dma_shape_uniform((int)vph + MT * vrow);
     const int step_tiles = nw * MT;
     const uint32_t first = (uint32_t)(t0 + wave * MT);          // (a (row, head) slice is below 4 GB: checked by the launcher)
     const uint8_t* k_src = kp_base - kph + first * (uint32_t)krow;
@@ -394,9 +369,9 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         const int nt = min(MT, t1 - tile);
         DmaShape sk = full_k, sn = full_kn, sv = full_vn;
         if (nt < MT) {
-            sk = dma_shape((int)kph + nt * krow, voff);
-            sn = dma_shape((int)knph + nt * kn_st * 2, voff);
-            sv = dma_shape((int)vnph + nt * 2, voff);
+            sk = dma_shape_uniform((int)kph + nt * krow);
+            sn = dma_shape_uniform((int)knph + nt * kn_st * 2);
+            sv = dma_shape_uniform((int)vnph + nt * 2);
         }
         dma_region<9>(k_src, kbuf, sk, voff);
         dma_region<2>(kn_src, kbuf + tl.kt, sn, voff);
@@ -409,7 +384,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     auto issue_v = [&](int tile) -> int {
         const int nt = min(MT, t1 - tile);
         DmaShape sv = full_v;
-        if (nt < MT) sv = dma_shape((int)vph + nt * vrow, voff);
+        if (nt < MT) sv = dma_shape_uniform((int)vph + nt * vrow);
         dma_region<5>(v_src, vbuf, sv, voff);
         v_src += v_step;
         return sv.nfull + 1;
@@ -420,9 +395,9 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     // ---- the set-up slots; the P buffers' high halves (the wait for the query rows also covers the
     // tables and the first K tile: all are needed now)
     {
-        if (tid < n_jobs) lds_put<uint4v>(job0_slot, job0);
-        if (nthr < n_jobs)                                    // (uniform) small work-groups only
-            for (int j = tid + nthr; j < n_jobs; j += nthr) {
+        if (tid < N_QJOBS) lds_put<uint4v>(job0_slot, job0);
+        if (nthr < N_QJOBS)                                   // (uniform) small work-groups only
+            for (int j = tid + nthr; j < N_QJOBS; j += nthr) {
                 uint32_t slot = 0;
                 const uint4v w = job_load(j, slot);
                 lds_put<uint4v>(slot, w);
@@ -479,9 +454,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
             uint32_t qp = qs_l;
             const uint32_t qstep = q_head >= 0 ? 16u : 0u;
             for (int s = 0; s < n_seg; s++) {
-                const uint2v sw = lds_at<uint2v>(SEG_OFF + s * 16);
                 const uint32_t n16 = lds_at<uint16_t>(knrow_l + 2 * s);
-                const uint32_t w0 = __builtin_amdgcn_readfirstlane(sw.x), tab = __builtin_amdgcn_readfirstlane(sw.y);
+                const uint32_t w0 = __builtin_amdgcn_readlane(seg_w0, s), tab = __builtin_amdgcn_readlane(seg_w1, s);
                 const int path = (int)(w0 & 15u), nu = (int)((w0 >> 4) & 255u);
                 const uint32_t xp = krow_l + (w0 >> 12);
                 const float n = bgtq_h2f((uint16_t)n16) * c2;

@@ -52,11 +52,20 @@ __device__ __forceinline__ void lds_put(uint32_t addr, T v) {
     *(__attribute__((address_space(3))) T*)(uintptr_t)addr = v;
 }
 
+// A wave-uniform pointer as a scalar register pair, also where the compiler computed it in vector registers
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
 // 16 bytes per lane from sbase + voff into LDS at lds_addr + lane * 16, for the lanes
 // set in `lanes`.  The execution mask is switched inside the block, so the copy needs
 // no divergent branch around it.
 __device__ __forceinline__ void dma16(uint32_t voff, const uint8_t* sbase, uint32_t lds_addr, uint64_t lanes) {
     uint64_t saved;
+    sbase = uniform_ptr(sbase);
+    asm volatile("" : "+s"(lanes));          // (a mask known at compile time must still arrive in a register pair)
     asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0\n"
                  : "=&s"(saved) : "v"(voff), "s"(sbase), "s"(lds_addr), "s"(lanes) : "memory", "m0");
@@ -65,6 +74,7 @@ __device__ __forceinline__ void dma16(uint32_t voff, const uint8_t* sbase, uint3
 // the instruction offset moves the global and the LDS address together.
 template <int OFF>
 __device__ __forceinline__ void dma_chunk(uint32_t voff, const uint8_t* sbase, uint32_t lds_addr) {
+    sbase = uniform_ptr(sbase);
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3\n"
                  :: "v"(voff), "s"(sbase), "s"(lds_addr), "n"(OFF) : "memory", "m0");
 }
@@ -81,6 +91,14 @@ __device__ __forceinline__ DmaShape dma_shape(int total, uint32_t voff) {
     DmaShape d;
     d.nfull = ((total + 1023) >> 10) - 1;
     d.last = __builtin_amdgcn_ballot_w64((int)voff < total - d.nfull * 1024);
+    return d;
+}
+// The same from wave-uniform values only (scalar arithmetic, no lane compare)
+__device__ __forceinline__ DmaShape dma_shape_uniform(int total) {
+    DmaShape d;
+    d.nfull = ((total + 1023) >> 10) - 1;
+    const int pieces = (total - d.nfull * 1024 + 15) >> 4;           // 1..64 lanes
+    d.last = pieces >= 64 ? ~0ull : ((1ull << pieces) - 1ull);
     return d;
 }
 // Issues the nfull + 1 loads of a range of at most NCH chunks.

@@ -39,6 +39,7 @@ PLAN_DTYPE = np.dtype([
     ('n_units', '<i4', (2,)), ('n_pair_units', '<i4', (2,)),
     ('kend', '<u4', (2,)), ('kfirst', '<u4', (2, 2)), ('reserved1', '<u4', (2,)),
     ('kprog', '<u4', (2, MAX_UNITS, 8)), ('kunit', '<u4', (2, MAX_UNITS)),
+    ('sseg', '<u4', (2, MAX_SEGMENTS, 4)), ('sunit', '<u4', (2, MAX_UNITS)),
     ('lut_image', '<u4', (2, 13824 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
 ], align=True)
 
@@ -90,6 +91,35 @@ def _raw_table(cb16: np.ndarray, bw: int) -> np.ndarray:
     return raw.view(np.uint32)
 
 
+
+
+PATH_B1, PATH_B2, PATH_B3, PATH_BYTE, PATH_RAW = 1, 2, 3, 4, 5
+
+
+def fill_segment_walk(p) -> None:
+    """The K record as the decode attention kernel walks it: per layout one word pair per
+    segment (unpack path, unit count, byte offset, table address) and the unit -> dims map."""
+    p['sseg'][...] = 0
+    p['sunit'][...] = 0
+    for layout in (K_BITPACKED, K_MIXED):
+        units, n_ptab = [], 0
+        for s in range(int(p['n_seg'])):
+            bw, ln, start = int(p['seg_bw'][s]), int(p['seg_len'][s]), int(p['seg_start'][s])
+            if layout == K_BITPACKED:
+                off = int(p['seg_pack_off'][s])
+                path = bw if bw <= 3 else PATH_BYTE if bw == 4 else PATH_RAW
+                table = LUT_K[bw] if bw <= 4 else LUT_KRAW + (bw - 5) * 512
+            else:
+                off = int(p['seg_mixed_off'][s])
+                path = PATH_BYTE if bw <= 4 else PATH_RAW
+                table = n_ptab * 1024 if bw <= 4 else LUTM_KRAW + (bw - 5) * 512
+                n_ptab += bw <= 4
+            n_u = (ln + 7) // 8
+            p['sseg'][layout, s] = [path | (n_u << 4) | (off << 12), VLUT_BYTES + table, 0, 0]
+            units += [(start + 8 * u) | (min(8, ln - 8 * u) << 8) for u in range(n_u)]
+        if len(units) > MAX_UNITS:
+            raise ValueError("segment table needs more units than the plan holds")
+        p['sunit'][layout, :len(units)] = units
 
 
 def fill_decode_steps(p) -> None:
@@ -159,6 +189,7 @@ def fill_decode_steps(p) -> None:
         t = _pair_table(p['v_lut_f16'], vb)
         p['vlut_image'][V_BITPACKED, :t.size] = t
         p['vlut_image'][V_NIBBLE, :256] = _byte_pair_table(p['v_lut_f16'], vb)
+    fill_segment_walk(p)
 
 
 def build_head_plan(quantizer) -> np.ndarray:

@@ -44,6 +44,12 @@ extern "C" {
 #define BGTQ_LUTM_KRAW   4096
 #define BGTQ_LUTM_KEND   6144
 #define BGTQ_LUT_IMAGE_BYTES 13824               /* room for either K image */
+/* how a segment's units are unpacked (bgtq_head_plan.sseg) */
+#define BGTQ_PATH_B1     1   /* bit-packed 1-bit codes: a unit is 1 byte, pair table of 4 entries x 32 replicas */
+#define BGTQ_PATH_B2     2   /* bit-packed 2-bit codes: 2 bytes, 16 entries x 32 replicas */
+#define BGTQ_PATH_B3     3   /* bit-packed 3-bit codes: 3 bytes, 64 entries x 32 replicas */
+#define BGTQ_PATH_BYTE   4   /* a byte holds a code pair as nibbles: 4 bytes, 256-entry table indexed by the byte */
+#define BGTQ_PATH_RAW    5   /* one byte per code: 8 bytes, 256 single fp16 entries */
 #define BGTQ_VLUT_BYTES  8192                    /* a V pair table: 64 entries x 32 replicas at most */
 
 /* error codes (negative); positive return values are hipError_t */
@@ -144,6 +150,16 @@ typedef struct bgtq_head_plan {
     uint32_t reserved1[2];
     uint32_t kprog[2][BGTQ_MAX_UNITS][8];
     uint32_t kunit[2][BGTQ_MAX_UNITS];
+    /*
+     * The same K record as the decode attention kernel walks it, segment by segment (one per K
+     * layout): sseg[l][s] = { path | units << 4 | byte offset of the segment in the record << 12,
+     * byte offset of the segment's table in the kernel's table area (BGTQ_VLUT_BYTES + offset
+     * inside lut_image[l]), 0, 0 } with path one of BGTQ_PATH_*; all zero past the last segment.
+     * sunit[l][u] = first packed dim of unit u | number of real dims (1..8) << 8, units numbered
+     * through the segments in order with no empty units between them; 0 past the last unit.
+     */
+    uint32_t sseg[2][BGTQ_MAX_SEGMENTS][4];
+    uint32_t sunit[2][BGTQ_MAX_UNITS];
     uint32_t lut_image[2][BGTQ_LUT_IMAGE_BYTES / 4];
     uint32_t vlut_image[2][BGTQ_VLUT_BYTES / 4];
 } bgtq_head_plan;
