@@ -259,6 +259,80 @@ __device__ __forceinline__ void run_segment(float (&S)[8], float n, uint32_t xp,
     for (int e = 0; e < HEADS; e++) S[e] = fmaf(n, acc.get(e), S[e]);
 }
 
+// A segment of exactly N units as straight-line code: all codes are requested first, then all table
+// words and query rows, then the MFMAs (two LDS round trips, no loop, no unit counter).  1-bit units
+// are one byte each, so one fetch serves three of them.
+template <int PATH, int HEADS, int N>
+__device__ __forceinline__ void seg_fixed(float (&S)[8], float n, uint32_t xp, uint32_t tb, uint32_t& qp, uint32_t qstep) {
+    constexpr int UB = unit_bytes<PATH>();
+    ScoreAcc<HEADS> acc;
+    half8 a[N];
+    uint4v w[N];
+    if (PATH == PATH_RAW) {
+        uint2v r[N];
+#pragma unroll
+        for (int i = 0; i < N; i++) r[i] = lds_codes8(xp + i * UB);
+        uint32_t ad[N][8];
+#pragma unroll
+        for (int i = 0; i < N; i++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint32_t x = e < 4 ? r[i].x : r[i].y;
+                ad[i][e] = and_or((e & 3) == 0 ? x << 1 : x >> ((e & 3) * 8 - 1), 0xFFu << 1, tb);    // byte e -> bits 1..8
+            }
+        uint32_t h16[N][8];
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) h16[i][e] = lds_at<uint16_t>(ad[i][e]);
+            a[i] = lds_at<half8>(qp + i * qstep);
+        }
+#pragma unroll
+        for (int i = 0; i < N; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) w[i][e] = h16[i][2 * e] | (h16[i][2 * e + 1] << 16);
+    } else {
+        constexpr uint32_t mask = PATH == 1 ? 0x3u << 7 : PATH == 2 ? 0xFu << 7 : PATH == 3 ? 0x3Fu << 7 : 0xFFu << 2;
+        uint32_t r[N];
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            if (PATH == PATH_B1) { if (i % 3 == 0) r[i] = fetch_unit<PATH>(xp + i); }
+            else r[i] = fetch_unit<PATH>(xp + i * UB);
+        }
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            uint32_t ad[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                if (PATH == PATH_B1) ad[p] = and_or(r[i - i % 3] >> (1 + 2 * p + 8 * (i % 3)), mask, tb);
+                else if (PATH <= 3) ad[p] = and_or(r[i] >> (1 + 2 * PATH * p), mask, tb);          // index to bits 7.., replica in tb
+                else ad[p] = and_or(p == 0 ? r[i] << 2 : r[i] >> (8 * p - 2), mask, tb);            // byte p -> bits 2..9
+            }
+#pragma unroll
+            for (int p = 0; p < 4; p++) w[i][p] = lds_at<uint32_t>(ad[p]);
+            a[i] = lds_at<half8>(qp + i * qstep);
+        }
+    }
+    acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+#pragma unroll
+    for (int i = 1; i < N; i++) acc.mma(a[i], __builtin_bit_cast(half8, w[i]));
+    qp += N * qstep;
+#pragma unroll
+    for (int e = 0; e < HEADS; e++) S[e] = fmaf(n, acc.get(e), S[e]);
+}
+
+// A segment of nu units: straight-line code for the usual sizes, the loop for long segments.
+template <int PATH, int HEADS>
+__device__ __forceinline__ void segment(float (&S)[8], float n, uint32_t xp, int nu, uint32_t tb, uint32_t& qp, uint32_t qstep) {
+    switch (nu) {
+    case 1: seg_fixed<PATH, HEADS, 1>(S, n, xp, tb, qp, qstep); break;
+    case 2: seg_fixed<PATH, HEADS, 2>(S, n, xp, tb, qp, qstep); break;
+    case 3: seg_fixed<PATH, HEADS, 3>(S, n, xp, tb, qp, qstep); break;
+    case 4: if (PATH != PATH_RAW) { seg_fixed<PATH, HEADS, PATH != PATH_RAW ? 4 : 1>(S, n, xp, tb, qp, qstep); break; }
+    default: run_segment<PATH, HEADS>(S, n, xp, nu, tb, qp, qstep); break;
+    }
+}
+
 // HEADS: query heads per KV head the MFMA layout serves (4 or 8)
 // VBW: bits per V code; VST: bytes from one V record to the next (the record itself is
 // 16 * VBW bytes; a padded stride keeps the rows of a tile on different LDS banks)
@@ -460,11 +534,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                 const uint32_t xp = krow_l + (w0 >> 12);
                 const float n = bgtq_h2f((uint16_t)n16) * c2;
                 switch (path) {
-                case PATH_B1: run_segment<PATH_B1, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
-                case PATH_B2: run_segment<PATH_B2, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
-                case PATH_B3: run_segment<PATH_B3, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
-                case PATH_BYTE: run_segment<PATH_BYTE, HEADS>(S, n, xp, nu, tab, qp, qstep); break;
-                default: run_segment<PATH_RAW, HEADS>(S, n, xp, nu, tab, qp, qstep); break;
+                case PATH_B1: segment<PATH_B1, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
+                case PATH_B2: segment<PATH_B2, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
+                case PATH_B3: segment<PATH_B3, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
+                case PATH_BYTE: segment<PATH_BYTE, HEADS>(S, n, xp, nu, tab, qp, qstep); break;
+                default: segment<PATH_RAW, HEADS>(S, n, xp, nu, tab, qp, qstep); break;
                 }
             }
         }
