@@ -60,6 +60,7 @@ _SIGNATURES = {
                                         c_p, c_i64, c_i64, c_i64,
                                         c_p, c_i, c_i, c_i, c_i, c_i,
                                         c_i, c_i, c_f, c_i, c_p, c_i64, c_i64, c_p, c_p]),
+    "bgtq_last_decode_path": (c_i, []),
     "bgtq_window_attn": (c_i, [c_p, c_i64, c_i64, c_p, c_p, c_i64, c_i64, c_i64, c_p, c_i,
                                c_i, c_i, c_i, c_f, c_p, c_p, c_p]),
     "bgtq_window_swap": (c_i, [c_p, c_p, c_i64, c_i64, c_i64, c_p, c_p, c_i64, c_i64, c_p, c_i, c_i, c_i,

@@ -588,6 +588,7 @@ __global__ __launch_bounds__(D) void window_swap_kernel(
 }  // namespace
 
 static int g_decode_path = 0;
+static int g_last_path = 0;      // kernel the last attention call ran: 1 layout-agnostic, 2 unit-program MFMA, 3 segment-loop MFMA
 
 // ---- partition results of bgtq_decode_attend_static ------------------------------------------
 // The partial vectors and log-sum-exps of the entry point that allocates nothing live in
@@ -622,6 +623,8 @@ int scratch_of_current_device(void** out) {
 }  // namespace
 
 extern "C" {
+
+int bgtq_last_decode_path(void) { return g_last_path; }
 
 int bgtq_set_decode_path(int path) {
     if (path < 0 || path > 3) return BGTQ_EINVAL;
@@ -683,14 +686,15 @@ int bgtq_decode_attn(const bgtq_head_plan* plans,
     hipStream_t st = (hipStream_t)stream;
     if (g_decode_path == 0 || g_decode_path == 3) {
         int rc = bgtq_launch_decode_seg(a, st);
-        if (rc != BGTQ_EUNSUPPORTED) return rc;
+        if (rc != BGTQ_EUNSUPPORTED) { g_last_path = 3; return rc; }
         if (g_decode_path == 3) return rc;
     }
     if (g_decode_path != 1) {
         int rc = bgtq_launch_decode_mfma(a, st);
-        if (rc != BGTQ_EUNSUPPORTED) return rc;
+        if (rc != BGTQ_EUNSUPPORTED) { g_last_path = 2; return rc; }
         if (g_decode_path == 2) return rc;        // forced fast path: report why it refused
     }
+    g_last_path = 1;
     if (gqa <= 4) return launch_generic<4>(a, st);
     if (gqa <= 8) return launch_generic<8>(a, st);
     return launch_generic<16>(a, st);
@@ -799,8 +803,8 @@ int bgtq_window_swap(void* kbuf, void* vbuf, int64_t w_sb, int64_t w_sh, int64_t
 }
 
 size_t bgtq_plan_sizeof(void) { return sizeof(bgtq_head_plan); }
-int bgtq_abi_version(void) { return 3; }
-int bgtq_decode_kernel_revision(void) { return 3; }
+int bgtq_abi_version(void) { return 4; }
+int bgtq_decode_kernel_revision(void) { return 4; }
 
 const char* bgtq_strerror(int code) {
     switch (code) {

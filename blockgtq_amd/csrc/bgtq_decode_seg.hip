@@ -62,8 +62,8 @@ constexpr int QS_OFF = VTAB_BYTES + KTAB_BYTES;
 // 16-byte slot per unit.  An odd number of slots per struct puts the structs a lane group reads
 // together on different banks.
 constexpr int QSTRUCT = (MAX_UNITS + 1) * 16;
-constexpr int PROW = MT * 4 + 32;                                // bytes from one head's P row to the next: rows land 8 banks apart
-constexpr int PBUF_BYTES = 8 * PROW;                             // P of a tile: [head][token], fp16 in the low half of a dword
+constexpr int PROW = MT * 4 + 32;                                // bytes from one head pair's P row to the next: rows land 8 banks apart
+constexpr int PBUF_BYTES = 4 * PROW;                             // P of a tile: [head pair][token], a dword holds heads 2j (low half) and 2j + 1
 constexpr int MERGE_BYTES = 64 + 8 * 32 * 16;                    // what a wave leaves for the merge: m, l, 8 heads x 128 floats
 
 __host__ __device__ constexpr int waves_off(int heads) { return QS_OFF + (heads + 1) * QSTRUCT; }
@@ -311,11 +311,18 @@ __device__ __forceinline__ void seg_fixed(float (&S)[8], float n, uint32_t xp, u
 #pragma unroll
             for (int p = 0; p < 4; p++) w[i][p] = lds_at<uint32_t>(ad[p]);
             a[i] = lds_at<half8>(qp + i * qstep);
+            // the MFMA of the unit before this one goes out while this unit's table words are on their way
+            if (i == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+            if (i > 1) acc.mma(a[i - 1], __builtin_bit_cast(half8, w[i - 1]));
         }
+        if (N == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+        else acc.mma(a[N - 1], __builtin_bit_cast(half8, w[N - 1]));
     }
-    acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+    if (PATH == PATH_RAW) {
+        acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
 #pragma unroll
-    for (int i = 1; i < N; i++) acc.mma(a[i], __builtin_bit_cast(half8, w[i]));
+        for (int i = 1; i < N; i++) acc.mma(a[i], __builtin_bit_cast(half8, w[i]));
+    }
     qp += N * qstep;
 #pragma unroll
     for (int e = 0; e < HEADS; e++) S[e] = fmaf(n, acc.get(e), S[e]);
@@ -466,7 +473,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     int tile = t0 + wave * MT;
     if (tile < t1) issue_k(tile);
 
-    // ---- the set-up slots; the P buffers' high halves (the wait for the query rows also covers the
+    // ---- the set-up slots (the wait for the query rows also covers the
     // tables and the first K tile: all are needed now)
     {
         if (tid < N_QJOBS) lds_put<uint4v>(job0_slot, job0);
@@ -476,9 +483,6 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                 const uint4v w = job_load(j, slot);
                 lds_put<uint4v>(slot, w);
             }
-#pragma unroll
-        for (int i = 0; i < PBUF_BYTES; i += 1024)
-            if (i + 1024 <= PBUF_BYTES || lane * 16 < PBUF_BYTES - i) lds_put<uint4v>(pbuf + i + lane * 16, (uint4v){0, 0, 0, 0});
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's table chunks and its first K tile
     __syncthreads();
@@ -493,15 +497,19 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const uint32_t qs_l = QS_OFF + (q_head >= 0 ? q_head : HEADS) * QSTRUCT;
     // PV operands: V table replica (the table sits at LDS address 0, so field bits OR-ed in never meet the
     // base; the 256-entry tables are not replicated), raw codes, P rows
+    // V table replica (the table sits at LDS address 0, so field bits OR-ed in never meet the base; the
+    // 256-entry tables are not replicated)
     constexpr bool V_UNREP = VBW == 4;                        // also every nibble record (VBW 4 by construction)
     constexpr int VWIN = V_UNREP ? 0 : 8;                     // replicated tables: codes fetched with the byte in front of them
     const uint32_t vbank = V_UNREP ? 0u : rep;
     constexpr int vshift = V_UNREP ? 2 : 7;
     const int vc = (int)vph + li * VBW - (V_UNREP ? 0 : 1);
     const uint32_t vbase = vbuf + (uint32_t)(vc & ~3) + (uint32_t)lg * 4 * vrow, v_sh = (uint32_t)vc & 3u;
-    const uint32_t p_wr = pbuf + (uint32_t)lane * 4;                             // + head * 256
-    const uint32_t p_rd = pbuf + (uint32_t)(li & 7) * PROW + (uint32_t)lg * 16;    // + block * 64
-    const uint32_t p_shift = (li & 8) ? 16u : 0u;              // rows 8..15 carry the odd dims: P in the high half
+    const uint32_t p_wr = pbuf + (uint32_t)lane * 4;                                   // + head pair * PROW
+    const uint32_t p_rd = pbuf + (uint32_t)((li & 7) >> 1) * PROW + (uint32_t)lg * 16;   // + block * 64
+    // A row (head h = li & 7, dim parity e = li >> 3) takes its head's half of the P dword into the half of
+    // parity e and zero into the other: a byte permute per dword
+    const uint32_t p_sel = (li & 8) ? ((li & 1) ? 0x03020C0Cu : 0x01000C0Cu) : ((li & 1) ? 0x0C0C0302u : 0x0C0C0100u);
 
     float m_ref[8], l_part[8];      // per head: reference in log2 units (never below a score seen), this lane's share of the denominator
 #pragma unroll
@@ -579,10 +587,13 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         {
             const float vn = live ? bgtq_h2f((uint16_t)vraw) : 0.f;
 #pragma unroll
-            for (int hh = 0; hh < 8; hh++) {
-                const float pe = live ? __builtin_amdgcn_exp2f(d[hh]) : 0.f;
-                l_part[hh] += pe;
-                lds_put<uint16_t>(p_wr + hh * PROW, bgtq_f2h(pe * vn));
+            for (int hh = 0; hh < 8; hh += 2) {
+                const float pe0 = live ? __builtin_amdgcn_exp2f(d[hh]) : 0.f;
+                const float pe1 = live ? __builtin_amdgcn_exp2f(d[hh + 1]) : 0.f;
+                l_part[hh] += pe0;
+                l_part[hh + 1] += pe1;
+                const half2v pk = {(_Float16)(pe0 * vn), (_Float16)(pe1 * vn)};
+                lds_put<uint32_t>(p_wr + (hh >> 1) * PROW, __builtin_bit_cast(uint32_t, pk));
             }
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // the V records of this tile are in LDS, P is written
@@ -604,10 +615,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
             for (int k = 0; k < 4; k++) {
                 const uint4v pw = lds_at<uint4v>(p_rd + k * 64);
                 uint4v W[4];                                  // [pair of the unit][token]
-                uint32_t raw[4], ad[4][4];
+                uint32_t raw[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) raw[i] = __builtin_amdgcn_alignbyte(vhi[i], vlo[i], v_sh);
                 __builtin_amdgcn_sched_barrier(0);
+                uint32_t ad[4][4];
 #pragma unroll
                 for (int e = 0; e < 4; e++)
 #pragma unroll
@@ -628,7 +640,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                 }
                 uint4v Pa;
 #pragma unroll
-                for (int i = 0; i < 4; i++) Pa[i] = pw[i] << p_shift;
+                for (int i = 0; i < 4; i++) Pa[i] = __builtin_amdgcn_perm(pw[i], pw[i], p_sel);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int jb = 0; jb < 4; jb++)

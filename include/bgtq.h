@@ -283,11 +283,20 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
 
 /*
  * Kernel selection of bgtq_decode_attn (process-wide; meant for tests and
- * profiling): 0 = automatic (MFMA kernel when the layout allows it, otherwise
- * the layout-agnostic kernel), 1 = always the layout-agnostic kernel,
- * 2 = MFMA kernel only (BGTQ_EUNSUPPORTED if it cannot take the call).
+ * profiling): 0 = automatic (the segment-loop MFMA kernel when the layout allows it, then
+ * the unit-program MFMA kernel, otherwise the layout-agnostic kernel), 1 = always the
+ * layout-agnostic kernel, 2 / 3 = unit-program / segment-loop MFMA kernel only
+ * (BGTQ_EUNSUPPORTED if it cannot take the call).
  */
 int bgtq_set_decode_path(int path);
+
+/*
+ * Which kernel the last bgtq_decode_attn of this process launched: 1 layout-agnostic,
+ * 2 unit-program MFMA, 3 segment-loop MFMA (0 before the first call).  The automatic
+ * choice falls back silently; callers that depend on the fast path check here.
+ * No counterpart in the reference.
+ */
+int bgtq_last_decode_path(void);
 
 /* Bytes of fp32 scratch bgtq_decode_attn needs for (B, n_q, n_splits). */
 size_t bgtq_workspace_bytes(int B, int n_q, int n_splits);
