@@ -23,7 +23,6 @@ SOURCES = {
     "bgtq_encode.hip": ["-ffp-contract=off"],
     "bgtq_decode.hip": ["-fno-strict-aliasing"],
     # LDS tiles are written as 128-bit / 16-bit words and read back as 32-bit words
-    "bgtq_decode_mfma.hip": ["-fno-strict-aliasing"],
     "bgtq_decode_seg.hip": ["-fno-strict-aliasing"],
     "bgtq_dequant.hip": [],
     "bgtq_prefill.hip": ["-fno-strict-aliasing"],

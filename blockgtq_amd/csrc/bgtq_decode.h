@@ -27,10 +27,7 @@ struct DecodeArgs {
     int per_tiles, rem_tiles;   // MFMA kernel, equal row lengths: tiles per partition, partitions with one more
 };
 
-// Fast path: MFMA kernel for bit-packed K and V records (bgtq_decode_mfma.hip).
+// Fast path: MFMA kernel for packed K and V records (bgtq_decode_seg.hip).
 // Returns BGTQ_EUNSUPPORTED when the arguments do not meet its layout
 // requirements, in which case the caller takes the layout-agnostic kernel.
-int bgtq_launch_decode_mfma(const DecodeArgs& a, hipStream_t stream);
-
-// Segment-loop MFMA kernel (bgtq_decode_seg.hip): same contract, same layout requirements.
 int bgtq_launch_decode_seg(const DecodeArgs& a, hipStream_t stream);

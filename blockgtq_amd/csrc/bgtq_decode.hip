@@ -48,7 +48,8 @@ __global__ __launch_bounds__(GT) void decode_generic_kernel(DecodeArgs a) {
     const bgtq_head_plan& P = a.plans[h];
     const int gqa = a.gqa;
 
-    const int T = a.seq_lens ? a.seq_lens[b] : a.T;
+    // (a length beyond the capacity the caller stated reads nothing past it)
+    const int T = a.seq_lens ? min(max(a.seq_lens[b], 0), a.T) : a.T;
     const int chunk = (T + a.n_splits - 1) / a.n_splits;
     const int t0 = min(c * chunk, T);
     const int t1 = min(t0 + chunk, T);
@@ -588,7 +589,7 @@ __global__ __launch_bounds__(D) void window_swap_kernel(
 }  // namespace
 
 static int g_decode_path = 0;
-static int g_last_path = 0;      // kernel the last attention call ran: 1 layout-agnostic, 2 unit-program MFMA, 3 segment-loop MFMA
+static int g_last_path = 0;      // kernel the last attention call ran: 1 layout-agnostic, 2 MFMA
 
 // ---- partition results of bgtq_decode_attend_static ------------------------------------------
 // The partial vectors and log-sum-exps of the entry point that allocates nothing live in
@@ -627,7 +628,7 @@ extern "C" {
 int bgtq_last_decode_path(void) { return g_last_path; }
 
 int bgtq_set_decode_path(int path) {
-    if (path < 0 || path > 3) return BGTQ_EINVAL;
+    if (path < 0 || path > 2) return BGTQ_EINVAL;
     g_decode_path = path;
     return BGTQ_OK;
 }
@@ -684,13 +685,8 @@ int bgtq_decode_attn(const bgtq_head_plan* plans,
     BGTQ_CHECK_ARG(v_row_width >= 1 && v_row_width <= BGTQ_D / 2);
     a.k_row_width = k_row_width; a.v_row_width = v_row_width;
     hipStream_t st = (hipStream_t)stream;
-    if (g_decode_path == 0 || g_decode_path == 3) {
-        int rc = bgtq_launch_decode_seg(a, st);
-        if (rc != BGTQ_EUNSUPPORTED) { g_last_path = 3; return rc; }
-        if (g_decode_path == 3) return rc;
-    }
     if (g_decode_path != 1) {
-        int rc = bgtq_launch_decode_mfma(a, st);
+        int rc = bgtq_launch_decode_seg(a, st);
         if (rc != BGTQ_EUNSUPPORTED) { g_last_path = 2; return rc; }
         if (g_decode_path == 2) return rc;        // forced fast path: report why it refused
     }

@@ -471,7 +471,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         return sv.nfull + 1;
     };
     int tile = t0 + wave * MT;
-    if (tile < t1) issue_k(tile);
+    if (tile < t1) { issue_k(tile); issue_v(tile); }        // the wave's first tile: K and V travel together
+    bool v_issued = true;
 
     // ---- the set-up slots (the wait for the query rows also covers the
     // tables and the first K tile: all are needed now)
@@ -525,7 +526,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         // wave's next tile when the V tile has, so every wait is for all loads in flight.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // K records and norms of this tile are in LDS
         __builtin_amdgcn_wave_barrier();
-        issue_v(tile);                                       // (the V buffer's last readers were the products of the previous tile)
+        if (!v_issued) issue_v(tile);                        // (the V buffer's last readers were the products of the previous tile)
+        v_issued = false;
         const uint32_t vraw = lds_at<uint16_t>(vn_l);
 
         // ---- scores of this lane's token, HEADS heads, in log2 units ----------------------------------

@@ -283,16 +283,15 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
 
 /*
  * Kernel selection of bgtq_decode_attn (process-wide; meant for tests and
- * profiling): 0 = automatic (the segment-loop MFMA kernel when the layout allows it, then
- * the unit-program MFMA kernel, otherwise the layout-agnostic kernel), 1 = always the
- * layout-agnostic kernel, 2 / 3 = unit-program / segment-loop MFMA kernel only
- * (BGTQ_EUNSUPPORTED if it cannot take the call).
+ * profiling): 0 = automatic (MFMA kernel when the layout allows it, otherwise
+ * the layout-agnostic kernel), 1 = always the layout-agnostic kernel,
+ * 2 = MFMA kernel only (BGTQ_EUNSUPPORTED if it cannot take the call).
  */
 int bgtq_set_decode_path(int path);
 
 /*
  * Which kernel the last bgtq_decode_attn of this process launched: 1 layout-agnostic,
- * 2 unit-program MFMA, 3 segment-loop MFMA (0 before the first call).  The automatic
+ * 2 MFMA (0 before the first call).  The automatic
  * choice falls back silently; callers that depend on the fast path check here.
  * No counterpart in the reference.
  */
@@ -374,6 +373,9 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
  * every call on a GPU uses that GPU's array: calls that overlap on one GPU (two
  * streams, two threads) race and must be serialised by the caller.  Nothing in the
  * array has to start at zero: each call overwrites every entry it later reads.
+ * The first call on a device asks the runtime for the array's address and sets kernel
+ * attributes, which are not stream operations: make one eager call per device before
+ * capturing this entry point into a HIP graph.
  */
 int bgtq_decode_attend_static(const bgtq_head_plan* plans,
                               const void* q_rot, int64_t q_sb, int64_t q_sh,

@@ -448,8 +448,7 @@ def test_with_buffer_manager_at_the_full_ragged_shape(oracle_lib, decode_path):
 
 
 @pytest.mark.parametrize("k_layout,v_layout,vb", [(0, 0, 3), (1, 1, 3), (1, 0, 4), (0, 1, 2), (1, 1, 4)])
-@pytest.mark.parametrize("forced", [3, 2])
-def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, vb, forced):
+def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, vb):
     """With the layout-agnostic kernel switched off, the MFMA kernel must accept bit-packed
     and mixed K records and bit-packed and nibble V records in any combination."""
     from blockgtq_amd import _capi
@@ -463,7 +462,7 @@ def test_mfma_kernel_takes_every_record_layout(oracle_lib, k_layout, v_layout, v
     vw = vp.shape[-1]
     vp_wide = torch.full((*vp.shape[:-1], P.cache_row_bytes(vw)), 0xA5, dtype=torch.uint8, device=DEV)[..., :vw]
     vp_wide.copy_(vp)
-    assert lib.bgtq_set_decode_path(forced) == 0
+    assert lib.bgtq_set_decode_path(2) == 0
     try:
         for ns in (1, 4):
             for vrec in (vp, vp_wide):
@@ -799,3 +798,73 @@ def test_manager_with_baked_q_proj_equals_manager_that_rotates_queries():
                 assert torch.equal(a._k_packed[li], b._k_packed[li]) and torch.equal(a._v_packed[li], b._v_packed[li])
                 assert torch.equal(a._k_norms[li], b._k_norms[li]) and torch.equal(a._v_norms[li], b._v_norms[li])
             a.increment_seq_len(); b.increment_seq_len()
+
+
+def test_plan_with_many_units_and_every_code_width(oracle_lib):
+    """Six segments (1..5 and 8 bits) of lengths 2, 2, 2, 10, 2, 110: 20 units, most of them in the last
+    segment (a loop, where the usual segments are straight-line code), 8 query heads per KV head,
+    bit-packed and mixed records."""
+    from blockgtq_amd.quantizer import build_batched_encode_args, encode_k_into, encode_v_into
+    alloc = [1, 2, 3] + [4] * 5 + [5] + [8] * 55
+    T, gqa = 300, 8
+    for kl in (0, 1):
+        q, en = make_quantizer(seed=3, alloc=alloc, device=DEV)
+        args = build_batched_encode_args([q], device=DEV)
+        assert int(args['plans_np']['n_seg'][0]) == 6
+        own = args['max_mixed_bytes'] if kl else args['max_tpb']
+        kw = P.cache_row_bytes(own)
+        k, v, qq = make_kv(en, T, seed=77, n_q=gqa)
+        kp = torch.zeros(1, 1, T + 2, kw, dtype=torch.uint8, device=DEV)
+        kn = torch.zeros(1, 1, T + 2, args['max_n_groups'], dtype=torch.float16, device=DEV)
+        vp = torch.zeros(1, 1, T + 2, args['v_packed_bytes'], dtype=torch.uint8, device=DEV)
+        vn = torch.zeros(1, 1, T + 2, dtype=torch.float16, device=DEV)
+        encode_k_into(args['plans'], torch.tensor(k[None, None]).to(DEV), kp, kn, 0, kw, args['max_n_groups'], kl)
+        encode_v_into(args['plans'], torch.tensor(v[None, None]).to(DEV), vp, vn, 0, args['v_packed_bytes'], 0)
+        q_rot = ops.rotate_q(args['plans'], torch.tensor(qq[None]).to(DEV), 1)
+        ref, ref_lse = _reference(oracle_lib, args['plans_np'], [q], kp.cpu().numpy(), kn.cpu().numpy(),
+                                  vp.cpu().numpy(), vn.cpu().numpy(), q_rot.cpu().numpy(), [T], gqa, kl, 0, 3)
+        for ns in (1, 3):
+            out, lse = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, T, n_splits=ns, k_layout=kl,
+                                            return_lse=True)
+            assert np.abs(out.float().cpu().numpy() - ref).max() < TOL, (kl, ns)
+            assert np.abs(lse.cpu().numpy() - ref_lse).max() < LSE_TOL
+
+
+def test_a_length_beyond_the_stated_capacity_is_clamped(oracle_lib):
+    """``T`` is the capacity bound of a ragged call: a row whose device-side length exceeds it
+    attends to ``T`` records, as if its length were ``T``."""
+    args, qs, q_rot, kp, kn, vp, vn = _build(192, 1, 5, 3, 2, 4, 2, 200, seed=41)
+    good = torch.tensor([200, 57], dtype=torch.int32, device=DEV)
+    bad = torch.tensor([100000, 57], dtype=torch.int32, device=DEV)
+    o0 = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 200, seq_lens=good, n_splits=4)
+    o1 = ops.decode_attention(args['plans'], q_rot, kp, kn, vp, vn, 200, seq_lens=bad, n_splits=4)
+    assert torch.equal(o0, o1)
+
+
+def test_mfma_kernel_refuses_strides_its_addressing_cannot_hold():
+    """The fast kernel forms addresses from 32-bit factors; strides or slices of 4 GB and more are
+    refused before anything is launched (forced fast path: the refusal is reported, not papered over)."""
+    from blockgtq_amd import _capi
+    lib = _capi.lib()
+    args, qs, q_rot, kp, kn, vp, vn = _build(192, 1, 5, 3, 1, 4, 1, 70, seed=43)
+    part = torch.empty(4 * 129, dtype=torch.float32, device=DEV)
+
+    def call(kp_sb, kp_st, T):
+        return lib.bgtq_decode_attn(
+            _capi.ptr(args['plans']), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1),
+            _capi.ptr(kp), kp_sb, kp.stride(1), kp_st, kp.shape[-1],
+            _capi.ptr(kn), kn.stride(0), kn.stride(1), kn.stride(2),
+            _capi.ptr(vp), vp.stride(0), vp.stride(1), vp.stride(2), vp.shape[-1],
+            _capi.ptr(vn), vn.stride(0), vn.stride(1), vn.stride(2),
+            None, T, 1, 1, 4, 1, _capi.ptr(part), _capi.ptr(part[4 * 128:]), 0, 0, 1.0 / 128 ** 0.5,
+            _capi.stream_ptr(q_rot.device))
+
+    assert lib.bgtq_set_decode_path(2) == 0
+    try:
+        assert call(kp.stride(0), kp.stride(2), 70) == 0
+        assert lib.bgtq_last_decode_path() == 2
+        assert call(1 << 32, kp.stride(2), 70) == -2            # batch stride
+        assert call(kp.stride(0), 1 << 26, 1) == -2             # (T + 64) * token stride >= 4 GB
+    finally:
+        lib.bgtq_set_decode_path(0)
+    torch.cuda.synchronize()

@@ -84,3 +84,43 @@ def test_static_entry_refuses_sizes_beyond_its_array():
         _capi.stream_ptr(out.device))
     assert rc == -3
     assert "maximum" in lib.bgtq_strerror(rc).decode()
+
+
+def test_static_entry_replays_in_a_graph_after_one_eager_call():
+    """The first call on a device looks up the array's address and sets kernel attributes (no
+    stream operations), so it is made eagerly; after that the entry point can be captured.  Every
+    replay, with eager work between the replays, must reproduce the eager result bit for bit."""
+    lib = _capi.lib()
+    args, _, q_rot, kp, kn, vp, vn = _build(192, 1, 5, 3, 2, 8, 2, 500, seed=25)
+    B, n_kv, gqa, T, ns = 2, 2, 8, 500, 4
+    scale = 1.0 / 128 ** 0.5
+    out_e = torch.empty(B, n_kv * gqa, 128, dtype=torch.float16, device=DEV)
+    out_g = torch.zeros_like(out_e)
+
+    def call(out):
+        _capi.check(lib.bgtq_decode_attend_static(
+            _capi.ptr(args['plans']), _capi.ptr(q_rot), q_rot.stride(0), q_rot.stride(1),
+            _capi.ptr(kp), kp.stride(0), kp.stride(1), kp.stride(2), kp.shape[-1],
+            _capi.ptr(kn), kn.stride(0), kn.stride(1), kn.stride(2),
+            _capi.ptr(vp), vp.stride(0), vp.stride(1), vp.stride(2), vp.shape[-1],
+            _capi.ptr(vn), vn.stride(0), vn.stride(1), vn.stride(2),
+            None, T, B, n_kv, gqa, ns, 0, 0, scale, 1, _capi.ptr(out), out.stride(0), out.stride(1), None,
+            _capi.stream_ptr(q_rot.device)), "bgtq_decode_attend_static")
+
+    call(out_e)                                   # eager warm-up: address look-up, attributes
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(out_g)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(out_g)
+    for i in range(3):
+        out_g.zero_()
+        (q_rot.float() * (i + 1)).sum().item()    # the program's own eager work and a synchronisation
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), i
