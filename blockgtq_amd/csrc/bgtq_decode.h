@@ -16,6 +16,7 @@ struct DecodeArgs {
     const uint16_t* vn; int64_t vn_sb, vn_sh, vn_st;
     const int32_t* seq_lens; int T;
     int B, n_kv, gqa, n_splits;
+    int gqa_all, head0;    // MFMA kernel: query heads per KV head in q and the partials, first head of this launch
     float* part_out; float* part_lse;
     int k_layout, v_layout;
     float scale;

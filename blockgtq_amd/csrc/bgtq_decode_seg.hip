@@ -376,7 +376,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     auto at_bh = [&](int64_t sb, int64_t sh, int elem) -> uint64_t {
         return ((uint64_t)(uint32_t)b * (uint32_t)sb + (uint64_t)(uint32_t)h * (uint32_t)sh) * (uint32_t)elem;
     };
-    const uint16_t* q_src = (const uint16_t*)((const uint8_t*)a.q + ((uint64_t)(uint32_t)b * (uint32_t)a.q_sb + (uint64_t)(uint32_t)(h * gqa) * (uint32_t)a.q_sh) * 2u);
+    const uint16_t* q_src = (const uint16_t*)((const uint8_t*)a.q + ((uint64_t)(uint32_t)b * (uint32_t)a.q_sb + (uint64_t)(uint32_t)(h * a.gqa_all + a.head0) * (uint32_t)a.q_sh) * 2u);
     const int n_seg = min(P.n_seg, BGTQ_MAX_SEGMENTS);
 
     // ---- set-up jobs: job j < (HEADS + 1) * MAX_UNITS fills one 16-byte query slot (head j / MAX_UNITS, the
@@ -704,7 +704,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         }
         const bool any = t1 > t0;
         const float inv = any ? 1.f / den : 0.f;
-        const size_t row = ((size_t)b * a.n_kv * gqa + (size_t)h * gqa + hq) * a.n_splits + c;
+        const size_t row = ((size_t)b * a.n_kv * a.gqa_all + (size_t)h * a.gqa_all + a.head0 + hq) * a.n_splits + c;
         float* dst = a.part_out + row * D + (idx >> 1) * 8 + (idx & 1);
 #pragma unroll
         for (int jb = 0; jb < 4; jb++) dst[2 * jb] = num[jb] * inv;
@@ -759,7 +759,25 @@ int launch(const DecodeArgs& a, hipStream_t st) {
 }  // namespace
 
 
-int bgtq_launch_decode_seg(const DecodeArgs& a, hipStream_t stream) {
+static int launch_group(const DecodeArgs& a, hipStream_t stream);
+
+int bgtq_launch_decode_seg(const DecodeArgs& all, hipStream_t stream) {
+    // one launch takes up to 8 query heads per KV head; 9..16 go as two launches over halves of the
+    // heads (the records are streamed twice, which still beats the generic kernel several times over)
+    if (all.gqa > 16) return BGTQ_EUNSUPPORTED;
+    const int n_groups = all.gqa > 8 ? 2 : 1, first = (all.gqa + n_groups - 1) / n_groups;
+    for (int g = 0; g < n_groups; g++) {
+        DecodeArgs a = all;
+        a.gqa_all = all.gqa;
+        a.head0 = g * first;
+        a.gqa = g == 0 ? first : all.gqa - first;
+        const int rc = launch_group(a, stream);
+        if (rc != BGTQ_OK) return rc;            // a refusal comes from the first group, before any launch
+    }
+    return BGTQ_OK;
+}
+
+static int launch_group(const DecodeArgs& a, hipStream_t stream) {
     // layout requirements of the fast path; anything else takes the generic kernel
     if (a.gqa > 8 || !(a.scale > 0.f)) return BGTQ_EUNSUPPORTED;
     // the kernel forms its addresses from 32-bit factors: batch and head strides, and the bytes of one

@@ -508,10 +508,11 @@ extern "C" int bgtq_prefill_attn(const bgtq_head_plan* plans,
                                  int k_layout, int v_layout, float scale, int unrotate,
                                  void* out, int64_t o_sb, int64_t o_sh, int64_t o_ss, void* stream) {
     BGTQ_CHECK_ARG(plans && q_rot && k_packed && k_norms && v_packed && v_norms && out);
-    BGTQ_CHECK_ARG(B > 0 && n_kv > 0 && gqa > 0 && S > 0 && T >= 0 && q_pos_offset >= 0);
+    BGTQ_CHECK_ARG(B >= 0 && n_kv > 0 && gqa > 0 && S >= 0 && T >= 0 && q_pos_offset >= 0);
+    if (B == 0 || S == 0) return BGTQ_OK;            // no query rows: nothing to write
     BGTQ_CHECK_ARG(k_layout == BGTQ_K_BITPACKED || k_layout == BGTQ_K_MIXED);
     BGTQ_CHECK_ARG(v_layout == BGTQ_V_BITPACKED || v_layout == BGTQ_V_NIBBLE);
-    // layout requirements of this kernel; callers fall back to bgtq_dequant_kv + their own attention
+    // layout requirements of this kernel; callers copy their records into rows that meet them
     if (gqa > ROWS || !(scale > 0.f)) return BGTQ_EUNSUPPORTED;
     if ((kp_st & 3) || (kp_sb & 3) || (kp_sh & 3) || ((uintptr_t)k_packed & 3)) return BGTQ_EUNSUPPORTED;
     if ((vp_st & 3) || (vp_sb & 3) || (vp_sh & 3) || ((uintptr_t)v_packed & 3)) return BGTQ_EUNSUPPORTED;

@@ -155,8 +155,8 @@ def fused_blockgtq_prefill_attention(
     q (B, gqa, S_q, D) fp16 already permuted + rotated; cache slices as for the
     decode entry.  Query token s sees records ``t <= q_pos_offset + s`` when
     ``is_causal``.  Returns (B, gqa, S_q, D) fp16.  ``bgtq_prefill_attn`` attends
-    straight over the records; argument sets it does not take are dequantised in
-    one pass (``bgtq_dequant_kv``) and go through the library's fused attention.
+    straight over the records; record tensors whose rows it cannot walk are first
+    copied into rows it can.
     ``block_q``, ``block_t`` and ``min_seg_for_dot`` tuned the reference kernel and
     are ignored."""
     assert q.dim() == 4
@@ -180,14 +180,9 @@ def fused_blockgtq_prefill_attention(
         v_norms = v_norms[..., 0]
     kl = _plan.K_MIXED if k_nibble else _plan.K_BITPACKED
     vl = _plan.V_NIBBLE if v_nibble else _plan.V_BITPACKED
-    out = ops.prefill_attention_packed(
-        plans, q.to(torch.float16).contiguous(), k_packed, k_norms, v_codes, v_norms, T, k_layout=kl, v_layout=vl,
+    return ops.prefill_attention_records(
+        plans, q.to(torch.float16), k_packed, k_norms, v_codes, v_norms, T, k_layout=kl, v_layout=vl,
         scale=scale, is_causal=is_causal, q_pos_offset=q_pos_offset, unrotate=v_rotation is not None)
-    if out is not None:
-        return out
-    k_hat, v_hat = ops.dequant_kv(plans, k_packed, k_norms, v_codes, v_norms, T, k_layout=kl, v_layout=vl)
-    v_rot = None if v_rotation is None else v_rotation.reshape(1, q.shape[-1], q.shape[-1])
-    return ops.prefill_attention(q.to(torch.float16), k_hat, v_hat, v_rot, scale, is_causal, q_pos_offset)
 
 
 def build_segments_from_pack_meta(pack_meta, codebook_flat=None, pos_centroids=None):

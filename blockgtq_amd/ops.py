@@ -6,10 +6,10 @@ per-KV-head Python loop of the reference (blockgtq/production_cache.py:234-262)
 has no counterpart here.
 """
 import math
+import warnings
 from typing import Optional
 
 import torch
-import torch.nn.functional as F
 
 from . import _capi, plan as _plan
 
@@ -49,6 +49,15 @@ def rotate_q(plans: torch.Tensor, q: torch.Tensor, n_kv: int) -> torch.Tensor:
         _capi.ptr(out), out.stride(0), out.stride(1),
         B, n_kv, n_q // n_kv, _capi.stream_ptr(q.device)), "bgtq_rotate_q")
     return out
+
+
+GENERIC_PATH, MFMA_PATH = 1, 2      # values of bgtq_last_decode_path()
+_paths_seen: dict = {}              # cache geometry -> kernel that bgtq_decode_attn chose for it
+
+
+def last_decode_path() -> int:
+    """Which kernel this process's last ``bgtq_decode_attn`` launched: 1 generic, 2 matrix-core."""
+    return _capi.lib().bgtq_last_decode_path()
 
 
 @torch.no_grad()
@@ -105,6 +114,15 @@ def decode_attention(plans: torch.Tensor, q_rot: torch.Tensor,
         _capi.ptr(seq_lens), int(T), B, n_kv, gqa, n_splits,
         _capi.ptr(part_out), _capi.ptr(part_lse), k_layout, v_layout, scale, st),
         "bgtq_decode_attn")
+    shape_key = (n_kv, gqa, k_packed.stride(2), v_packed.stride(2), k_norms.stride(2), k_layout, v_layout)
+    if shape_key not in _paths_seen:
+        _paths_seen[shape_key] = path = L.bgtq_last_decode_path()
+        if path == GENERIC_PATH:
+            warnings.warn(f"bgtq_decode_attn runs its generic kernel (several times slower than the matrix-core "
+                          f"one) for n_kv={n_kv}, gqa={gqa}, K rows {k_packed.stride(2)} B, V rows "
+                          f"{v_packed.stride(2)} B: the fast kernel takes gqa <= 16, K rows that follow each "
+                          f"other at a multiple of 4 bytes (4..128), V rows of 16..64 bytes at most 4 bytes apart",
+                          RuntimeWarning, stacklevel=2)
     out = torch.empty((B, n_q, D), dtype=torch.float16, device=q_rot.device)
     lse = torch.empty((B, n_q), dtype=torch.float32, device=q_rot.device) if return_lse else None
     n_extra = 0
@@ -259,7 +277,7 @@ def prefill_attention_packed(plans: torch.Tensor, q_rot: torch.Tensor, k_packed:
     q_rot (B, n_q, S, D) fp16 rotated queries; cache tensors as for ``decode_attention``.
     Query token s sees records ``t <= q_pos_offset + s`` when ``is_causal``.  Returns
     (B, n_q, S, D) fp16, or ``None`` when the kernel does not take this argument set
-    (the caller then dequantises with ``dequant_kv`` and uses ``prefill_attention``)."""
+    (``prefill_attention_records`` copies records into rows the kernel can walk first)."""
     _capi.require_cuda(k_packed, "k_packed")
     assert q_rot.dtype == torch.float16 and q_rot.dim() == 4 and q_rot.stride(-1) == 1
     assert k_packed.dtype == torch.uint8 and k_packed.stride(-1) == 1
@@ -287,32 +305,41 @@ def prefill_attention_packed(plans: torch.Tensor, q_rot: torch.Tensor, k_packed:
     return out
 
 
-@torch.no_grad()
-def prefill_attention(q_rot: torch.Tensor, k_hat: torch.Tensor, v_hat: torch.Tensor,
-                      v_rot: Optional[torch.Tensor] = None, scale: Optional[float] = None,
-                      is_causal: bool = True, q_pos_offset: int = 0) -> torch.Tensor:
-    """Attention of many query tokens over dequantised records.
+def _packed_rows(rec: torch.Tensor, T: int, width: int, v_rows: bool = False) -> torch.Tensor:
+    """The first ``T`` records of a (B, n_kv, >=T, >=width) uint8 cache tensor in the row layout the
+    prompt-phase kernel takes (rows that follow each other at a stride of ``width`` rounded up to 4
+    bytes; V rows of 32 or 64 bytes may sit 4 bytes apart): the tensor itself when it already has it,
+    a copy otherwise."""
+    row = (width + 3) // 4 * 4
+    ok = rec.stride(2) == row or (v_rows and rec.stride(2) == row + 4)
+    if ok and rec.stride(0) % 4 == 0 and rec.stride(1) % 4 == 0 and rec.data_ptr() % 4 == 0:
+        return rec
+    out = torch.zeros((rec.shape[0], rec.shape[1], T, row), dtype=torch.uint8, device=rec.device)
+    out[..., :width] = rec[:, :, :T, :width]
+    return out
 
-    q_rot (B, n_q, S, D) fp16 rotated queries; k_hat / v_hat (B, n_kv, T, D) from
-    ``dequant_kv``; ``v_rot`` (n_kv, D, D) fp32 un-rotation or None.  Query
-    token s sees records ``t <= q_pos_offset + s`` when ``is_causal``.  The
-    score/value GEMMs are the library's fused attention; returns (B, n_q, S, D) fp16."""
+
+@torch.no_grad()
+def prefill_attention_records(plans, q_rot, k_packed, k_norms, v_packed, v_norms, T, *, k_layout=_plan.K_BITPACKED,
+                              v_layout=_plan.V_BITPACKED, scale=None, is_causal=True, q_pos_offset=0,
+                              unrotate=True, k_row_width=None, v_row_width=None) -> torch.Tensor:
+    """``prefill_attention_packed`` for any tensor layout: records whose rows the kernel cannot walk
+    (token stride other than the row width, odd alignment) are first copied into rows it can, queries
+    are made contiguous; an argument set the kernel still refuses raises."""
+    k_row_width = k_packed.shape[-1] if k_row_width is None else k_row_width
+    v_row_width = v_packed.shape[-1] if v_row_width is None else v_row_width
     B, n_q, S, D = q_rot.shape
-    n_kv, T = k_hat.shape[1], k_hat.shape[2]
-    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
-    if is_causal and q_pos_offset == 0 and S == T:
-        out = F.scaled_dot_product_attention(q_rot, k_hat, v_hat, is_causal=True, scale=scale,
-                                             enable_gqa=True)
-    else:
-        mask = None
-        if is_causal:
-            t = torch.arange(T, device=q_rot.device)
-            mask = t[None, :] <= (q_pos_offset + torch.arange(S, device=q_rot.device))[:, None]
-        out = F.scaled_dot_product_attention(q_rot, k_hat, v_hat, attn_mask=mask, scale=scale,
-                                             enable_gqa=True)
-    if v_rot is not None:
-        gqa = n_q // n_kv
-        o = out.reshape(B, n_kv, gqa * S, D).float() @ v_rot.to(out.device, torch.float32).unsqueeze(0)
-        out = o.reshape(B, n_q, S, D).to(torch.float16)
+    if T == 0 or B == 0:
+        return torch.zeros((B, n_q, S, D), dtype=torch.float16, device=q_rot.device)
+    kp = _packed_rows(k_packed, T, k_row_width)
+    vp = _packed_rows(v_packed, T, v_row_width, v_rows=True)
+    vn = v_norms if v_norms.stride(-1) == 1 else v_norms.contiguous()
+    out = prefill_attention_packed(plans, q_rot.contiguous(), kp, k_norms.contiguous() if k_norms.stride(-1) != 1 else k_norms,
+                                   vp, vn, T, k_layout=k_layout, v_layout=v_layout, scale=scale, is_causal=is_causal,
+                                   q_pos_offset=q_pos_offset, unrotate=unrotate,
+                                   k_row_width=kp.stride(2), v_row_width=v_row_width)
+    if out is None:
+        raise RuntimeError("bgtq_prefill_attn does not take this argument set (more than 256 query heads per "
+                           "KV head, a V record that is not 16, 32, 48 or 64 bytes, or more than 8 norm columns)")
     return out
 

@@ -46,18 +46,10 @@ def packed_prefill_attention(cache, li, q, T, q_pos_offset=0):
         qg = q.reshape(B, cache.nkv, cache.gqa * S, D).float()
         q_rot = (qg @ q_mat.unsqueeze(0)).to(torch.float16).reshape(B, n_q, S, D)
     plans = cache.batched_args[li]['plans']
-    out = ops.prefill_attention_packed(
-        plans, q_rot.contiguous(), cache.k_packed[li], cache.k_norms[li], cache.v_packed[li], cache.v_norms[li], T,
+    return ops.prefill_attention_records(
+        plans, q_rot, cache.k_packed[li], cache.k_norms[li], cache.v_packed[li], cache.v_norms[li], T,
         k_layout=cache._k_layout, v_layout=cache._v_layout, scale=cache.scale, is_causal=True,
         q_pos_offset=q_pos_offset, k_row_width=cache.k_bytes_per_tok, v_row_width=cache.vpb)
-    if out is not None:
-        return out
-    # argument sets the fused kernel does not take: one dequantisation pass + the library's attention
-    k_hat, v_hat = ops.dequant_kv(
-        plans, cache.k_packed[li], cache.k_norms[li], cache.v_packed[li], cache.v_norms[li], T,
-        k_layout=cache._k_layout, v_layout=cache._v_layout,
-        k_row_width=cache.k_bytes_per_tok, v_row_width=cache.vpb)
-    return ops.prefill_attention(q_rot, k_hat, v_hat, v_rot, cache.scale, True, q_pos_offset)
 
 
 @torch.no_grad()

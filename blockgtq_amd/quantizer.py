@@ -492,6 +492,26 @@ def compress_k_mixed_batched(k_flat: torch.Tensor, args: dict, block_n: int = 32
     return _batched_k(k_flat, args, _plan.K_MIXED, args['max_mixed_bytes'])
 
 
+@torch.no_grad()
+def compress_k_nibble4_batched(k_flat: torch.Tensor, args: dict, block_n: int = 32):
+    """(n_kv, N, D) fp16 -> every code of a vector as a nibble, two per byte in
+    packed order (even position in the low nibble; codes wider than 4 bits keep
+    their low 4), (n_kv, N, D/2) uint8, and raw group norms (n_kv, N,
+    max_n_groups) fp32.  Reference: blockgtq/quantizer.py:1751-1841."""
+    _capi.require_cuda(k_flat, "k_flat")
+    n_kv, N, hd = k_flat.shape
+    ng = args['max_n_groups']
+    x = k_flat.to(torch.float16).contiguous()
+    codes = torch.empty(n_kv, N, hd, dtype=torch.uint8, device=k_flat.device)
+    norms = torch.zeros(n_kv, N, ng, dtype=torch.float32, device=k_flat.device)
+    L, st = _capi.lib(), _capi.stream_ptr(k_flat.device)
+    for h in range(n_kv):
+        _capi.check(L.bgtq_compress_k_codes(
+            _capi.ptr(args['plans'][h * _plan.PLAN_DTYPE.itemsize:]), _capi.ptr(x[h]), N, _capi.ptr(codes[h]), _capi.ptr(norms[h]),
+            ng, 0, _plan.QUANT_LUT256, st), "bgtq_compress_k_codes")
+    return ((codes[..., 0::2] & 0xF) | ((codes[..., 1::2] & 0xF) << 4)).contiguous(), norms
+
+
 def _batched_v(v_flat, args, layout, width):
     n_kv, N, hd = v_flat.shape
     packed = torch.empty(1, n_kv, N, width, dtype=torch.uint8, device=v_flat.device)

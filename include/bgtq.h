@@ -464,9 +464,15 @@ int bgtq_dequant_kv(const bgtq_head_plan* plans,
  *              (bgtq_rotate_q semantics), strides q_sb/q_sh/q_ss in halves, rows 16-byte aligned
  *   cache      as for bgtq_decode_attn (same strides, layouts and row widths)
  *   out        fp16 [B][n_kv*gqa][S][128], strides o_sb/o_sh/o_ss in halves
- * Returns BGTQ_EUNSUPPORTED for argument sets outside the kernel's layout requirements
- * (those of bgtq_decode_attn's fast path, any gqa <= 256); callers then use
- * bgtq_dequant_kv and an attention of their own.
+ * B == 0 or S == 0 returns BGTQ_OK with nothing written.  Returns BGTQ_EUNSUPPORTED,
+ * with nothing launched, unless all of these hold: gqa <= 256, scale > 0, T > 0;
+ * K rows follow each other (kp_st == k_row_width, 4..128, a multiple of 4; kp_sb, kp_sh
+ * and the base multiples of 4); kn_st in 1..8; v_row_width one of 16, 32, 48, 64 (64 for
+ * the nibble layout) with v_row_width <= vp_st <= v_row_width + 4 and vp_* and the base
+ * multiples of 4; vn_st == 1; query strides multiples of 8 halves and a 16-byte base;
+ * output strides multiples of 4 halves and an 8-byte base.  A caller whose cache does
+ * not meet them copies the records into rows that do (a cache filled by bgtq_encode_append
+ * into tensors allocated at bgtq_cache_row_bytes already does).
  */
 int bgtq_prefill_attn(const bgtq_head_plan* plans,
                       const void* q_rot, int64_t q_sb, int64_t q_sh, int64_t q_ss,

@@ -85,13 +85,14 @@ CASES = [  # budget mn mx vb n_kv gqa B T k_layout v_layout
     (64, 1, 1, 1, 1, 1, 3, 64, 0, 1),
     (192, 3, 3, 3, 3, 2, 1, 513, 0, 0),
     (192, 1, 5, 3, 2, 7, 1, 400, 0, 0),       # odd head groups on either side of the 8-head schedule
-    (192, 1, 5, 3, 1, 12, 2, 333, 0, 0),
+    (192, 1, 5, 3, 1, 12, 2, 333, 0, 0),      # 9..16 heads: two launches of the matrix-core kernel
+    (192, 1, 5, 3, 2, 9, 1, 333, 1, 0),
     (160, 1, 6, 4, 2, 3, 2, 200, 1, 1),
 ]
 
 
 @pytest.mark.parametrize("case", CASES)
-def test_decode_matches_checker(oracle_lib, case):
+def test_decode_matches_checker(oracle_lib, case, decode_path):
     budget, mn, mx, vb, n_kv, gqa, B, T, kl, vl = case
     args, qs, q_rot, kp, kn, vp, vn = _build(budget, mn, mx, vb, n_kv, gqa, B, T, seed=budget + T, k_layout=kl, v_layout=vl)
     ref, ref_lse = _reference(oracle_lib, args['plans_np'], qs, kp.cpu().numpy(), kn.cpu().numpy(),
@@ -102,6 +103,7 @@ def test_decode_matches_checker(oracle_lib, case):
         torch.cuda.synchronize()
         assert np.abs(out.float().cpu().numpy() - ref).max() < TOL
         assert np.abs(lse.cpu().numpy() - ref_lse).max() < LSE_TOL
+        assert ops.last_decode_path() == (ops.MFMA_PATH if decode_path == "auto" else ops.GENERIC_PATH)
 
 
 def test_tiny_contexts_and_empty_partitions(oracle_lib):
@@ -639,14 +641,35 @@ def test_prompt_kernel_all_heads_in_one_launch(oracle_lib, decode_path, gqa, n_k
 
 
 def test_prompt_kernel_refuses_layouts_it_cannot_take():
-    """Strided K records or misaligned query rows come back as 'unsupported' (None here), so that callers
-    can take the dequantise-then-attend route; nothing is launched."""
+    """Strided K records come back as 'unsupported' from the entry point (None here) with nothing
+    launched; the host wrapper copies such records into rows the kernel walks and gives the very
+    result of the conforming call, so no other attention stands behind the kernel.  An empty batch
+    is no error."""
+    from blockgtq_amd import _capi
     args, qs, q_rot1, kp, kn, vp, vn = _build(192, 1, 5, 3, 1, 4, 1, 100, seed=5)
-    q = torch.zeros(1, 4, 8, 128, dtype=torch.float16, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(6)
+    q = torch.randn(1, 4, 8, 128, generator=g, device=DEV).half()
     wide = torch.zeros(1, 1, 102, kp.shape[-1] + 4, dtype=torch.uint8, device=DEV)
     wide[..., :kp.shape[-1]] = kp
-    assert ops.prefill_attention_packed(args['plans'], q, wide[..., :kp.shape[-1]], kn, vp, vn, 100) is None
-    assert ops.prefill_attention_packed(args['plans'], q, kp, kn, vp, vn, 100) is not None
+    strided = wide[..., :kp.shape[-1]]
+    assert ops.prefill_attention_packed(args['plans'], q, strided, kn, vp, vn, 100) is None
+    want = ops.prefill_attention_packed(args['plans'], q, kp, kn, vp, vn, 100, q_pos_offset=92)
+    assert want is not None
+    got = ops.prefill_attention_records(args['plans'], q, strided, kn, vp, vn, 100, q_pos_offset=92)
+    assert torch.equal(got, want)
+    odd_q = torch.zeros(1, 4, 8, 132, dtype=torch.float16, device=DEV)[..., 2:130]
+    odd_q.copy_(q)
+    assert torch.equal(ops.prefill_attention_records(args['plans'], odd_q, kp, kn, vp, vn, 100, q_pos_offset=92), want)
+    assert ops.prefill_attention_records(args['plans'], q[:0], kp[:0], kn[:0], vp[:0], vn[:0], 100).shape == (0, 4, 8, 128)
+    code = _capi.lib().bgtq_prefill_attn(
+        _capi.ptr(args['plans']), _capi.ptr(q), q.stride(0), q.stride(1), q.stride(2),
+        _capi.ptr(kp), kp.stride(0), kp.stride(1), kp.stride(2), kp.shape[-1],
+        _capi.ptr(kn), kn.stride(0), kn.stride(1), kn.stride(2),
+        _capi.ptr(vp), vp.stride(0), vp.stride(1), vp.stride(2), vp.shape[-1],
+        _capi.ptr(vn), vn.stride(0), vn.stride(1), vn.stride(2),
+        0, 1, 4, 8, 100, 92, 1, 0, 0, 0.088, 1,
+        _capi.ptr(want), want.stride(0), want.stride(1), want.stride(2), _capi.stream_ptr(torch.device(DEV)))
+    assert code == 0
 
 
 def test_merge_entry_point_refuses_what_its_kernel_cannot_take():
@@ -868,3 +891,51 @@ def test_mfma_kernel_refuses_strides_its_addressing_cannot_hold():
     finally:
         lib.bgtq_set_decode_path(0)
     torch.cuda.synchronize()
+
+
+def test_prompt_kernel_at_the_end_to_end_layer_shape(oracle_lib, decode_path):
+    """``bgtq_prefill_attn`` at the layer shape of the end-to-end workload (4 rows, 16 query / 2 KV heads,
+    8192-token prompt, K3V3): sampled query rows (first, last, work-group and tile edges, random ones)
+    against fp64 attention over the checker's dequantised records, then a chunk of 512 queries at
+    position 7680 of the same cache."""
+    if decode_path == "generic":
+        pytest.skip("one kernel serves this entry point")
+    B, n_kv, gqa, T = 4, 2, 8, 8192
+    args, qs, _, kp, kn, vp, vn = _build(192, 1, 8, 3, n_kv, gqa, B, T, seed=501)
+    gen = torch.Generator().manual_seed(502)
+    q = (torch.randn(B, n_kv * gqa, T, 128, generator=gen) * 0.6).half().to(DEV)
+
+    def rot(x):                                        # (B, n_q, S, D) -> rotated, one launch
+        Bq, nq, S, D = x.shape
+        flat = x.permute(0, 2, 1, 3).reshape(Bq * S, nq, D).contiguous()
+        return ops.rotate_q(args['plans'], flat, n_kv).reshape(Bq, S, nq, D).permute(0, 2, 1, 3).contiguous()
+
+    q_rot = rot(q)
+    out = ops.prefill_attention_packed(args['plans'], q_rot, kp, kn, vp, vn, T, is_causal=True)
+    assert out is not None and out.shape == (B, n_kv * gqa, T, 128)
+    chunk = ops.prefill_attention_packed(args['plans'], q_rot[:, :, 7680:].contiguous(), kp, kn, vp, vn, T,
+                                         is_causal=True, q_pos_offset=7680)
+    assert chunk is not None and chunk.shape == (B, n_kv * gqa, 512, 128)
+    rng = np.random.default_rng(503)
+    edges = [0, 1, 31, 32, 63, 64, 65, 127, 128, 255, 256, 257, 511, 512, 1023, 1024, 4095, 4096, 4097,
+             7679, 7680, 7681, 8127, 8128, 8190, 8191]
+    got, got_c, qr = out.float().cpu().numpy(), chunk.float().cpu().numpy(), q_rot.cpu().numpy()
+    for b in range(B):
+        for h in range(n_kv):
+            pl = args['plans_np'][h:h + 1]
+            ng = int(pl[0]['n_seg'])
+            k_hat = oracle_lib.dequant_k(pl, oracle_lib.unpack_k(pl, kp[b, h, :T].cpu().numpy(), 0),
+                                         kn[b, h, :T, :max(ng, 1)].cpu().numpy()).astype(np.float64)
+            v_hat = oracle_lib.dequant_v(pl, oracle_lib.unpack_v(vp[b, h, :T].cpu().numpy(), 3, False),
+                                         vn[b, h, :T].cpu().numpy()).astype(np.float64)
+            R = pl[0]['v_rot'].reshape(128, 128).astype(np.float64)
+            rows = sorted(set(edges) | set(int(x) for x in rng.integers(0, T, 38)))
+            for sidx in rows:
+                qv = qr[b, h * gqa:(h + 1) * gqa, sidx].astype(np.float64)          # (gqa, 128)
+                lg = qv @ k_hat[:sidx + 1].T * 128 ** -0.5
+                pr = np.exp(lg - lg.max(-1, keepdims=True))
+                pr /= pr.sum(-1, keepdims=True)
+                ref = (pr @ v_hat[:sidx + 1]) @ R
+                assert np.abs(got[b, h * gqa:(h + 1) * gqa, sidx] - ref).max() < TOL, (b, h, sidx)
+                if sidx >= 7680:
+                    assert np.abs(got_c[b, h * gqa:(h + 1) * gqa, sidx - 7680] - ref).max() < TOL, (b, h, sidx)

@@ -271,3 +271,27 @@ def test_appends_past_the_cache_capacity_write_nothing(oracle_lib):
                     vc, wn = oracle_lib.encode_v(pl, v[b, h].cpu().numpy())
                     assert np.array_equal(vp[b, h, t0:t0 + n_in].cpu().numpy(), oracle_lib.pack_v(vc, 3)[:n_in])
                     assert (kp[b, h, :min(t0, cap)] == 0xEE).all()
+
+
+def test_every_code_as_a_nibble_for_all_heads(oracle_lib):
+    """``compress_k_nibble4_batched``: byte j of a record holds the codes at packed positions 2j
+    (low nibble) and 2j+1 of the checker's code vector, codes wider than four bits cut to their low
+    four; the norms are the checker's raw group norms."""
+    from blockgtq_amd.quantizer import build_batched_encode_args, compress_k_nibble4_batched
+    made = [make_quantizer(seed=70 + h, head=h, device=DEV, min_bits=0, max_bits=6, budget=170) for h in range(3)]
+    qs = [m[0] for m in made]
+    args = build_batched_encode_args(qs, device=DEV)
+    N = 77
+    k = np.stack([make_kv(made[h][1], N, seed=90 + h)[0] for h in range(3)])
+    nib, norms = compress_k_nibble4_batched(torch.tensor(k).to(DEV), args)
+    assert nib.shape == (3, N, 64) and nib.dtype == torch.uint8
+    assert norms.shape == (3, N, args['max_n_groups']) and norms.dtype == torch.float32
+    nib, norms = nib.cpu().numpy(), norms.cpu().numpy()
+    wide = False
+    for h in range(3):
+        codes, raw, _ = oracle_lib.encode_k(args['plans_np'][h:h + 1], k[h])
+        wide |= bool((codes > 15).any())
+        assert np.array_equal(nib[h], (codes[:, 0::2] & 15) | ((codes[:, 1::2] & 15) << 4))
+        ng = raw.shape[1]
+        assert np.array_equal(norms[h][:, :min(ng, norms.shape[2])], raw[:, :norms.shape[2]])
+    assert wide
