@@ -36,6 +36,7 @@
 // Merge  every wave leaves its reference, denominator and sums in its own (then dead) tile
 //        buffers; after one barrier the first 32 * gqa threads fold the waves.
 #include <atomic>
+#include <type_traits>
 
 #include "bgtq_decode.h"
 #include "bgtq_lds.h"
@@ -45,7 +46,7 @@ namespace {
 constexpr int D = BGTQ_D;
 constexpr int MT = 64;             // tokens per wave tile
 constexpr int MAX_UNITS = BGTQ_MAX_UNITS;
-constexpr int MAX_WAVES = 12;
+constexpr int MAX_WAVES = 16;          // four per SIMD: the register budget of a wave is 128
 constexpr int MAX_KN = 8;          // norm columns per token row
 constexpr int LDS_LIMIT = 160 * 1024;
 constexpr float REFRESH = 4.0f;    // log2 headroom put above the largest score when the reference is refreshed
@@ -75,14 +76,15 @@ __host__ __device__ constexpr int vlut_bytes(int vbw, bool nibble) {
 __host__ __device__ inline TileLayout tile_layout(int krow, int vrow, int kn_st) {
     TileLayout t;
     t.kt = (MT * krow + 32 + 15) & ~15;
+    if (t.kt < PBUF_BYTES) t.kt = PBUF_BYTES;       // P of a tile takes the place of its K records
     t.vt = (MT * vrow + 32 + 15) & ~15;
     t.knr = (MT * kn_st * 2 + 16 + 15) & ~15;
     t.vnr = MT * 2 + 16;
     t.kbuf = t.kt + t.knr + t.vnr;
     return t;
 }
-__host__ __device__ inline int wave_lds_bytes(const TileLayout& t) {
-    const int tiles = t.kbuf + t.vt + PBUF_BYTES;
+__host__ __device__ inline int wave_lds_bytes(const TileLayout& t, bool p_over_k) {
+    const int tiles = t.kbuf + t.vt + (p_over_k ? 0 : PBUF_BYTES);
     return tiles > MERGE_BYTES ? tiles : MERGE_BYTES;
 }
 
@@ -149,36 +151,6 @@ template <> struct ScoreAcc<8> {
 // Code paths of a segment (word 0 of its LDS parameters, bits 0..3)
 enum { PATH_B1 = BGTQ_PATH_B1, PATH_B2 = BGTQ_PATH_B2, PATH_B3 = BGTQ_PATH_B3, PATH_BYTE = BGTQ_PATH_BYTE, PATH_RAW = BGTQ_PATH_RAW };
 
-// bytes of one unit in the record
-template <int PATH> __host__ __device__ constexpr int unit_bytes() { return PATH <= 3 ? PATH : PATH == PATH_BYTE ? 4 : 8; }
-
-// The unit's bytes as one register.  Bit-packed units of 1..3 bytes are fetched with the byte in
-// front of them, so that the unit sits at bits 8..31 and every field reaches its table-index
-// position (bit 7 up) with a right shift; byte-pair units are fetched as they lie.
-template <int PATH>
-__device__ __forceinline__ uint32_t fetch_unit(uint32_t xp) {
-    const uint32_t x = PATH <= 3 ? xp - 1u : xp;
-    uint32_t lo, hi;
-    lds_read2(x & ~3u, lo, hi);
-    return __builtin_amdgcn_alignbyte(hi, lo, x);
-}
-// the four pair-table words of the unit in register r
-template <int PATH>
-__device__ __forceinline__ uint4v unit_words(uint32_t r, uint32_t tb, uint32_t mask) {
-    uint32_t ad[4];
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-        if (PATH <= 3) {
-            ad[p] = and_or(r >> (1 + 2 * PATH * p), mask, tb);           // index to bits 7.., replica in tb
-        } else {
-            ad[p] = and_or(p == 0 ? r << 2 : r >> (8 * p - 2), mask, tb);  // byte p -> bits 2..9
-        }
-    }
-    uint4v w;
-#pragma unroll
-    for (int p = 0; p < 4; p++) w[p] = lds_at<uint32_t>(ad[p]);
-    return w;
-}
 // raw-byte units: one byte and one 2-byte table read per code
 __device__ __forceinline__ uint4v raw_unit_words(uint32_t xp, uint32_t tb) {
     const uint2v r = lds_codes8(xp);
@@ -193,151 +165,106 @@ __device__ __forceinline__ uint4v raw_unit_words(uint32_t xp, uint32_t tb) {
     return w;
 }
 
-// All units of one segment: nu >= 1 units of PATH starting at LDS byte address xp of this lane's record,
-// A rows from qp (advanced by qstep a unit: 16 for the lanes that hold a head's rows, 0 for the lanes
-// that read the zero row).  Units go two at a time: the table words and query rows of both are in
-// flight together, and so are the codes of the two after them.  The segment's sums, scaled by the
-// token's norm n of the segment, are added to S.
-template <int PATH, int HEADS>
-__device__ __forceinline__ void run_segment(float (&S)[8], float n, uint32_t xp, int nu, uint32_t tb, uint32_t& qp, uint32_t qstep) {
-    constexpr int UB = unit_bytes<PATH>();
+// A run of NU units of W-bit codes read through pair tables (W = 1..3 bit-packed, 4: nibbles), as
+// straight-line code.  The run starts m bytes behind the 4-byte aligned LDS address a0 of this lane's
+// record; its bytes are read as aligned dwords and brought to bit 0 by one byte funnel each, after
+// which every field position is a constant: a field reaches its table-index position (bit SH up)
+// with one shift, or one bit funnel where it straddles two dwords.  A rows come from qa + 16 * unit.
+// The run's sums, scaled by the token's norm n of the segment, are added to S.
+template <int W, int HEADS, int NU>
+__device__ __forceinline__ void step_pairs(float (&S)[8], float n, uint32_t a0, uint32_t m, uint32_t tab, uint32_t rep, uint32_t qa) {
+    constexpr int SH = W == 4 ? 2 : 7;                     // 256-entry tables are not replicated
+    constexpr uint32_t MASK = ((1u << (2 * W)) - 1u) << SH;
+    constexpr int ND = (NU * W + 3) / 4;
+    const uint32_t tb = W == 4 ? tab : (tab | rep);
+    uint32_t r[ND + 1], e[ND];
+#pragma unroll
+    for (int i = 0; i <= ND; i++) r[i] = lds_at<uint32_t>(a0 + 4 * i);      // (the last one may lie past the run: inside the tile buffer's slack)
+#pragma unroll
+    for (int i = 0; i < ND; i++) e[i] = __builtin_amdgcn_alignbyte(r[i + 1], r[i], m);
     ScoreAcc<HEADS> acc;
-    if (PATH == PATH_RAW) {
-        {
-            const uint4v w = raw_unit_words(xp, tb);
-            const half8 a = lds_at<half8>(qp);
-            acc.mma0(a, __builtin_bit_cast(half8, w));
+    half8 a[NU];
+    uint4v w[NU];
+#pragma unroll
+    for (int k = 0; k < NU; k++) {
+        uint32_t ad[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const int pos = 8 * W * k + 2 * W * p, i = pos >> 5, b = pos & 31;
+            uint32_t x;
+            if (b + 2 * W > 32) x = __builtin_amdgcn_alignbit(e[i + 1 < ND ? i + 1 : i], e[i], b - SH);
+            else if (b > SH) x = e[i] >> (b - SH);
+            else if (b < SH) x = e[i] << (SH - b);
+            else x = e[i];
+            ad[p] = and_or(x, MASK, tb);
         }
-        for (int j = 1; j < nu; j++) {
-            xp += UB;
-            qp += qstep;
-            const uint4v w = raw_unit_words(xp, tb);
-            const half8 a = lds_at<half8>(qp);
-            acc.mma(a, __builtin_bit_cast(half8, w));
+#pragma unroll
+        for (int p = 0; p < 4; p++) w[k][p] = lds_at<uint32_t>(ad[p]);
+        a[k] = lds_at<half8>(qa + 16 * k);
+        // the MFMA of the unit before this one goes out while this unit's table words are on their way
+        if (k == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+        if (k > 1) acc.mma(a[k - 1], __builtin_bit_cast(half8, w[k - 1]));
+    }
+    if (NU == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+    else acc.mma(a[NU - 1], __builtin_bit_cast(half8, w[NU - 1]));
+#pragma unroll
+    for (int e8 = 0; e8 < HEADS; e8++) S[e8] = fmaf(n, acc.get(e8), S[e8]);
+}
+
+// A run of NU units of 5-bit codes stored one per byte: two bytes that follow each other index the
+// 1024-entry pair table (entry address = byte 0 << 2 | byte 1 << 7), which sits at a fixed place of
+// the table area and is not replicated.
+template <int HEADS, int NU>
+__device__ __forceinline__ void step_raw5(float (&S)[8], float n, uint32_t a0, uint32_t m, uint32_t qa) {
+    constexpr uint32_t TAB = VTAB_BYTES + BGTQ_LUT_K5P;
+    constexpr int ND = 2 * NU;
+    uint32_t r[ND + 1], e[ND];
+#pragma unroll
+    for (int i = 0; i <= ND; i++) r[i] = lds_at<uint32_t>(a0 + 4 * i);
+#pragma unroll
+    for (int i = 0; i < ND; i++) e[i] = __builtin_amdgcn_alignbyte(r[i + 1], r[i], m);
+    ScoreAcc<HEADS> acc;
+    half8 a[NU];
+    uint4v w[NU];
+#pragma unroll
+    for (int k = 0; k < NU; k++) {
+        uint32_t ad[4];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t x = e[2 * k + i];
+            ad[2 * i] = and_or(x >> 1, 0xF80u, (x << 2) & 0x7Cu);
+            ad[2 * i + 1] = and_or(x >> 17, 0xF80u, (x >> 14) & 0x7Cu);
         }
-        qp += qstep;
-    } else {
-        constexpr uint32_t mask = PATH == 1 ? 0x3u << 7 : PATH == 2 ? 0xFu << 7 : PATH == 3 ? 0x3Fu << 7 : 0xFFu << 2;
-        uint32_t r0 = fetch_unit<PATH>(xp), r1 = fetch_unit<PATH>(xp + UB);
-        int left = nu;
-        {   // the first unit, or the first two when the count is even: what is left is a whole number of pairs
-            const uint4v w0 = unit_words<PATH>(r0, tb, mask);
-            const half8 a0 = lds_at<half8>(qp);
-            if (nu & 1) {
-                xp += UB;
-                qp += qstep;
-                r0 = r1;
-                r1 = fetch_unit<PATH>(xp + UB);
-                acc.mma0(a0, __builtin_bit_cast(half8, w0));
-                left -= 1;
-            } else {
-                const uint4v w1 = unit_words<PATH>(r1, tb, mask);
-                const half8 a1 = lds_at<half8>(qp + qstep);
-                xp += 2 * UB;
-                qp += 2 * qstep;
-                r0 = fetch_unit<PATH>(xp);
-                r1 = fetch_unit<PATH>(xp + UB);
-                acc.mma0(a0, __builtin_bit_cast(half8, w0));
-                acc.mma(a1, __builtin_bit_cast(half8, w1));
-                left -= 2;
-            }
-        }
-        for (; left > 0; left -= 2) {
-            const uint4v w0 = unit_words<PATH>(r0, tb, mask);
-            const half8 a0 = lds_at<half8>(qp);
-            const uint4v w1 = unit_words<PATH>(r1, tb, mask);
-            const half8 a1 = lds_at<half8>(qp + qstep);
-            xp += 2 * UB;
-            qp += 2 * qstep;
-            r0 = fetch_unit<PATH>(xp);              // (past the segment's last unit: inside the tile buffer's slack, unused)
-            r1 = fetch_unit<PATH>(xp + UB);
-            acc.mma(a0, __builtin_bit_cast(half8, w0));
-            acc.mma(a1, __builtin_bit_cast(half8, w1));
-        }
+#pragma unroll
+        for (int p = 0; p < 4; p++) w[k][p] = lds_at<uint32_t>(ad[p] + TAB);
+        a[k] = lds_at<half8>(qa + 16 * k);
+        if (k == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+        if (k > 1) acc.mma(a[k - 1], __builtin_bit_cast(half8, w[k - 1]));
+    }
+    if (NU == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
+    else acc.mma(a[NU - 1], __builtin_bit_cast(half8, w[NU - 1]));
+#pragma unroll
+    for (int e8 = 0; e8 < HEADS; e8++) S[e8] = fmaf(n, acc.get(e8), S[e8]);
+}
+
+// A run of nu units of one byte per code: one 2-byte table read per code.
+template <int HEADS>
+__device__ __forceinline__ void step_raw(float (&S)[8], float n, uint32_t xp, int nu, uint32_t tb, uint32_t qa) {
+    ScoreAcc<HEADS> acc;
+    {
+        const uint4v w = raw_unit_words(xp, tb);
+        const half8 a = lds_at<half8>(qa);
+        acc.mma0(a, __builtin_bit_cast(half8, w));
+    }
+    for (int j = 1; j < nu; j++) {
+        xp += 8;
+        qa += 16;
+        const uint4v w = raw_unit_words(xp, tb);
+        const half8 a = lds_at<half8>(qa);
+        acc.mma(a, __builtin_bit_cast(half8, w));
     }
 #pragma unroll
     for (int e = 0; e < HEADS; e++) S[e] = fmaf(n, acc.get(e), S[e]);
-}
-
-// A segment of exactly N units as straight-line code: all codes are requested first, then all table
-// words and query rows, then the MFMAs (two LDS round trips, no loop, no unit counter).  1-bit units
-// are one byte each, so one fetch serves three of them.
-template <int PATH, int HEADS, int N>
-__device__ __forceinline__ void seg_fixed(float (&S)[8], float n, uint32_t xp, uint32_t tb, uint32_t& qp, uint32_t qstep) {
-    constexpr int UB = unit_bytes<PATH>();
-    ScoreAcc<HEADS> acc;
-    half8 a[N];
-    uint4v w[N];
-    if (PATH == PATH_RAW) {
-        uint2v r[N];
-#pragma unroll
-        for (int i = 0; i < N; i++) r[i] = lds_codes8(xp + i * UB);
-        uint32_t ad[N][8];
-#pragma unroll
-        for (int i = 0; i < N; i++)
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint32_t x = e < 4 ? r[i].x : r[i].y;
-                ad[i][e] = and_or((e & 3) == 0 ? x << 1 : x >> ((e & 3) * 8 - 1), 0xFFu << 1, tb);    // byte e -> bits 1..8
-            }
-        uint32_t h16[N][8];
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) h16[i][e] = lds_at<uint16_t>(ad[i][e]);
-            a[i] = lds_at<half8>(qp + i * qstep);
-        }
-#pragma unroll
-        for (int i = 0; i < N; i++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) w[i][e] = h16[i][2 * e] | (h16[i][2 * e + 1] << 16);
-    } else {
-        constexpr uint32_t mask = PATH == 1 ? 0x3u << 7 : PATH == 2 ? 0xFu << 7 : PATH == 3 ? 0x3Fu << 7 : 0xFFu << 2;
-        uint32_t r[N];
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            if (PATH == PATH_B1) { if (i % 3 == 0) r[i] = fetch_unit<PATH>(xp + i); }
-            else r[i] = fetch_unit<PATH>(xp + i * UB);
-        }
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            uint32_t ad[4];
-#pragma unroll
-            for (int p = 0; p < 4; p++) {
-                if (PATH == PATH_B1) ad[p] = and_or(r[i - i % 3] >> (1 + 2 * p + 8 * (i % 3)), mask, tb);
-                else if (PATH <= 3) ad[p] = and_or(r[i] >> (1 + 2 * PATH * p), mask, tb);          // index to bits 7.., replica in tb
-                else ad[p] = and_or(p == 0 ? r[i] << 2 : r[i] >> (8 * p - 2), mask, tb);            // byte p -> bits 2..9
-            }
-#pragma unroll
-            for (int p = 0; p < 4; p++) w[i][p] = lds_at<uint32_t>(ad[p]);
-            a[i] = lds_at<half8>(qp + i * qstep);
-            // the MFMA of the unit before this one goes out while this unit's table words are on their way
-            if (i == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
-            if (i > 1) acc.mma(a[i - 1], __builtin_bit_cast(half8, w[i - 1]));
-        }
-        if (N == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
-        else acc.mma(a[N - 1], __builtin_bit_cast(half8, w[N - 1]));
-    }
-    if (PATH == PATH_RAW) {
-        acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));
-#pragma unroll
-        for (int i = 1; i < N; i++) acc.mma(a[i], __builtin_bit_cast(half8, w[i]));
-    }
-    qp += N * qstep;
-#pragma unroll
-    for (int e = 0; e < HEADS; e++) S[e] = fmaf(n, acc.get(e), S[e]);
-}
-
-// A segment of nu units: straight-line code for the usual sizes, the loop for long segments.
-template <int PATH, int HEADS>
-__device__ __forceinline__ void segment(float (&S)[8], float n, uint32_t xp, int nu, uint32_t tb, uint32_t& qp, uint32_t qstep) {
-    switch (nu) {
-    case 1: seg_fixed<PATH, HEADS, 1>(S, n, xp, tb, qp, qstep); break;
-    case 2: seg_fixed<PATH, HEADS, 2>(S, n, xp, tb, qp, qstep); break;
-    case 3: seg_fixed<PATH, HEADS, 3>(S, n, xp, tb, qp, qstep); break;
-    case 4: if (PATH != PATH_RAW) { seg_fixed<PATH, HEADS, PATH != PATH_RAW ? 4 : 1>(S, n, xp, tb, qp, qstep); break; }
-    default: run_segment<PATH, HEADS>(S, n, xp, nu, tb, qp, qstep); break;
-    }
 }
 
 // HEADS: query heads per KV head the MFMA layout serves (4 or 8)
@@ -377,35 +304,48 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         return ((uint64_t)(uint32_t)b * (uint32_t)sb + (uint64_t)(uint32_t)h * (uint32_t)sh) * (uint32_t)elem;
     };
     const uint16_t* q_src = (const uint16_t*)((const uint8_t*)a.q + ((uint64_t)(uint32_t)b * (uint32_t)a.q_sb + (uint64_t)(uint32_t)(h * a.gqa_all + a.head0) * (uint32_t)a.q_sh) * 2u);
-    const int n_seg = min(P.n_seg, BGTQ_MAX_SEGMENTS);
+    const int n_walk = min((int)P.n_walk[kl], BGTQ_MAX_WALK);
 
     // ---- set-up jobs: job j < (HEADS + 1) * MAX_UNITS fills one 16-byte query slot (head j / MAX_UNITS, the
-    // last struct is the zero row) from the plan's unit map.  The loads of a thread's first job go out
-    // here, the LDS slots are written once the streaming loads have been issued.
+    // last struct is the zero row) from the plan's unit map: a slot holds the unit's up to 8 query values,
+    // zero where the unit has no dim.  The first N_QJOBS threads take one job each; their loads are written
+    // as instructions of their own, so that the wait for them can leave the tile loads issued later in flight.
     constexpr int N_QJOBS = (HEADS + 1) * MAX_UNITS;
-    auto job_load = [&](int j, uint32_t& slot) -> uint4v {
-        uint4v w = {0, 0, 0, 0};
-        const int jh = j / MAX_UNITS, ju = j - jh * MAX_UNITS;
-        slot = QS_OFF + jh * QSTRUCT + ju * 16;
-        const uint32_t dsc = P.sunit[kl][ju];
-        const int d0 = (int)(dsc & 0xFF), len = (int)(dsc >> 8);
-        if (jh < gqa && jh < HEADS && len > 0) {
-            const uint32_t* row = (const uint32_t*)(q_src + jh * a.q_sh + d0);        // d0 is even
+    auto job_slot = [&](int j) -> uint32_t { const int jh = j / MAX_UNITS; return QS_OFF + jh * QSTRUCT + (j - jh * MAX_UNITS) * 16; };
+    auto job_mask = [&](uint4v w, int len) -> uint4v {
 #pragma unroll
-            for (int pp = 0; pp < 4; pp++)
-                w[pp] = row[min(pp, (D - d0) / 2 - 1)] &
-                        ((2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u));
-        }
+        for (int pp = 0; pp < 4; pp++) w[pp] &= (2 * pp < len ? 0xFFFFu : 0u) | (2 * pp + 1 < len ? 0xFFFF0000u : 0u);
         return w;
     };
-    uint4v job0 = {0, 0, 0, 0};
-    uint32_t job0_slot = 0;
-    if (tid < N_QJOBS) job0 = job_load(tid, job0_slot);
+    const bool job_wave = wave * 64 < N_QJOBS;               // (uniform)
+    uint32_t job_dsc = 0;
+    if (job_wave) {                                           // (every lane of the wave loads: no lane keeps an older value)
+        const uint32_t* src = &P.sunit[kl][tid % MAX_UNITS];
+        asm volatile("global_load_dword %0, %1, off" : "=v"(job_dsc) : "v"(src) : "memory");
+    }
     // segment words: lane s of every wave keeps the two words of segment s (read back with v_readlane)
-    uint32_t seg_w0 = 0, seg_w1 = 0;
-    if (lane < n_seg) {
-        seg_w0 = P.sseg[kl][lane][0];
-        seg_w1 = P.sseg[kl][lane][1];
+    uint32_t seg_w0 = 0, seg_w1 = 0, seg_w2 = 0;
+    if (lane < n_walk) {
+        seg_w0 = P.swalk[kl][lane][0];
+        seg_w1 = P.swalk[kl][lane][1];
+        seg_w2 = P.swalk[kl][lane][2];
+    }
+
+    // the query words of this thread's job: requested as soon as the unit's dims are known
+    uint4v job_w = {0, 0, 0, 0};
+    int job_len = 0;
+    if (job_wave) {
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(job_dsc) :: "memory");
+        const int jh = tid / MAX_UNITS, d0 = (int)(job_dsc & 0xFF);
+        job_len = (tid < N_QJOBS && jh < gqa && jh < HEADS) ? (int)(job_dsc >> 8) : 0;
+        {   // every lane loads (a lane without a job reads the first head's row and masks everything out)
+            const uint32_t* row = (const uint32_t*)(q_src + (job_len > 0 ? jh : 0) * a.q_sh + d0);     // d0 is even
+            const int last = (D - d0) / 2 - 1;                                        // (a unit's words past the row's end repeat its last one: masked out below)
+            const uint32_t *r1 = row + min(1, last), *r2 = row + min(2, last), *r3 = row + min(3, last);
+            asm volatile("global_load_dword %0, %4, off\n\tglobal_load_dword %1, %5, off\n\t"
+                         "global_load_dword %2, %6, off\n\tglobal_load_dword %3, %7, off"
+                         : "=&v"(job_w[0]), "=&v"(job_w[1]), "=&v"(job_w[2]), "=&v"(job_w[3]) : "v"(row), "v"(r1), "v"(r2), "v"(r3) : "memory");
+        }
     }
 
     // ---- tables by DMA: V table at LDS offset 0, K tables behind it; the chunks are dealt round-robin
@@ -414,7 +354,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     {
         const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
         const uint8_t* kimg_src = (const uint8_t*)P.lut_image[kl];
-        const int vbytes = vlut_bytes(VBW, vnib), kbytes = kimg_bytes(kl);
+        const int vbytes = vlut_bytes(VBW, vnib), kbytes = P.n_walk[2 + kl] ? BGTQ_LUT_K5PEND : kimg_bytes(kl);
         const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
         for (int cc = wave; cc < vch + kch; cc += nw) {
             const uint8_t* src;
@@ -430,7 +370,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const int wave_bytes = a.wave_bytes;
     const uint32_t kbuf = WAVES_OFF + wave * wave_bytes;                       // K records, K norms, V norms
     const uint32_t vbuf = kbuf + tl.kbuf;                                     // V records
-    const uint32_t pbuf = vbuf + tl.vt;                                       // P * v_norm of the tile
+    const bool p_over_k = a.p_over_k != 0;                                    // P * v_norm of the tile: over its K records (read by then), or behind the V tile
+    const uint32_t pbuf = p_over_k ? kbuf : vbuf + tl.vt;
     const uint8_t* kp_base = a.kp + at_bh(a.kp_sb, a.kp_sh, 1);
     const uint8_t* vp_base = a.vp + at_bh(a.vp_sb, a.vp_sh, 1);
     const uint8_t* kn_base = (const uint8_t*)a.kn + at_bh(a.kn_sb, a.kn_sh, 2);
@@ -439,53 +380,81 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
     const DmaShape full_k = dma_shape_uniform((int)kph + MT * krow), full_kn = dma_shape_uniform((int)knph + MT * kn_st * 2);
     const DmaShape full_vn = dma_shape_uniform((int)vnph + MT * 2), full_v = dma_shape_uniform((int)vph + MT * vrow);
+    auto tail_of = [&](const uint8_t* base, uint32_t lds, const DmaShape& d) -> DmaTail {
+        return DmaTail{base + d.nfull * 1024, lds + (uint32_t)d.nfull * 1024u, d.last};
+    };
+    const uint8_t *k_al = kp_base - kph, *kn_al = kn_base - knph, *vn_al = vn_base - vnph, *v_al = vp_base - vph;
+    const uint32_t knbuf = kbuf + tl.kt, vnbuf = knbuf + tl.knr;
+    const DmaTail tail_k = tail_of(k_al, kbuf, full_k), tail_kn = tail_of(kn_al, knbuf, full_kn);
+    const DmaTail tail_vn = tail_of(vn_al, vnbuf, full_vn), tail_v = tail_of(v_al, vbuf, full_v);
     const int step_tiles = nw * MT;
     const uint32_t first = (uint32_t)(t0 + wave * MT);          // (a (row, head) slice is below 4 GB: checked by the launcher)
-    const uint8_t* k_src = kp_base - kph + first * (uint32_t)krow;
-    const uint8_t* kn_src = kn_base - knph + first * (uint32_t)(kn_st * 2);
-    const uint8_t* vn_src = vn_base - vnph + first * 2u;
-    const uint8_t* v_src = vp_base - vph + first * (uint32_t)vrow;
+    // a lane's byte offset from the aligned base of each range, for the wave's current tile
+    uint32_t voff_k = voff + first * (uint32_t)krow, voff_kn = voff + first * (uint32_t)(kn_st * 2);
+    uint32_t voff_vn = voff + first * 2u, voff_v = voff + first * (uint32_t)vrow;
     const int k_step = step_tiles * krow, kn_step = step_tiles * kn_st * 2, vn_step = step_tiles * 2, v_step = step_tiles * vrow;
     auto issue_k = [&](int tile) -> int {
         const int nt = min(MT, t1 - tile);
-        DmaShape sk = full_k, sn = full_kn, sv = full_vn;
-        if (nt < MT) {
-            sk = dma_shape_uniform((int)kph + nt * krow);
-            sn = dma_shape_uniform((int)knph + nt * kn_st * 2);
-            sv = dma_shape_uniform((int)vnph + nt * 2);
+        int n_loads;
+        if (nt == MT) {
+            dma_chunks(voff_k, k_al, kbuf, full_k.nfull);
+            if (full_kn.nfull) dma_chunks(voff_kn, kn_al, knbuf, full_kn.nfull);
+            dma_tails(voff_k, tail_k, voff_kn, tail_kn, voff_vn, tail_vn);
+            n_loads = full_k.nfull + full_kn.nfull + 3;
+        } else {
+            const DmaShape sk = dma_shape_uniform((int)kph + nt * krow), sn = dma_shape_uniform((int)knph + nt * kn_st * 2);
+            const DmaShape sv = dma_shape_uniform((int)vnph + nt * 2);
+            dma_chunks(voff_k, k_al, kbuf, sk.nfull);
+            dma_chunks(voff_kn, kn_al, knbuf, sn.nfull);
+            dma_tails(voff_k, tail_of(k_al, kbuf, sk), voff_kn, tail_of(kn_al, knbuf, sn), voff_vn, tail_of(vn_al, vnbuf, sv));
+            n_loads = sk.nfull + sn.nfull + 3;
         }
-        dma_region<9>(k_src, kbuf, sk, voff);
-        dma_region<2>(kn_src, kbuf + tl.kt, sn, voff);
-        dma_region<1>(vn_src, kbuf + tl.kt + tl.knr, sv, voff);
-        k_src += k_step;
-        kn_src += kn_step;
-        vn_src += vn_step;
-        return sk.nfull + sn.nfull + sv.nfull + 3;
+        voff_k += k_step;
+        voff_kn += kn_step;
+        voff_vn += vn_step;
+        return n_loads;
     };
     auto issue_v = [&](int tile) -> int {
         const int nt = min(MT, t1 - tile);
-        DmaShape sv = full_v;
-        if (nt < MT) sv = dma_shape_uniform((int)vph + nt * vrow);
-        dma_region<5>(v_src, vbuf, sv, voff);
-        v_src += v_step;
-        return sv.nfull + 1;
+        int n_loads;
+        if (nt == MT) {
+            dma_chunks(voff_v, v_al, vbuf, full_v.nfull);
+            dma_tail(voff_v, tail_v);
+            n_loads = full_v.nfull + 1;
+        } else {
+            const DmaShape sv = dma_shape_uniform((int)vph + nt * vrow);
+            dma_chunks(voff_v, v_al, vbuf, sv.nfull);
+            dma_tail(voff_v, tail_of(v_al, vbuf, sv));
+            n_loads = sv.nfull + 1;
+        }
+        voff_v += v_step;
+        return n_loads;
     };
     int tile = t0 + wave * MT;
-    if (tile < t1) { issue_k(tile); issue_v(tile); }        // the wave's first tile: K and V travel together
-    bool v_issued = true;
+    int tile_loads = 0;
+    if (tile < t1) { tile_loads = issue_k(tile); tile_loads += issue_v(tile); }        // the wave's first tile: K and V travel together
+    bool v_issued = true, fresh = true;                    // (fresh: the wave has no sums yet)
 
-    // ---- the set-up slots (the wait for the query rows also covers the
-    // tables and the first K tile: all are needed now)
-    {
-        if (tid < N_QJOBS) lds_put<uint4v>(job0_slot, job0);
-        if (nthr < N_QJOBS)                                   // (uniform) small work-groups only
-            for (int j = tid + nthr; j < N_QJOBS; j += nthr) {
-                uint32_t slot = 0;
-                const uint4v w = job_load(j, slot);
-                lds_put<uint4v>(slot, w);
-            }
+    // ---- the set-up slots.  The wait covers this wave's table chunks and query words and leaves its
+    // first tile in flight: the tile is waited for where it is used, by this wave alone
+    wait_loads(tile_loads);
+    if (job_wave) {
+        asm volatile("" : "+v"(job_w[0]), "+v"(job_w[1]), "+v"(job_w[2]), "+v"(job_w[3]) :: "memory");
+        if (tid < N_QJOBS) lds_put<uint4v>(job_slot(tid), job_mask(job_w, job_len));
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this wave's table chunks and its first K tile
+    if (nthr < N_QJOBS)                                   // (uniform) small work-groups only: the other jobs, with plain loads
+        for (int j = tid + nthr; j < N_QJOBS; j += nthr) {
+            const int jh = j / MAX_UNITS;
+            const uint32_t dsc = P.sunit[kl][j - jh * MAX_UNITS];
+            const int d0 = (int)(dsc & 0xFF), len = (jh < gqa && jh < HEADS) ? (int)(dsc >> 8) : 0;
+            uint4v w = {0, 0, 0, 0};
+            if (len > 0) {
+                const uint32_t* row = (const uint32_t*)(q_src + jh * a.q_sh + d0);
+#pragma unroll
+                for (int pp = 0; pp < 4; pp++) w[pp] = row[min(pp, (D - d0) / 2 - 1)];
+            }
+            lds_put<uint4v>(job_slot(j), job_mask(w, len));
+        }
     __syncthreads();
 
     const float c2 = a.scale * 1.44269504088896340736f;      // scores are kept in log2 units
@@ -535,58 +504,79 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
 #pragma unroll
         for (int hh = 0; hh < 8; hh++) S[hh] = 0.f;
         {
-            uint32_t qp = qs_l;
-            const uint32_t qstep = q_head >= 0 ? 16u : 0u;
-            for (int s = 0; s < n_seg; s++) {
-                const uint32_t n16 = lds_at<uint16_t>(knrow_l + 2 * s);
+            for (int s = 0; s < n_walk; s++) {
                 const uint32_t w0 = __builtin_amdgcn_readlane(seg_w0, s), tab = __builtin_amdgcn_readlane(seg_w1, s);
-                const int path = (int)(w0 & 15u), nu = (int)((w0 >> 4) & 255u);
-                const uint32_t xp = krow_l + (w0 >> 12);
+                const uint32_t w2 = __builtin_amdgcn_readlane(seg_w2, s);
+                const uint32_t n16 = lds_at<uint16_t>(knrow_l + ((w2 >> 8) & 0xFFu));
+                const uint32_t a0 = krow_l + (w2 & 0xFFu), qa = qs_l + (w2 >> 16);
                 const float n = bgtq_h2f((uint16_t)n16) * c2;
-                switch (path) {
-                case PATH_B1: segment<PATH_B1, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
-                case PATH_B2: segment<PATH_B2, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
-                case PATH_B3: segment<PATH_B3, HEADS>(S, n, xp, nu, tab | rep, qp, qstep); break;
-                case PATH_BYTE: segment<PATH_BYTE, HEADS>(S, n, xp, nu, tab, qp, qstep); break;
-                default: segment<PATH_RAW, HEADS>(S, n, xp, nu, tab, qp, qstep); break;
+#define BGTQ_STEP(W, NU) case (W - 1) * 8 + NU - 1: step_pairs<W, HEADS, NU>(S, n, a0, w0, tab, rep, qa); break;
+#define BGTQ_STEPS(W) BGTQ_STEP(W, 1) BGTQ_STEP(W, 2) BGTQ_STEP(W, 3) BGTQ_STEP(W, 4) BGTQ_STEP(W, 5) BGTQ_STEP(W, 6) BGTQ_STEP(W, 7) BGTQ_STEP(W, 8)
+                switch (w0 >> 2) {
+                BGTQ_STEPS(1) BGTQ_STEPS(2) BGTQ_STEPS(3) BGTQ_STEPS(4)
+                case BGTQ_STEP_RAW5 + 0: step_raw5<HEADS, 1>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 1: step_raw5<HEADS, 2>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 2: step_raw5<HEADS, 3>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 3: step_raw5<HEADS, 4>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 4: step_raw5<HEADS, 5>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 5: step_raw5<HEADS, 6>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 6: step_raw5<HEADS, 7>(S, n, a0, w0, qa); break;
+                case BGTQ_STEP_RAW5 + 7: step_raw5<HEADS, 8>(S, n, a0, w0, qa); break;
+                default: step_raw<HEADS>(S, n, a0 + (w0 & 3u), (int)(w0 >> 2) - BGTQ_STEP_RAW + 1, tab, qa); break;
                 }
+#undef BGTQ_STEPS
+#undef BGTQ_STEP
             }
         }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
 
         // ---- online softmax: lane = token ----------------------------------------------------
-        const bool live = lane < nt;
-        float d[8];
+        // FULL: every lane holds a token (all tiles but a row's last); FRESH: the wave's first tile (no
+        // sums to rescale yet).  Both are wave-uniform and known before the tile: four copies of the code.
+        auto softmax = [&](auto full_c, auto fresh_c) {
+            constexpr bool FULL = decltype(full_c)::value, FRESH = decltype(fresh_c)::value;
+            const bool live = FULL || lane < nt;
+            float d[8];
 #pragma unroll
-        for (int hh = 0; hh < 8; hh++) d[hh] = S[hh] - m_ref[hh];
-        float mx = fmaxf(fmaxf(fmaxf(d[0], d[1]), fmaxf(d[2], d[3])), fmaxf(fmaxf(d[4], d[5]), fmaxf(d[6], d[7])));
-        if (__builtin_amdgcn_ballot_w64(live && mx > 0.f)) {   // wave-uniform, rare after the first tiles
-            float alpha[8], wm[8];
-#pragma unroll
-            for (int hh = 0; hh < 8; hh++) wm[hh] = live ? S[hh] : -INFINITY;
-            wave_max8(wm);
-#pragma unroll
-            for (int hh = 0; hh < 8; hh++) {
-                const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wm[hh]), 63));
-                const float m_new = top > m_ref[hh] ? top + REFRESH : m_ref[hh];
-                alpha[hh] = (m_ref[hh] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref[hh] - m_new);
-                l_part[hh] *= alpha[hh];
-                m_ref[hh] = m_new;
-                d[hh] = S[hh] - m_new;
+            for (int hh = 0; hh < 8; hh++) d[hh] = S[hh] - m_ref[hh];
+            bool refresh = FRESH;
+            if (!FRESH) {
+                const float mx = fmaxf(fmaxf(fmaxf(d[0], d[1]), fmaxf(d[2], d[3])), fmaxf(fmaxf(d[4], d[5]), fmaxf(d[6], d[7])));
+                refresh = __builtin_amdgcn_ballot_w64(live && mx > 0.f) != 0;       // wave-uniform, rare after the first tiles
             }
-            // acc rows are heads 4(lg & 1) + r
+            if (refresh) {
+                float wm[8];
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const uint32_t pick = (lg & 1) ? 0xFFFFFFFFu : 0u;     // (bitwise: keeps the factors in registers)
-                const float al = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, alpha[4 + r]) & pick) |
-                                                           (__builtin_bit_cast(uint32_t, alpha[r]) & ~pick));
+                for (int hh = 0; hh < 8; hh++) wm[hh] = live ? S[hh] : -INFINITY;
+                wave_max8(wm);
+                float alpha[8];
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[e][r] *= al;
+                for (int hh = 0; hh < 8; hh++) {
+                    const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wm[hh]), 63));
+                    if (FRESH) {
+                        m_ref[hh] = top + REFRESH;
+                    } else {
+                        const float m_new = top > m_ref[hh] ? top + REFRESH : m_ref[hh];
+                        alpha[hh] = __builtin_amdgcn_exp2f(m_ref[hh] - m_new);
+                        l_part[hh] *= alpha[hh];
+                        m_ref[hh] = m_new;
+                    }
+                    d[hh] = S[hh] - m_ref[hh];
+                }
+                if (!FRESH) {
+                    // acc rows are heads 4(lg & 1) + r
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const uint32_t pick = (lg & 1) ? 0xFFFFFFFFu : 0u;     // (bitwise: keeps the factors in registers)
+                        const float al = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, alpha[4 + r]) & pick) |
+                                                                   (__builtin_bit_cast(uint32_t, alpha[r]) & ~pick));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[e][r] *= al;
+                    }
+                }
             }
-        }
-        // P * v_norm, formed in fp32 and rounded to fp16 once, goes to LDS as [head][token]
-        {
+            // P * v_norm, formed in fp32 and rounded to fp16 once, goes to LDS as [head pair][token]
             const float vn = live ? bgtq_h2f((uint16_t)vraw) : 0.f;
 #pragma unroll
             for (int hh = 0; hh < 8; hh += 2) {
@@ -597,10 +587,13 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                 const half2v pk = {(_Float16)(pe0 * vn), (_Float16)(pe1 * vn)};
                 lds_put<uint32_t>(p_wr + (hh >> 1) * PROW, __builtin_bit_cast(uint32_t, pk));
             }
-        }
+        };
+        if (nt == MT) { if (fresh) softmax(std::true_type{}, std::true_type{}); else softmax(std::true_type{}, std::false_type{}); }
+        else          { if (fresh) softmax(std::false_type{}, std::true_type{}); else softmax(std::false_type{}, std::false_type{}); }
+        fresh = false;
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // the V records of this tile are in LDS, P is written
         __builtin_amdgcn_wave_barrier();
-        if (more) issue_k(tile + step_tiles);                // all reads of the K buffer and of the norms are done
+        if (more && !p_over_k) issue_k(tile + step_tiles);   // all reads of the K buffer and of the norms are done
 
         {
             // values.  The product runs over (token, dim parity) pairs: A row (head h, parity e')
@@ -651,8 +644,9 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        asm volatile("" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();     // V buffer and P buffer are rewritten from here on
+        if (more && p_over_k) issue_k(tile + step_tiles);
     }
 
     // ---- merge the waves -------------------------------------------------------------
@@ -713,8 +707,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
 }
 
 template <int HEADS>
-size_t seg_smem_bytes(const TileLayout& tl, int nw) {
-    return (size_t)waves_off(HEADS) + (size_t)nw * wave_lds_bytes(tl);
+size_t seg_smem_bytes(const TileLayout& tl, int nw, bool p_over_k) {
+    return (size_t)waves_off(HEADS) + (size_t)nw * wave_lds_bytes(tl, p_over_k);
 }
 
 template <int HEADS, int VBW, int VST>
@@ -724,11 +718,15 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
     const int tiles = (a.T + MT - 1) / MT;
     int nw = (tiles + a.n_splits - 1) / a.n_splits;
     nw = nw < 1 ? 1 : nw > MAX_WAVES ? MAX_WAVES : nw;
-    while (nw > 1 && seg_smem_bytes<HEADS>(a.tl, nw) > (size_t)LDS_LIMIT) nw--;
-    const size_t smem = seg_smem_bytes<HEADS>(a.tl, nw);
+    // P of a tile has a buffer of its own where that leaves room for the waves wanted, else it
+    // goes over the tile's K records and the next K tile is requested a phase later
+    const bool over = seg_smem_bytes<HEADS>(a.tl, nw, false) > (size_t)LDS_LIMIT;
+    while (nw > 1 && seg_smem_bytes<HEADS>(a.tl, nw, over) > (size_t)LDS_LIMIT) nw--;
+    const size_t smem = seg_smem_bytes<HEADS>(a.tl, nw, over);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
     a.nw = nw;
-    a.wave_bytes = wave_lds_bytes(a.tl);
+    a.p_over_k = over ? 1 : 0;
+    a.wave_bytes = wave_lds_bytes(a.tl, over);
     a.per_tiles = tiles / a.n_splits;
     a.rem_tiles = tiles - a.per_tiles * a.n_splits;
     auto kern = decode_seg_kernel<HEADS, VBW, VST>;

@@ -115,6 +115,64 @@ __device__ __forceinline__ void dma_region(const uint8_t* src_al, uint32_t lds_a
     dma16(voff, src_al + d.nfull * 1024, lds_addr + d.nfull * 1024, d.last);
 }
 
+// N (1..4) whole 1 KB chunks that follow each other, through one setting of M0: lane l copies the 16
+// bytes at sbase + voff (+ 1024 a chunk; voff = 16 l + the tile's distance from sbase) to lds + 16 l.
+template <int N>
+__device__ __forceinline__ void dma_full(uint32_t voff, const uint8_t* sbase, uint32_t lds) {
+    static_assert(N >= 1 && N <= 4, "the instruction offset reaches 4 chunks");
+    if (N == 1) asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n" :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+    if (N == 2) asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024\n"
+                             :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+    if (N == 3) asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+                             "global_load_lds_dwordx4 %0, %1 offset:2048\n" :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+    if (N == 4) asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+                             "global_load_lds_dwordx4 %0, %1 offset:2048\n\tglobal_load_lds_dwordx4 %0, %1 offset:3072\n"
+                             :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+}
+// n (0..8) whole chunks
+__device__ __forceinline__ void dma_chunks(uint32_t voff, const uint8_t* sbase, uint32_t lds, int n) {
+    sbase = uniform_ptr(sbase);
+    if (n >= 4) {
+        dma_full<4>(voff, sbase, lds);
+        if (n == 4) return;
+        voff += 4096;
+        lds += 4096;
+        n -= 4;
+    }
+    switch (n) {
+    case 1: dma_full<1>(voff, sbase, lds); break;
+    case 2: dma_full<2>(voff, sbase, lds); break;
+    case 3: dma_full<3>(voff, sbase, lds); break;
+    case 4: dma_full<4>(voff, sbase, lds); break;
+    default: break;
+    }
+}
+// One chunk each of up to three ranges, for the lanes of its mask: the execution mask is saved and
+// restored once around all of them.
+struct DmaTail { const uint8_t* src; uint32_t lds; uint64_t lanes; };
+__device__ __forceinline__ void dma_tails(uint32_t v0, const DmaTail& t0, uint32_t v1, const DmaTail& t1, uint32_t v2, const DmaTail& t2) {
+    uint64_t saved;
+    const uint8_t *s0 = uniform_ptr(t0.src), *s1 = uniform_ptr(t1.src), *s2 = uniform_ptr(t2.src);
+    uint64_t m0 = t0.lanes, m1 = t1.lanes, m2 = t2.lanes;
+    asm volatile("" : "+s"(m0), "+s"(m1), "+s"(m2));
+    asm volatile("s_mov_b64 %0, exec\n\t"
+                 "s_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %10, %1\n\t"
+                 "s_mov_b64 exec, %6\n\ts_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %11, %4\n\t"
+                 "s_mov_b64 exec, %9\n\ts_mov_b32 m0, %8\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %12, %7\n\t"
+                 "s_mov_b64 exec, %0\n"
+                 : "=&s"(saved)
+                 : "s"(s0), "s"(t0.lds), "s"(m0), "s"(s1), "s"(t1.lds), "s"(m1), "s"(s2), "s"(t2.lds), "s"(m2), "v"(v0), "v"(v1), "v"(v2)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma_tail(uint32_t v0, const DmaTail& t0) {
+    uint64_t saved;
+    const uint8_t* s0 = uniform_ptr(t0.src);
+    uint64_t m0 = t0.lanes;
+    asm volatile("" : "+s"(m0));
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %1\n\ts_mov_b64 exec, %0\n"
+                 : "=&s"(saved) : "s"(s0), "s"(t0.lds), "s"(m0), "v"(v0) : "memory", "m0");
+}
+
 // Waits until at most n of the loads issued so far are still in flight.
 __device__ __forceinline__ void wait_loads(int n) {
 #define BGTQ_WAIT_CASE(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;

@@ -13,6 +13,7 @@ MAX_SEGMENTS = 8
 MAX_CENTROIDS = 256
 LUT_BINS = 256
 MAX_UNITS = 24
+MAX_WALK = 12
 
 K_BITPACKED, K_MIXED = 0, 1
 V_BITPACKED, V_NIBBLE = 0, 1
@@ -39,13 +40,13 @@ PLAN_DTYPE = np.dtype([
     ('n_units', '<i4', (2,)), ('n_pair_units', '<i4', (2,)),
     ('kend', '<u4', (2,)), ('kfirst', '<u4', (2, 2)), ('reserved1', '<u4', (2,)),
     ('kprog', '<u4', (2, MAX_UNITS, 8)), ('kunit', '<u4', (2, MAX_UNITS)),
-    ('sseg', '<u4', (2, MAX_SEGMENTS, 4)), ('sunit', '<u4', (2, MAX_UNITS)),
-    ('lut_image', '<u4', (2, 13824 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
+    ('swalk', '<u4', (2, MAX_WALK, 4)), ('n_walk', '<u4', (4,)), ('sunit', '<u4', (2, MAX_UNITS)),
+    ('lut_image', '<u4', (2, 17920 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
 ], align=True)
 
 # byte offsets inside lut_image[K_BITPACKED] / lut_image[K_MIXED] (BGTQ_LUT_* / BGTQ_LUTM_* of include/bgtq.h)
 LUT_K = {3: 0, 2: 8192, 4: 10240, 1: 11264}    # each on a multiple of its size once VLUT_BYTES is added
-LUT_KRAW, LUT_IMAGE_BYTES = 11776, 13824
+LUT_KRAW, LUT_K5P, LUT_IMAGE_BYTES = 11776, 13824, 17920
 LUTM_KRAW = 4096
 VLUT_BYTES = 8192          # the kernel's table area starts with the V table; the K image follows it
 
@@ -94,31 +95,44 @@ def _raw_table(cb16: np.ndarray, bw: int) -> np.ndarray:
 
 
 PATH_B1, PATH_B2, PATH_B3, PATH_BYTE, PATH_RAW = 1, 2, 3, 4, 5
+STEP_RAW, STEP_RAW5 = 32, 40
 
 
 def fill_segment_walk(p) -> None:
-    """The K record as the decode attention kernel walks it: per layout one word pair per
-    segment (unpack path, unit count, byte offset, table address) and the unit -> dims map."""
-    p['sseg'][...] = 0
+    """The K record as the decode attention kernel walks it: per layout a list of steps (runs of
+    up to 8 units of one segment: kind, table address, byte offset, norm column, first unit) and
+    the unit -> dims map."""
+    p['swalk'][...] = 0
+    p['n_walk'][...] = 0
     p['sunit'][...] = 0
     for layout in (K_BITPACKED, K_MIXED):
-        units, n_ptab = [], 0
+        units, steps, n_ptab = [], [], 0
         for s in range(int(p['n_seg'])):
             bw, ln, start = int(p['seg_bw'][s]), int(p['seg_len'][s]), int(p['seg_start'][s])
             if layout == K_BITPACKED:
                 off = int(p['seg_pack_off'][s])
-                path = bw if bw <= 3 else PATH_BYTE if bw == 4 else PATH_RAW
-                table = LUT_K[bw] if bw <= 4 else LUT_KRAW + (bw - 5) * 512
+                w = bw if bw <= 4 else 0
+                table = LUT_K[bw] if bw <= 4 else LUT_K5P if bw == 5 else LUT_KRAW + (bw - 5) * 512
             else:
                 off = int(p['seg_mixed_off'][s])
-                path = PATH_BYTE if bw <= 4 else PATH_RAW
-                table = n_ptab * 1024 if bw <= 4 else LUTM_KRAW + (bw - 5) * 512
+                w = 4 if bw <= 4 else 0
+                table = n_ptab * 1024 if bw <= 4 else LUT_K5P if bw == 5 else LUTM_KRAW + (bw - 5) * 512
                 n_ptab += bw <= 4
+            if bw == 5:
+                p['n_walk'][2 + layout] = 1
             n_u = (ln + 7) // 8
-            p['sseg'][layout, s] = [path | (n_u << 4) | (off << 12), VLUT_BYTES + table, 0, 0]
+            unit_bytes = w if w else 8
+            for u0 in range(0, n_u, 8):
+                run = min(8, n_u - u0)
+                at = off + u0 * unit_bytes
+                kind = (w - 1) * 8 + run - 1 if w else (STEP_RAW5 if bw == 5 else STEP_RAW) + run - 1
+                steps.append([(at & 3) | (kind << 2), VLUT_BYTES + table,
+                              (at & ~3) | (2 * s << 8) | (16 * (len(units) + u0) << 16), 0])
             units += [(start + 8 * u) | (min(8, ln - 8 * u) << 8) for u in range(n_u)]
-        if len(units) > MAX_UNITS:
-            raise ValueError("segment table needs more units than the plan holds")
+        if len(units) > MAX_UNITS or len(steps) > MAX_WALK:
+            raise ValueError("segment table needs more units or steps than the plan holds")
+        p['swalk'][layout, :len(steps)] = steps
+        p['n_walk'][layout] = len(steps)
         p['sunit'][layout, :len(units)] = units
 
 
@@ -154,6 +168,9 @@ def fill_decode_steps(p) -> None:
             else:
                 table = (LUT_KRAW if layout == K_BITPACKED else LUTM_KRAW) + (bw - 5) * 512
                 img[table // 4:table // 4 + 128] = _raw_table(cb, bw)
+                if bw == 5:
+                    e = np.arange(1024)
+                    img[LUT_K5P // 4:LUT_K5P // 4 + 1024] = cb[e & 31].astype(np.uint32) | (cb[e >> 5].astype(np.uint32) << 16)
                 unit_bytes = 8
                 row = [0, 0, 0, 0, 0, VLUT_BYTES + table, 0]
             if bw > 4 and len(units) % 2:

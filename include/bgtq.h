@@ -29,6 +29,9 @@ extern "C" {
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
 #define BGTQ_STATIC_SCRATCH_BYTES (8u << 20)  /* partition results of bgtq_decode_attend_static */
+#define BGTQ_MAX_WALK      12    /* steps of the decode kernel's walk over one K record, see bgtq_head_plan.swalk */
+#define BGTQ_STEP_RAW      32    /* first step kind of raw-byte runs */
+#define BGTQ_STEP_RAW5     40    /* first step kind of raw-byte runs of 5-bit codes, read in pairs through the table at BGTQ_LUT_K5P */
 #define BGTQ_MAX_UNITS     24    /* 8-dim units of one K record, see bgtq_head_plan.kunit */
 /* byte offsets inside bgtq_head_plan.lut_image[BGTQ_K_BITPACKED] (= offsets in the decode kernel's table area) */
 /* (every pair table starts on a multiple of its own size in the kernel's table area, which puts the K image
@@ -43,8 +46,11 @@ extern "C" {
 #define BGTQ_LUTM_K0     0
 #define BGTQ_LUTM_KRAW   4096
 #define BGTQ_LUTM_KEND   6144
-#define BGTQ_LUT_IMAGE_BYTES 13824               /* room for either K image */
-/* how a segment's units are unpacked (bgtq_head_plan.sseg) */
+#define BGTQ_LUT_K5P     13824                   /* either image: 1024 entries (c0 | c1 << 5) for the 5-bit codebook, not
+                                                  * replicated; present when n_walk[2 + layout] is non-zero */
+#define BGTQ_LUT_K5PEND  17920
+#define BGTQ_LUT_IMAGE_BYTES 17920               /* room for either K image */
+/* how a segment's units are unpacked */
 #define BGTQ_PATH_B1     1   /* bit-packed 1-bit codes: a unit is 1 byte, pair table of 4 entries x 32 replicas */
 #define BGTQ_PATH_B2     2   /* bit-packed 2-bit codes: 2 bytes, 16 entries x 32 replicas */
 #define BGTQ_PATH_B3     3   /* bit-packed 3-bit codes: 3 bytes, 64 entries x 32 replicas */
@@ -151,14 +157,25 @@ typedef struct bgtq_head_plan {
     uint32_t kprog[2][BGTQ_MAX_UNITS][8];
     uint32_t kunit[2][BGTQ_MAX_UNITS];
     /*
-     * The same K record as the decode attention kernel walks it, segment by segment (one per K
-     * layout): sseg[l][s] = { path | units << 4 | byte offset of the segment in the record << 12,
-     * byte offset of the segment's table in the kernel's table area (BGTQ_VLUT_BYTES + offset
-     * inside lut_image[l]), 0, 0 } with path one of BGTQ_PATH_*; all zero past the last segment.
+     * The same K record as the decode attention kernel walks it, step by step (one walk per K
+     * layout).  A step is a run of 1..8 units (8 consecutive packed dims each, the last unit of a
+     * segment may hold fewer) of one segment; a segment of more than 8 units is cut into several
+     * steps that name the same norm column.  swalk[l][i] = {
+     *   (byte offset of the run in the record & 3) | step kind << 2,
+     *   byte offset of the segment's table in the kernel's table area (BGTQ_VLUT_BYTES + offset
+     *   inside lut_image[l]),
+     *   (byte offset of the run & ~3) | norm column * 2 << 8 | index of the run's first unit * 16 << 16,
+     *   0 }
+     * with step kind = (w - 1) * 8 + (units - 1) for codes read through pair tables (w = 1..3:
+     * bit-packed codes of w bits; w = 4: a byte holds a code pair as nibbles, which is every
+     * segment of up to 4 bits in BGTQ_K_MIXED), BGTQ_STEP_RAW5 + (units - 1) for 5-bit codes stored one
+     * per byte and BGTQ_STEP_RAW + (units - 1) for wider codes stored one per byte.  n_walk[l] steps;
+     * all zero past the last.
      * sunit[l][u] = first packed dim of unit u | number of real dims (1..8) << 8, units numbered
      * through the segments in order with no empty units between them; 0 past the last unit.
      */
-    uint32_t sseg[2][BGTQ_MAX_SEGMENTS][4];
+    uint32_t swalk[2][BGTQ_MAX_WALK][4];
+    uint32_t n_walk[4];                         /* [l]: steps of layout l; [2 + l]: 1 when lut_image[l] holds the 5-bit pair table */
     uint32_t sunit[2][BGTQ_MAX_UNITS];
     uint32_t lut_image[2][BGTQ_LUT_IMAGE_BYTES / 4];
     uint32_t vlut_image[2][BGTQ_VLUT_BYTES / 4];
