@@ -672,37 +672,48 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                              (float4v){acc[0][r], acc[1][r], acc[2][r], acc[3][r]});
     }
     __syncthreads();
-    for (int i = tid; i < gqa * 32; i += nthr) {
-        const int hq = i >> 5, idx = i & 31;
-        float mw[MAX_WAVES], lw[MAX_WAVES];
-        float4v ow[MAX_WAVES];
-#pragma unroll
-        for (int w = 0; w < MAX_WAVES; w++) {                 // all reads go out before the first is used
-            const uint32_t wb = WAVES_OFF + (uint32_t)(min(w, nw - 1) * wave_bytes);
-            mw[w] = lds_at<float>(wb + hq * 4);
-            lw[w] = lds_at<float>(wb + 32 + hq * 4);
-            ow[w] = lds_at<float4v>(wb + 64 + (hq * 32 + idx) * 16);
-        }
+    // The fold runs in two short steps so that every wave takes part.  Step 1, one thread per (wave, head):
+    // the head's reference over all waves, this wave's factor 2^(m_wave - m) and that factor times the
+    // wave's denominator, left in LDS where the query rows were.  Step 2, one thread per (head, output):
+    // the 16 scaled sums, the denominator, one store.
+    constexpr uint32_t F_OFF = QS_OFF, FL_OFF = QS_OFF + 8 * MAX_WAVES * 4, M_OFF = QS_OFF + 16 * MAX_WAVES * 4;
+    static_assert((HEADS + 1) * QSTRUCT >= 16 * MAX_WAVES * 4 + 32, "the fold's factors take the place of the query rows");
+    auto wave_base = [&](int w) -> uint32_t { return WAVES_OFF + (uint32_t)(min(w, nw - 1) * wave_bytes); };
+    for (int i = tid; i < 8 * MAX_WAVES; i += nthr) {
+        const int hh = i & 7, w = i >> 3;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < MAX_WAVES; w++) if (w < nw) m = fmaxf(m, mw[w]);
-        float den = 0.f;
-        float4v num = {0, 0, 0, 0};
+        for (int x = 0; x < MAX_WAVES; x++) m = fmaxf(m, lds_at<float>(wave_base(x) + hh * 4));     // (waves past the last repeat it)
+        const float mine = lds_at<float>(wave_base(w) + hh * 4), l = lds_at<float>(wave_base(w) + 32 + hh * 4);
+        const float f = (w < nw && mine != -INFINITY) ? __builtin_amdgcn_exp2f(mine - m) : 0.f;
+        lds_put<float>(F_OFF + (hh * MAX_WAVES + w) * 4, f);
+        lds_put<float>(FL_OFF + (hh * MAX_WAVES + w) * 4, f * l);
+        if (w == 0) lds_put<float>(M_OFF + hh * 4, m);
+    }
+    __syncthreads();
+    for (int i = tid; i < gqa * 128; i += nthr) {
+        const int hq = i >> 7, e = i & 127;                    // e = (li * 2 + (lg >> 1)) * 4 + jb
+        float4v f4[MAX_WAVES / 4], fl4[MAX_WAVES / 4];
 #pragma unroll
-        for (int w = 0; w < MAX_WAVES; w++) {
-            if (w < nw) {
-                const float f = (mw[w] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw[w] - m);
-                den += f * lw[w];
-                num += f * ow[w];
-            }
+        for (int x = 0; x < MAX_WAVES / 4; x++) {
+            f4[x] = lds_at<float4v>(F_OFF + (hq * MAX_WAVES + 4 * x) * 4);
+            fl4[x] = lds_at<float4v>(FL_OFF + (hq * MAX_WAVES + 4 * x) * 4);
+        }
+        float o[MAX_WAVES];
+#pragma unroll
+        for (int w = 0; w < MAX_WAVES; w++) o[w] = lds_at<float>(wave_base(w) + 64 + (hq * 128 + e) * 4);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < MAX_WAVES; w++) {                 // (a wave past the last has factor 0)
+            num = fmaf(f4[w >> 2][w & 3], o[w], num);
+            den += fl4[w >> 2][w & 3];
         }
         const bool any = t1 > t0;
         const float inv = any ? 1.f / den : 0.f;
         const size_t row = ((size_t)b * a.n_kv * a.gqa_all + (size_t)h * a.gqa_all + a.head0 + hq) * a.n_splits + c;
-        float* dst = a.part_out + row * D + (idx >> 1) * 8 + (idx & 1);
-#pragma unroll
-        for (int jb = 0; jb < 4; jb++) dst[2 * jb] = num[jb] * inv;
-        if (idx == 0) a.part_lse[row] = any ? (m + log2f(den)) * 0.69314718055994530942f : -INFINITY;
+        const int x = e >> 2;
+        a.part_out[row * D + (x >> 1) * 8 + (e & 3) * 2 + (x & 1)] = num * inv;
+        if (e == 0) a.part_lse[row] = any ? (lds_at<float>(M_OFF + hq * 4) + log2f(den)) * 0.69314718055994530942f : -INFINITY;
     }
 }
 

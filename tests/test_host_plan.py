@@ -317,6 +317,58 @@ def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, b
             assert int(tn[c0 | (c1 << 4)]) == int(vl[c0]) | (int(vl[c1]) << 16)
 
 
+@pytest.mark.parametrize("alloc", [None, [3] * 64, [1, 2, 3] + [4] * 5 + [5] + [8] * 55, [5] * 40 + [2] * 24])
+def test_record_walk_covers_every_unit_once(alloc):
+    """The decode kernel's walk over a K record: steps of at most 8 units, each inside one segment,
+    in record order; a step's byte offset, first unit, norm column, kind and table follow from the
+    segment table; units tile the segments' dims; 5-bit codes come with their pair table."""
+    from blockgtq_amd import plan as P
+    q, _ = make_quantizer(seed=17, min_bits=1, max_bits=8, budget=200, alloc=alloc)
+    p = q.plan()[0]
+    n_seg = int(p['n_seg'])
+    for layout in (P.K_BITPACKED, P.K_MIXED):
+        n_walk = int(p['n_walk'][layout])
+        assert 1 <= n_walk <= P.MAX_WALK and not p['swalk'][layout, n_walk:].any()
+        steps = [[int(x) for x in row] for row in p['swalk'][layout, :n_walk]]
+        units = [int(x) for x in p['sunit'][layout]]
+        i = u = n_ptab = 0
+        for s in range(n_seg):
+            bw, ln, start = int(p['seg_bw'][s]), int(p['seg_len'][s]), int(p['seg_start'][s])
+            off = int(p['seg_pack_off' if layout == P.K_BITPACKED else 'seg_mixed_off'][s])
+            w = (bw if layout == P.K_BITPACKED else 4) if bw <= 4 else 0
+            n_u = (ln + 7) // 8
+            for k in range(n_u):                                   # the unit map: 8 dims a unit, the last one shorter
+                assert units[u + k] == (start + 8 * k) | (min(8, ln - 8 * k) << 8)
+            done = 0
+            while done < n_u:
+                w0, tab, w2, w3 = steps[i]
+                run = min(8, n_u - done)
+                at = off + done * (w if w else 8)
+                kind = (w - 1) * 8 + run - 1 if w else (P.STEP_RAW5 if bw == 5 else P.STEP_RAW) + run - 1
+                assert w0 == (at & 3) | (kind << 2) and w3 == 0
+                assert w2 == (at & ~3) | (2 * s << 8) | (16 * (u + done) << 16)
+                if w and layout == P.K_BITPACKED:
+                    assert tab == P.VLUT_BYTES + P.LUT_K[bw]
+                elif w:
+                    assert tab == P.VLUT_BYTES + 1024 * n_ptab
+                elif bw == 5:
+                    assert tab == P.VLUT_BYTES + P.LUT_K5P
+                else:
+                    assert tab == P.VLUT_BYTES + (P.LUT_KRAW if layout == P.K_BITPACKED else P.LUTM_KRAW) + (bw - 5) * 512
+                done += run
+                i += 1
+            u += n_u
+            n_ptab += bw <= 4 and layout == P.K_MIXED
+        assert i == n_walk and not any(units[u:])
+        has5 = 5 in [int(b) for b in p['seg_bw'][:n_seg]]
+        assert int(p['n_walk'][2 + layout]) == int(has5)
+        if has5:
+            cb = p['k_codebook_f16'][[int(b) for b in p['seg_bw'][:n_seg]].index(5)]
+            t = p['lut_image'][layout][P.LUT_K5P // 4:][:1024]
+            for c0, c1 in ((0, 0), (31, 0), (0, 31), (7, 19), (31, 31)):
+                assert int(t[c0 | (c1 << 5)]) == int(cb[c0]) | (int(cb[c1]) << 16)
+
+
 # ---------------------------------------------------------------- V packing
 @pytest.mark.parametrize("bits", [1, 2, 3, 4])
 def test_v_packing_matches_a_plain_bit_stream(bits):
