@@ -1,40 +1,41 @@
 // Decode attention over packed K and V records (gfx950): the bandwidth kernel.
 //
-// One work-group of up to 12 waves owns one partition of one (batch row, KV head).  The
+// One work-group of up to 16 waves owns one partition of one (batch row, KV head).  The
 // 64-token tiles of a (batch row, KV head) are dealt to the partitions as evenly as whole
 // tiles allow and round-robin to the waves of a partition; every wave walks its tiles with
 // a private online softmax and the waves are merged through LDS at the end.
 //
 // Data movement.  A tile of packed records is one contiguous byte range of the cache.  It
 // goes from HBM straight into LDS with global_load_lds_dwordx4 (aligned 16-byte pieces, the
-// 16-byte phase of the source is kept) into the wave's own K buffer as soon as QK^T of the
-// previous tile has read it, V likewise after PV, and the fp16 norms travel the same way.
+// 16-byte phase of the source is kept) into the wave's own K buffer as soon as the previous
+// tile is done with it, V likewise, and the fp16 norms travel the same way.  The set-up
+// barrier waits for the tables and query rows only; a wave waits for its own tile.
 //
-// What bounds the kernel is the LDS pipe (one wave instruction per two clocks per CU at
-// best) and then vector-ALU issue, not HBM: every table lookup is an LDS read.  The kernel
-// is therefore written around the number of LDS instructions per tile:
+// What bounds the kernel is instruction issue (a wave issues at most one instruction per ten
+// clocks or so, a SIMD one per three to four over its waves, whatever the class), not HBM:
+// it is written around the number of instructions per tile.
 //
-// QK^T   lane = token.  The K record is walked segment by segment (a segment is a run of dims
-//        of one code width, so field positions are compile-time constants inside a segment's
-//        loop and nothing but the segment's table address and byte offset is read per
-//        segment).  A "unit" is 8 consecutive codes: one aligned 8-byte read and a byte funnel
-//        shift bring the unit's bytes into a register, four {shift, and-or, 4-byte table read}
-//        triples turn it into the eight fp16 operands of one MFMA k-group.  Tables of at most
-//        64 entries are replicated 32 times (entry stride 128 bytes): LDS serves the 32 lanes
-//        of a half-wave together and the replicas put them on 32 different banks.
+// QK^T   lane = token.  The K record is walked step by step; a step is a run of up to 8 units
+//        (8 consecutive codes each) of one segment, and there is one straight-line body per
+//        (code width, unit count): the run's bytes are read as aligned dwords, one byte funnel
+//        per dword brings them to bit 0, and from there every field position is a constant:
+//        {shift, and-or, 4-byte table read} per code pair.  Tables of at most 64 entries are
+//        replicated 32 times (entry stride 128 bytes): LDS serves the 32 lanes of a half-wave
+//        together and the replicas put them on 32 different banks.
 //        One MFMA per unit: B = dequantised K (one token per lane), A = the unit's rotated
 //        queries, zero outside the lane's own lane group ("block diagonal"), so every lane
 //        receives the scores of its own token for all heads: v_mfma_f32_32x32x16_f16 for up
 //        to 8 heads (lanes 0..31 and 32..63 are the two diagonal blocks), v_mfma_f32_16x16x32_f16
-//        for up to 4.  The A rows are read from LDS once per unit (16 bytes a lane).  The
-//        units of a segment accumulate in the MFMA and the segment's sum is scaled by the
-//        token's fp16 norm of that segment in fp32.
+//        for up to 4.  The A rows are read from LDS once per unit (16 bytes a lane, immediate
+//        offsets).  The units of a step accumulate in the MFMA and the step's sum is scaled by
+//        the token's fp16 norm of that segment in fp32.
 // Softmax lane = token, exponentials relative to a per-head wave-uniform reference that is kept
 //        above every score seen so far and only moved when a score exceeds it.
 // PV     P * v_norm goes through LDS once into the A layout of the value product, which runs
 //        over (token, dim parity) pairs so that a V table word is an MFMA operand as it comes.
 // Merge  every wave leaves its reference, denominator and sums in its own (then dead) tile
-//        buffers; after one barrier the first 32 * gqa threads fold the waves.
+//        buffers; one thread per (wave, head) works out the factors, one per (head, output)
+//        folds the waves.
 #include <atomic>
 #include <type_traits>
 
