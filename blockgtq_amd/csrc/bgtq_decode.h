@@ -26,6 +26,12 @@ struct DecodeArgs {
     int p_over_k;          // MFMA kernel: the P tile lies over the K tile (no buffer of its own)
     TileLayout tl;
     int wave_bytes;        // MFMA kernel: LDS bytes of one wave's buffers
+    // MFMA kernel: 1 when every (row, head) slice of the four cache tensors starts on a 16-byte boundary;
+    // then a whole 64-token tile of the K records, K norms, V norms and V records is nfull[i] whole 1 KB
+    // loads and one more for the lanes in last[i]
+    int aligned16;
+    int nfull[4];
+    uint64_t last[4];
     int per_tiles, rem_tiles;   // MFMA kernel, equal row lengths: tiles per partition, partitions with one more
 };
 

@@ -177,7 +177,10 @@ __device__ __forceinline__ void step_pairs(float (&S)[8], float n, uint32_t a0, 
     constexpr int SH = W == 4 ? 2 : 7;                     // 256-entry tables are not replicated
     constexpr uint32_t MASK = ((1u << (2 * W)) - 1u) << SH;
     constexpr int ND = (NU * W + 3) / 4;
-    const uint32_t tb = W == 4 ? tab : (tab | rep);
+    // (bit-packed codes of 1..3 bits: the table sits at a fixed place of the table area; nibble tables are one per
+    // segment and their address comes with the step)
+    constexpr uint32_t FIXED = VTAB_BYTES + (W == 1 ? BGTQ_LUT_K1 : W == 2 ? BGTQ_LUT_K2 : BGTQ_LUT_K3);
+    const uint32_t tb = W == 4 ? tab : (rep | FIXED);
     uint32_t r[ND + 1], e[ND];
 #pragma unroll
     for (int i = 0; i <= ND; i++) r[i] = lds_at<uint32_t>(a0 + 4 * i);      // (the last one may lie past the run: inside the tile buffer's slack)
@@ -350,14 +353,15 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     }
 
     // ---- tables by DMA: V table at LDS offset 0, K tables behind it; the chunks are dealt round-robin
-    // to the waves
+    // to the first four waves (the others go straight on to their first tile)
     const uint32_t voff = (uint32_t)lane * 16;
-    {
+    const int tab_waves = min(nw, 4);
+    if (wave < tab_waves) {
         const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
         const uint8_t* kimg_src = (const uint8_t*)P.lut_image[kl];
         const int vbytes = vlut_bytes(VBW, vnib), kbytes = P.n_walk[2 + kl] ? BGTQ_LUT_K5PEND : kimg_bytes(kl);
         const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
-        for (int cc = wave; cc < vch + kch; cc += nw) {
+        for (int cc = wave; cc < vch + kch; cc += tab_waves) {
             const uint8_t* src;
             uint32_t dst;
             int left;
@@ -377,10 +381,21 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const uint8_t* vp_base = a.vp + at_bh(a.vp_sb, a.vp_sh, 1);
     const uint8_t* kn_base = (const uint8_t*)a.kn + at_bh(a.kn_sb, a.kn_sh, 2);
     const uint8_t* vn_base = (const uint8_t*)a.vn + at_bh(a.vn_sb, a.vn_sh, 2);
-    const uint32_t kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
-    const uint32_t knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
-    const DmaShape full_k = dma_shape_uniform((int)kph + MT * krow), full_kn = dma_shape_uniform((int)knph + MT * kn_st * 2);
-    const DmaShape full_vn = dma_shape_uniform((int)vnph + MT * 2), full_v = dma_shape_uniform((int)vph + MT * vrow);
+    // (every slice on a 16-byte boundary, the usual case: the phases are zero and the launcher has worked
+    // out how a whole tile of each range is cut into 1 KB loads)
+    uint32_t kph = 0, vph = 0, knph = 0, vnph = 0;
+    DmaShape full_k, full_kn, full_vn, full_v;
+    if (a.aligned16) {
+        full_k = DmaShape{a.nfull[0], a.last[0]};
+        full_kn = DmaShape{a.nfull[1], a.last[1]};
+        full_vn = DmaShape{a.nfull[2], a.last[2]};
+        full_v = DmaShape{a.nfull[3], a.last[3]};
+    } else {
+        kph = (uint32_t)((uintptr_t)kp_base & 15), vph = (uint32_t)((uintptr_t)vp_base & 15);
+        knph = (uint32_t)((uintptr_t)kn_base & 15), vnph = (uint32_t)((uintptr_t)vn_base & 15);
+        full_k = dma_shape_uniform((int)kph + MT * krow), full_kn = dma_shape_uniform((int)knph + MT * kn_st * 2);
+        full_vn = dma_shape_uniform((int)vnph + MT * 2), full_v = dma_shape_uniform((int)vph + MT * vrow);
+    }
     auto tail_of = [&](const uint8_t* base, uint32_t lds, const DmaShape& d) -> DmaTail {
         return DmaTail{base + d.nfull * 1024, lds + (uint32_t)d.nfull * 1024u, d.last};
     };
@@ -506,12 +521,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         for (int hh = 0; hh < 8; hh++) S[hh] = 0.f;
         {
             for (int s = 0; s < n_walk; s++) {
-                const uint32_t w0 = __builtin_amdgcn_readlane(seg_w0, s), tab = __builtin_amdgcn_readlane(seg_w1, s);
-                const uint32_t w2 = __builtin_amdgcn_readlane(seg_w2, s);
+                const uint32_t w0 = __builtin_amdgcn_readlane(seg_w0, s), w2 = __builtin_amdgcn_readlane(seg_w2, s);
                 const uint32_t n16 = lds_at<uint16_t>(knrow_l + ((w2 >> 8) & 0xFFu));
                 const uint32_t a0 = krow_l + (w2 & 0xFFu), qa = qs_l + (w2 >> 16);
-                const float n = bgtq_h2f((uint16_t)n16) * c2;
-#define BGTQ_STEP(W, NU) case (W - 1) * 8 + NU - 1: step_pairs<W, HEADS, NU>(S, n, a0, w0, tab, rep, qa); break;
+                const float n = bgtq_h2f((uint16_t)n16);
+#define BGTQ_STEP(W, NU) case (W - 1) * 8 + NU - 1: step_pairs<W, HEADS, NU>(S, n, a0, w0, W == 4 ? __builtin_amdgcn_readlane(seg_w1, s) : 0u, rep, qa); break;
 #define BGTQ_STEPS(W) BGTQ_STEP(W, 1) BGTQ_STEP(W, 2) BGTQ_STEP(W, 3) BGTQ_STEP(W, 4) BGTQ_STEP(W, 5) BGTQ_STEP(W, 6) BGTQ_STEP(W, 7) BGTQ_STEP(W, 8)
                 switch (w0 >> 2) {
                 BGTQ_STEPS(1) BGTQ_STEPS(2) BGTQ_STEPS(3) BGTQ_STEPS(4)
@@ -523,7 +537,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
                 case BGTQ_STEP_RAW5 + 5: step_raw5<HEADS, 6>(S, n, a0, w0, qa); break;
                 case BGTQ_STEP_RAW5 + 6: step_raw5<HEADS, 7>(S, n, a0, w0, qa); break;
                 case BGTQ_STEP_RAW5 + 7: step_raw5<HEADS, 8>(S, n, a0, w0, qa); break;
-                default: step_raw<HEADS>(S, n, a0 + (w0 & 3u), (int)(w0 >> 2) - BGTQ_STEP_RAW + 1, tab, qa); break;
+                default: step_raw<HEADS>(S, n, a0 + (w0 & 3u), (int)(w0 >> 2) - BGTQ_STEP_RAW + 1, __builtin_amdgcn_readlane(seg_w1, s), qa); break;
                 }
 #undef BGTQ_STEPS
 #undef BGTQ_STEP
@@ -540,7 +554,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
             const bool live = FULL || lane < nt;
             float d[8];
 #pragma unroll
-            for (int hh = 0; hh < 8; hh++) d[hh] = S[hh] - m_ref[hh];
+            for (int hh = 0; hh < 8; hh++) d[hh] = __builtin_fmaf(S[hh], c2, -m_ref[hh]);      // S is in natural units, the reference in log2 units
             bool refresh = FRESH;
             if (!FRESH) {
                 const float mx = fmaxf(fmaxf(fmaxf(d[0], d[1]), fmaxf(d[2], d[3])), fmaxf(fmaxf(d[4], d[5]), fmaxf(d[6], d[7])));
@@ -555,15 +569,16 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
 #pragma unroll
                 for (int hh = 0; hh < 8; hh++) {
                     const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wm[hh]), 63));
+                    const float top2 = top * c2;
                     if (FRESH) {
-                        m_ref[hh] = top + REFRESH;
+                        m_ref[hh] = top2 + REFRESH;
                     } else {
-                        const float m_new = top > m_ref[hh] ? top + REFRESH : m_ref[hh];
+                        const float m_new = top2 > m_ref[hh] ? top2 + REFRESH : m_ref[hh];
                         alpha[hh] = __builtin_amdgcn_exp2f(m_ref[hh] - m_new);
                         l_part[hh] *= alpha[hh];
                         m_ref[hh] = m_new;
                     }
-                    d[hh] = S[hh] - m_ref[hh];
+                    d[hh] = __builtin_fmaf(S[hh], c2, -m_ref[hh]);
                 }
                 if (!FRESH) {
                     // acc rows are heads 4(lg & 1) + r
@@ -739,6 +754,19 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
     a.nw = nw;
     a.p_over_k = over ? 1 : 0;
     a.wave_bytes = wave_lds_bytes(a.tl, over);
+    {
+        // slices that all start on 16-byte boundaries: the cut of a whole tile into 1 KB loads is the same everywhere
+        const int64_t al[] = {(int64_t)(uintptr_t)a.kp, a.kp_sb, a.kp_sh, (int64_t)(uintptr_t)a.kn, 2 * a.kn_sb, 2 * a.kn_sh,
+                              (int64_t)(uintptr_t)a.vp, a.vp_sb, a.vp_sh, (int64_t)(uintptr_t)a.vn, 2 * a.vn_sb, 2 * a.vn_sh};
+        a.aligned16 = 1;
+        for (int64_t v : al) if (v & 15) a.aligned16 = 0;
+        const int bytes[4] = {MT * a.k_row_width, MT * (int)a.kn_st * 2, MT * 2, MT * VST};
+        for (int r = 0; r < 4; r++) {
+            const int nfull = ((bytes[r] + 1023) >> 10) - 1, pieces = (bytes[r] - nfull * 1024 + 15) >> 4;
+            a.nfull[r] = nfull;
+            a.last[r] = pieces >= 64 ? ~0ull : ((1ull << pieces) - 1ull);
+        }
+    }
     a.per_tiles = tiles / a.n_splits;
     a.rem_tiles = tiles - a.per_tiles * a.n_splits;
     auto kern = decode_seg_kernel<HEADS, VBW, VST>;
