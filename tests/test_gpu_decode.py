@@ -88,6 +88,8 @@ CASES = [  # budget mn mx vb n_kv gqa B T k_layout v_layout
     (192, 1, 5, 3, 1, 12, 2, 333, 0, 0),      # 9..16 heads: two launches of the matrix-core kernel
     (192, 1, 5, 3, 2, 9, 1, 333, 1, 0),
     (160, 1, 6, 4, 2, 3, 2, 200, 1, 1),
+    (192, 1, 5, 3, 2, 8, 2, 1022, 0, 0),      # T + 2 rows: every (row, head) slice of the cache starts on a 16-byte boundary
+    (192, 1, 8, 3, 2, 4, 2, 510, 1, 1),
 ]
 
 
