@@ -150,7 +150,7 @@ def run(model_name="qwen2.5-3b", batch=4, prompt_len=8192, new_tokens=256, k_bit
             ids.copy_(lg.argmax(-1))
             pos.add_(1)
 
-        state = (ids.clone(), pos.clone(), cache._seq_lens.clone(), cache.seq_len)
+        state = (ids.clone(), pos.clone(), cache._lens2.clone(), cache.seq_len)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -161,7 +161,7 @@ def run(model_name="qwen2.5-3b", batch=4, prompt_len=8192, new_tokens=256, k_bit
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             step()
-        ids.copy_(state[0]); pos.copy_(state[1]); cache._seq_lens.copy_(state[2])
+        ids.copy_(state[0]); pos.copy_(state[1]); cache._lens2.copy_(state[2])
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(n_graph):

@@ -36,6 +36,7 @@ class BlockGTQProductionCache:
         self.scale = 1.0 / math.sqrt(hd)
         self.seq_len = 0
         self._seq_lens = None
+        self._lens2 = None
         self._static_T = None          # launch bound used instead of seq_len in graph mode
         self.max_T = max_T
 
@@ -83,12 +84,20 @@ class BlockGTQProductionCache:
         The cache keeps its own copy and advances it in place."""
         if seq_lens is None:
             self._seq_lens = None
+            self._lens2 = None
             self._static_T = None
             return
-        t = torch.as_tensor(seq_lens, dtype=torch.int32).to(self.device).clone()
+        t = torch.as_tensor(seq_lens, dtype=torch.int32).to(self.device)
         assert t.numel() == self.B
-        self._seq_lens = t
+        self._set_device_lengths(t)
         self.seq_len = int(t.max().item())
+
+    def _set_device_lengths(self, lens):
+        """Row 0: tokens in the cache per batch row (the append position); row 1: one more (what a
+        single-token step attends over).  Both advance together, so a step launches no arithmetic
+        on the lengths."""
+        self._lens2 = torch.stack([lens.to(torch.int32), lens.to(torch.int32) + 1]).contiguous()
+        self._seq_lens = self._lens2[0]
 
     def use_device_lengths(self):
         """Keep the lengths on the device only, so that a decode step contains no
@@ -97,7 +106,7 @@ class BlockGTQProductionCache:
         the device copy, launches are sized for ``max_T``.  ``seq_len`` on the host
         then counts the steps issued, not replays."""
         if self._seq_lens is None:
-            self._seq_lens = torch.full((self.B,), self.seq_len, dtype=torch.int32, device=self.device)
+            self._set_device_lengths(torch.full((self.B,), self.seq_len, dtype=torch.int32, device=self.device))
         self._static_T = self.max_T
 
     # ---------------------------------------------------------------- decode
@@ -124,7 +133,7 @@ class BlockGTQProductionCache:
                 plans, k16, v16, q3.contiguous(), self.k_packed[li], self.k_norms[li],
                 self.v_packed[li], self.v_norms[li], t_pos, self.k_bytes_per_tok, self.max_ng,
                 self.vpb, self.nkv, self._k_layout, self._v_layout, self.quant_mode)
-        lens = self._seq_lens + S if self._seq_lens is not None else None
+        lens = None if self._seq_lens is None else self._lens2[1] if S == 1 else self._seq_lens + S
         out = ops.decode_attention(
             plans, q3.contiguous(), self.k_packed[li], self.k_norms[li],
             self.v_packed[li], self.v_norms[li], T, seq_lens=lens, n_splits=self.n_splits,
@@ -135,7 +144,7 @@ class BlockGTQProductionCache:
     def increment_seq_len(self, by=1):
         self.seq_len += by
         if self._seq_lens is not None:
-            self._seq_lens.add_(by)
+            self._lens2.add_(by)
 
     # ------------------------------------------------------------ accounting
     def cache_memory_bytes(self) -> int:
