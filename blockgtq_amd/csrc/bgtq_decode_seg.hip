@@ -329,7 +329,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     }
     // segment words: lane s of every wave keeps the two words of segment s (read back with v_readlane)
     uint32_t seg_w0 = 0, seg_w1 = 0, seg_w2 = 0;
-    if (lane < n_walk) {
+    if (lane < BGTQ_MAX_WALK) {                            // (steps past the last are zero in the plan: no wait for the count)
         seg_w0 = P.swalk[kl][lane][0];
         seg_w1 = P.swalk[kl][lane][1];
         seg_w2 = P.swalk[kl][lane][2];
