@@ -92,10 +92,6 @@ __device__ inline void split_row(int64_t n, int S, int& b, int& s) {
 // every later table access is an LDS read instead of one more dependent trip to memory.
 struct StagedK {
     int hdr[56];                 // n_seg .. seg_identity, as at the start of bgtq_head_plan
-    int group_of[D];
-    int head_perm[D];
-    float lut_offset[D];
-    float lut_inv_scale[D];
     uint8_t code_lut[BGTQ_MAX_SEGMENTS * BGTQ_LUT_BINS];
     float centroids[BGTQ_MAX_SEGMENTS * 32];   // first 32 levels of every segment (bw <= 5)
 };
@@ -167,10 +163,6 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         if (j < 16) { sp.centroids[j] = P.v_centroids[j]; sp.boundaries[j] = P.v_boundaries[j]; }
     } else {
         if (j < 56) sp.hdr[j] = ((const int*)&P)[j];
-        sp.group_of[j] = P.group_of[j];
-        sp.head_perm[j] = P.head_perm[j];
-        sp.lut_offset[j] = P.lut_offset[j];
-        sp.lut_inv_scale[j] = P.lut_inv_scale[j];
 #pragma unroll
         for (int i = 0; i < 4; i++)
             ((uint32_t*)sp.code_lut)[j + i * NT] = ((const uint32_t*)&P.code_lut[0][0])[j + i * NT];
@@ -181,7 +173,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
     uint16_t xr[ROWS];                 // raw rows of the tile about to be processed
-    int tp[ROWS == 2 ? 2 : 1];         // decode append: their cache positions, fetched with them
+    int tp[2];         // decode append: their cache positions, fetched with them
     auto fetch_rows = [&](int64_t tile) {
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
@@ -192,13 +184,22 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
                 int b, s;
                 split_row(n, a.S, b, s);
                 v = a.x[b * a.x_sb + h * a.x_sh + s * a.x_ss + j];
-                if (ROWS == 2) t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+                if (ROWS <= 2) t = (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             }
             xr[r] = v;
-            if (ROWS == 2) tp[r] = t;
+            if (ROWS <= 2) tp[r] = t;
         }
     };
     fetch_rows(bx);
+    int4 k_dim = {0, 0, 0, 0};
+    uint2 k_byte = {0u, 0u};
+    float k_lut_off = 0.f, k_lut_scale = 0.f;
+    if constexpr (!IS_V) {
+        k_dim = *(const int4*)P.enc_dim[j];
+        k_byte = *(const uint2*)P.enc_byte[a.layout == BGTQ_K_MIXED ? 1 : 0][j];
+        k_lut_off = P.lut_offset[j];
+        k_lut_scale = P.lut_inv_scale[j];
+    }
     // Decode append (2-row tiles) is latency bound.  K: the whole rotation matrix is requested now,
     // before anything else is known (which rows a thread needs is only known once the plan is in
     // LDS), 16 bytes a lane and contiguous across the wave (32 loads a thread), and parked in LDS
@@ -206,65 +207,64 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     // their column slices per tile instead.
     // V's rotation is dense and is needed later than its rows: its column comes straight into
     // registers, one 4-byte load per matrix row (the wide loads of the whole matrix land later).
-    constexpr bool STAGED = ROWS == 2 && !IS_V;
-    constexpr int PF = (ROWS == 2 && IS_V) ? D : 0;
+    constexpr bool STAGED = ROWS <= 2 && !IS_V;
+    constexpr int PF = (ROWS <= 2 && IS_V) ? D : 0;
     rot_piece rst[STAGED ? D / 4 : 1];
     float rpre[PF > 0 ? PF : 1];
-    if constexpr (STAGED) fetch_rotation(RT, j, rst);
+    // K, where no rotated segment is longer than BGTQ_ROT_COL dims: the plan also holds every dim's
+    // rotation column cut down to its segment, which goes straight into registers (12 wide loads
+    // instead of 32 and no trip through LDS)
+    constexpr int RC = STAGED ? BGTQ_ROT_COL : 4;
+    float rc[RC];
+    bool compact = false;
+    if constexpr (STAGED) {
+        compact = P.rot_compact[0] != 0;                 // (uniform)
+        if (compact) {
+#pragma unroll
+            for (int i = 0; i < RC / 4; i++) {
+                const float4 v = *(const float4*)&P.k_rot_cols[j][4 * i];
+                rc[4 * i] = v.x; rc[4 * i + 1] = v.y; rc[4 * i + 2] = v.z; rc[4 * i + 3] = v.w;
+            }
+        } else {
+            fetch_rotation(RT, j, rst);
+        }
+    }
     if constexpr (PF > 0) {
 #pragma unroll
         for (int i = 0; i < PF; i++) rpre[i] = RT[i * D + j];
     }
     __syncthreads();
 
-    // ---- per-thread static data -------------------------------------------
+    // ---- per-thread static data: K threads read theirs ready-made from the plan (requested in the
+    // first burst), V needs none -------------------------------------------
     int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
     float lut_off_j = 0.f, lut_scale_j = 0.f;          // K: this dim's cell-search parameters
-    if constexpr (!IS_V) {
-        lut_off_j = sp.lut_offset[j];
-        lut_scale_j = sp.lut_inv_scale[j];
-        n_seg = sp.hdr[H_NSEG];
-        g = sp.group_of[j];
-        src_dim = sp.head_perm[j];
-        if (g >= 0) { gs = sp.hdr[H_START + g]; ge = gs + sp.hdr[H_LEN + g]; ident = sp.hdr[H_IDENT + g]; }
-        else        { gs = 0; ge = 0; }
-    }
-
-    // ---- pack geometry of output byte j (row independent) ------------------------
-    int mode = 0;        // 0: zero fill, 1: bit stream, 2: raw byte copy
+    int mode = 0;        // output byte j: 0: zero fill, 1: bit stream, 2: raw byte copy
     int c0 = 0, clen = 0, bw = 1, idx = 0;
-    if constexpr (IS_V) {
+    StreamSlot slot{0, 0, 0};
+    if constexpr (!IS_V) {
+        lut_off_j = k_lut_off;
+        lut_scale_j = k_lut_scale;
+        n_seg = sp.hdr[H_NSEG];
+        g = k_dim.x;
+        gs = k_dim.y;
+        ge = k_dim.z;
+        ident = k_dim.w & 0xFF;
+        src_dim = k_dim.w >> 8;
+        mode = (int)(k_byte.x & 3u);
+        bw = (int)((k_byte.x >> 2) & 15u);
+        slot = StreamSlot{0, (int)(k_byte.x >> 8), (int)((k_byte.x >> 6) & 3u)};
+        c0 = (int)k_byte.y;                             // (the slot's first code is folded into the base)
+    } else {
         bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : sp.v_bits;
         if (j < bgtq_seg_bytes(bw, D)) { mode = 1; c0 = 0; clen = D; idx = j; }
-    } else if (a.layout == BGTQ_K_MIXED) {
-        int z = sp.hdr[H_NZERO], nps = sp.hdr[H_NOPACK_START];
-        int nib = (nps - z) >> 1;
-        if (j < nib)                             { mode = 1; bw = 4; c0 = z; clen = nps - z; idx = j; }
-        else if (j < nib + sp.hdr[H_NOPACK_LEN]) { mode = 2; c0 = nps + (j - nib); }
-    } else {
-        // all table reads of the walk go out together (read one segment at a time, every
-        // iteration waits for its own LDS round trip)
-        int offs[BGTQ_MAX_SEGMENTS], sbs[BGTQ_MAX_SEGMENTS], sls[BGTQ_MAX_SEGMENTS], sts[BGTQ_MAX_SEGMENTS];
-#pragma unroll
-        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) {
-            offs[s] = sp.hdr[H_PACK_OFF + s]; sbs[s] = sp.hdr[H_BW + s];
-            sls[s] = sp.hdr[H_LEN + s];       sts[s] = sp.hdr[H_START + s];
-        }
-#pragma unroll
-        for (int s = 0; s < BGTQ_MAX_SEGMENTS; s++) {
-            const int off = offs[s], sb = sbs[s], sl = sls[s];
-            if (s < n_seg && j >= off && j < off + bgtq_seg_bytes(sb, sl)) {
-                if (sb >= 5) { mode = 2; c0 = sts[s] + (j - off); }
-                else         { mode = 1; bw = sb; c0 = sts[s]; clen = sl; idx = j - off; }
-            }
-        }
+        if (mode == 1) slot = stream_slot(clen, bw, idx);
     }
-    const StreamSlot slot = mode == 1 ? stream_slot(clen, bw, idx) : StreamSlot{0, 0, 0};
 
     for (int64_t tile = bx; tile < n_tiles; tile += tile_stride) {
     const int64_t row0 = tile * ROWS;
     int tcur[2] = {0, 0};              // this tile's positions (the prefetch below overwrites tp)
-    if (ROWS == 2) { tcur[0] = tp[0]; tcur[1] = tp[ROWS == 2 ? 1 : 0]; }
+    if (ROWS <= 2) { tcur[0] = tp[0]; tcur[1] = tp[ROWS == 2 ? 1 : 0]; }
     // ---- 1. rows to LDS, next tile's rows on their way, gather by head_perm (K) -------------
 #pragma unroll
     for (int r = 0; r < ROWS; r++) xraw[r][j] = xr[r];
@@ -307,7 +307,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         xh[r] = v;
         xs[r][j] = v;     // only this thread ever touched xs[r][j] since the barrier
     }
-    if constexpr (STAGED) park_rotation(rot_s, j, rst);   // (every tile of the walk: the registers stay as they are)
+    if constexpr (STAGED) { if (!compact) park_rotation(rot_s, j, rst); }   // (every tile of the walk: the registers stay as they are)
     __syncthreads();
 
     // ---- 4. rotate ------------------------------------------------------------
@@ -321,6 +321,27 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
 #pragma unroll
         for (int r = 0; r < ROWS; r++) y[r] = 0.f;
         if constexpr (STAGED) {
+            if (compact) {
+                // the column is in registers: the row values of a batch are read ahead of the chain
+                constexpr int CB = 16;
+#pragma unroll
+                for (int i0 = 0; i0 < RC; i0 += CB) {
+                    if (gs + i0 < ge) {
+                        float xv[ROWS][CB];
+#pragma unroll
+                        for (int i = 0; i < CB; i++)
+#pragma unroll
+                            for (int r = 0; r < ROWS; r++) xv[r][i] = xs[r][min(gs + i0 + i, ge - 1)];
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int i = 0; i < CB; i++)
+                            if (gs + i0 + i < ge) {
+#pragma unroll
+                                for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xv[r][i], rc[i0 + i], y[r]);
+                            }
+                    }
+                }
+            } else
             // column j of the parked rotation against the rows, the LDS reads a batch ahead of
             // the chain that consumes them
             {
@@ -498,7 +519,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         if (n < N && gg < width) {
             int b, s;
             split_row(n, a.S, b, s);
-            int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            int64_t t = ROWS <= 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             if (t >= 0 && t < a.max_T)
                 a.norms[b * a.n_sb + h * a.n_sh + t * a.n_st + gg] = bgtq_f2h(nrm_out[r][gg]);
         }
@@ -512,10 +533,10 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             if (n >= N) break;
             int b, s;
             split_row(n, a.S, b, s);
-            int64_t t = ROWS == 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
+            int64_t t = ROWS <= 2 ? tcur[r & 1] : (a.t_pos ? a.t_pos[b] : a.t_pos_scalar) + s;
             if (t < 0 || t >= a.max_T) continue;
             unsigned v = 0;
-            if (mode == 1)      v = ROWS == 2 ? stream_byte_batched(&cds[r][c0], slot, bw) : stream_byte(&cds[r][c0], slot, bw);
+            if (mode == 1)      v = ROWS <= 2 ? stream_byte_batched(&cds[r][c0], slot, bw) : stream_byte(&cds[r][c0], slot, bw);
             else if (mode == 2) v = cds[r][c0];
             a.packed[b * a.p_sb + h * a.p_sh + t * a.p_st + j] = (uint8_t)v;
         }
@@ -527,7 +548,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
 template <int ROWS, bool IS_V>
 __global__ __launch_bounds__(NT) void encode_kernel(EncodeArgs a) {
     const int64_t N = (int64_t)a.B * a.S;
-    __shared__ __align__(16) float rot_s[(ROWS == 2 && !IS_V) ? D * D : 4];
+    __shared__ __align__(16) float rot_s[(ROWS <= 2 && !IS_V) ? D * D : 4];
     encode_rows<ROWS, IS_V>(a, blockIdx.x, blockIdx.y, (N + ROWS - 1) / ROWS, gridDim.x, rot_s);
 }
 // The prefill-sized encoder is throughput bound: at least 4 waves per SIMD (128 registers a
@@ -546,7 +567,10 @@ int launch_encode(const EncodeArgs& a, hipStream_t st) {
     // Few rows (decode append): small tiles so every row gets its own work-group
     // and the step stays latency-bound; many rows (prefill): 16-row tiles so the
     // rotation matrix is amortised.
-    if (N <= 64) {
+    if (N <= 32) {               // one row a work-group: the shortest chain of dependent stages
+        dim3 grid((unsigned)N, (unsigned)a.n_kv);
+        hipLaunchKernelGGL((encode_kernel<1, IS_V>), grid, dim3(NT), 0, st, a);
+    } else if (N <= 64) {
         dim3 grid((unsigned)((N + 1) / 2), (unsigned)a.n_kv);
         hipLaunchKernelGGL((encode_kernel<2, IS_V>), grid, dim3(NT), 0, st, a);
     } else {
@@ -654,19 +678,21 @@ __global__ __launch_bounds__(NT) void rotate_q_kernel(RotQArgs a) {
     rotate_q_block(a, blockIdx.x, rot_s);
 }
 
+constexpr int PREP_ROWS = 1;       // rows of a work-group in the one-launch preparation
+
 // ---- decode-step preparation: append-encode K and V and rotate the queries, one launch ----
-// Work-groups [0, nk) encode K row pairs, [nk, nk + nv) V row pairs, the rest rotate one or four
-// query heads each.
+// Work-groups [0, nk) encode one K row each, [nk, nk + nv) one V row each, the rest rotate one or
+// four query heads each.
 __global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs av, RotQArgs aq,
                                                      int k_tiles, int v_tiles) {
     __shared__ __align__(16) float rot_s[D * D];       // the work-group's rotation, whatever its role
     int bid = blockIdx.x;
     const int nk = k_tiles * ak.n_kv, nv = v_tiles * av.n_kv;
     if (bid < nk) {
-        encode_rows<2, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles, rot_s);
+        encode_rows<PREP_ROWS, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles, rot_s);
     } else if (bid < nk + nv) {
         bid -= nk;
-        encode_rows<2, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles, rot_s);
+        encode_rows<PREP_ROWS, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles, rot_s);
     } else {
         rotate_q_block(aq, bid - (nk + nv), rot_s);
     }
@@ -830,7 +856,7 @@ int bgtq_decode_prepare(const bgtq_head_plan* plans,
     }
     const int group = rotate_q_group_size(B, n_kv * gqa);
     RotQArgs aq{plans, (const uint16_t*)q, q_sr, q_sh, (uint16_t*)q_rot, qr_sr, qr_sh, B, n_kv * gqa, gqa, group};
-    const int tiles = (int)((N + 1) / 2);
+    const int tiles = (int)((N + PREP_ROWS - 1) / PREP_ROWS);
     const unsigned blocks = (unsigned)(2 * tiles * n_kv) + (with_q ? rotate_q_blocks(B, n_kv, gqa, group) : 0u);
     hipLaunchKernelGGL(prepare_kernel, dim3(blocks), dim3(NT), 0, (hipStream_t)stream, ak, av, aq, tiles, tiles);
     return bgtq_launch_status();

@@ -14,6 +14,7 @@ MAX_CENTROIDS = 256
 LUT_BINS = 256
 MAX_UNITS = 24
 MAX_WALK = 12
+ROT_COL = 48
 
 K_BITPACKED, K_MIXED = 0, 1
 V_BITPACKED, V_NIBBLE = 0, 1
@@ -34,6 +35,8 @@ PLAN_DTYPE = np.dtype([
     ('k_centroids', '<f4', (_S, _C)), ('k_boundaries', '<f4', (_S, _C)),
     ('k_codebook_f16', '<u2', (_S, _C)),
     ('k_rot_T', '<f4', (_D * _D,)),
+    ('k_rot_cols', '<f4', (_D, ROT_COL)), ('rot_compact', '<i4', (4,)),
+    ('enc_dim', '<i4', (_D, 4)), ('enc_byte', '<u4', (2, _D, 2)),
     ('v_centroids', '<f4', (16,)), ('v_boundaries', '<f4', (16,)),
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
@@ -136,6 +139,51 @@ def fill_segment_walk(p) -> None:
         p['sunit'][layout, :len(units)] = units
 
 
+def _seg_bytes(bw: int, ln: int) -> int:
+    return {1: (ln + 7) // 8, 2: (ln + 3) // 4, 3: (ln + 7) // 8 * 3, 4: (ln + 1) // 2}.get(bw, ln)
+
+
+def fill_encoder_tables(p) -> None:
+    """Per packed dim and per record byte what the K encoder's threads would otherwise derive from
+    the segment table: the dim's segment range, source dim and rotation flag, and the codes a
+    record byte is made of (both K layouts)."""
+    n_seg, D = int(p['n_seg']), HEAD_DIM
+    for j in range(D):
+        g = int(p['group_of'][j])
+        gs = int(p['seg_start'][g]) if g >= 0 else 0
+        ge = gs + int(p['seg_len'][g]) if g >= 0 else 0
+        ident = int(p['seg_identity'][g]) if g >= 0 else 0
+        p['enc_dim'][j] = [g, gs, ge, ident | (int(p['head_perm'][j]) << 8)]
+    p['enc_byte'][...] = 0
+    z, nps, npl = int(p['n_zero_dims']), int(p['nopack_start']), int(p['nopack_len'])
+    for j in range(D):
+        for layout in (K_BITPACKED, K_MIXED):
+            mode = bw = c0 = clen = idx = 0
+            if layout == K_MIXED:
+                nib = (nps - z) >> 1
+                if j < nib:
+                    mode, bw, c0, clen, idx = 1, 4, z, nps - z, j
+                elif j < nib + npl:
+                    mode, c0 = 2, nps + (j - nib)
+            else:
+                for s in range(n_seg):
+                    off, sb, sl = int(p['seg_pack_off'][s]), int(p['seg_bw'][s]), int(p['seg_len'][s])
+                    if off <= j < off + _seg_bytes(sb, sl):
+                        if sb >= 5:
+                            mode, c0 = 2, int(p['seg_start'][s]) + (j - off)
+                        else:
+                            mode, bw, c0, clen, idx = 1, sb, int(p['seg_start'][s]), sl, j - off
+            if mode == 1:
+                bit0 = idx * 8
+                first = bit0 // bw
+                skip = bit0 - first * bw
+                last = min((bit0 + 7) // bw, clen - 1)
+                n = max(last - first + 1, 0)
+                p['enc_byte'][layout, j] = [1 | (bw << 2) | (skip << 6) | (n << 8), c0 + first]
+            elif mode == 2:
+                p['enc_byte'][layout, j] = [2, c0]
+
+
 def fill_decode_steps(p) -> None:
     """Derive the unit programs of both K record layouts and the table images from the
     segment table, codebooks and V LUT already stored in plan ``p`` (a 0-d structured array)."""
@@ -207,6 +255,7 @@ def fill_decode_steps(p) -> None:
         p['vlut_image'][V_BITPACKED, :t.size] = t
         p['vlut_image'][V_NIBBLE, :256] = _byte_pair_table(p['v_lut_f16'], vb)
     fill_segment_walk(p)
+    fill_encoder_tables(p)
 
 
 def build_head_plan(quantizer) -> np.ndarray:
@@ -263,6 +312,19 @@ def build_head_plan(quantizer) -> np.ndarray:
     p['lut_offset'] = q._lut_offsets.detach().cpu().numpy()
     p['lut_inv_scale'] = q._lut_inv_scales.detach().cpu().numpy()
     p['k_rot_T'] = rot_T.reshape(-1)
+    # the rotation by columns, each cut down to its own diagonal block (read by the single-row append)
+    p['k_rot_cols'][...] = 0
+    compact = True
+    for g in range(len(widths)):
+        s0, ln = int(p['seg_start'][g]), int(p['seg_len'][g])
+        if int(p['seg_identity'][g]):
+            continue
+        if ln > ROT_COL:
+            compact = False
+            continue
+        p['k_rot_cols'][s0:s0 + ln, :ln] = rot_T[s0:s0 + ln, s0:s0 + ln].T
+    p['rot_compact'][...] = 0
+    p['rot_compact'][0] = int(compact)
 
     nv = 1 << q._v_bits
     vc = q._v_centroids_f32.detach().cpu().numpy()

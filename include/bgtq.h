@@ -29,6 +29,7 @@ extern "C" {
 #define BGTQ_MAX_GQA       16    /* query heads per KV head */
 #define BGTQ_MAX_SPLITS    512   /* FlashDecoding partitions per (batch, KV head) */
 #define BGTQ_STATIC_SCRATCH_BYTES (8u << 20)  /* partition results of bgtq_decode_attend_static */
+#define BGTQ_ROT_COL       48    /* longest rotated segment that bgtq_head_plan.k_rot_cols holds */
 #define BGTQ_MAX_WALK      12    /* steps of the decode kernel's walk over one K record, see bgtq_head_plan.swalk */
 #define BGTQ_STEP_RAW      32    /* first step kind of raw-byte runs */
 #define BGTQ_STEP_RAW5     40    /* first step kind of raw-byte runs of 5-bit codes, read in pairs through the table at BGTQ_LUT_K5P */
@@ -107,6 +108,20 @@ typedef struct bgtq_head_plan {
     float    k_boundaries[BGTQ_MAX_SEGMENTS][BGTQ_MAX_CENTROIDS]; /* 2^bw-1 valid, +inf after */
     uint16_t k_codebook_f16[BGTQ_MAX_SEGMENTS][BGTQ_MAX_CENTROIDS];
     float    k_rot_T[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];  /* y = xhat @ k_rot_T, block diagonal */
+    /* the same rotation by columns, each cut down to its own diagonal block: k_rot_cols[j][i] =
+     * k_rot_T[(start of j's segment + i) * 128 + j], 0 past the segment's end.  Filled (rot_compact[0] = 1)
+     * when no rotated segment is longer than BGTQ_ROT_COL dims: the single-row append reads a dim's
+     * column from here without knowing the segment table first */
+    float    k_rot_cols[BGTQ_HEAD_DIM][BGTQ_ROT_COL];
+    int32_t  rot_compact[4];                    /* [0]: k_rot_cols is filled; rest padding */
+    /* what the K encoder's thread j needs, ready-made: as owner of packed dim j
+     * enc_dim[j] = { segment of the dim (-1: a 0-bit dim), first dim of that segment, one past its
+     * last, seg_identity | head_perm[j] << 8 }, and as writer of record byte j (one table per K layout)
+     * enc_byte[l][j] = { mode | code width << 2 | skip << 6 | n << 8, first code }: mode 0 writes 0,
+     * mode 1 the byte of the LSB-first stream that holds the n codes from `first code` on, less the
+     * `skip` low bits that belong to the byte before, mode 2 the code itself */
+    int32_t  enc_dim[BGTQ_HEAD_DIM][4];
+    uint32_t enc_byte[2][BGTQ_HEAD_DIM][2];
     /* V tables */
     float    v_centroids[16];
     float    v_boundaries[16];                  /* 2^v_bits-1 valid, +inf after */

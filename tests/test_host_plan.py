@@ -369,6 +369,69 @@ def test_record_walk_covers_every_unit_once(alloc):
                 assert int(t[c0 | (c1 << 5)]) == int(cb[c0]) | (int(cb[c1]) << 16)
 
 
+@pytest.mark.parametrize("alloc,mn,mx", [(None, 1, 7), (None, 0, 4), ([3] * 64, 1, 8), ([1, 2, 3] + [4] * 5 + [5] + [8] * 55, 1, 8)])
+def test_encoder_tables_write_the_record_an_independent_packer_writes(alloc, mn, mx):
+    """The K encoder's ready-made tables: `enc_dim` repeats the segment table per dim; a record
+    assembled byte by byte from `enc_byte` (mode, width, skip, count, first code) equals, segment by
+    segment, the independent LSB-first bit-stream writer (whole 8-code groups for 3-bit codes), the
+    nibble stream and the raw bytes; `k_rot_cols` holds every rotated dim's column of its block."""
+    from blockgtq_amd import plan as P
+    q, _ = make_quantizer(seed=23, min_bits=mn, max_bits=mx, budget=190, alloc=alloc)
+    p = q.plan()[0]
+    n_seg = int(p['n_seg'])
+    segs = [(int(p['seg_bw'][s]), int(p['seg_start'][s]), int(p['seg_len'][s])) for s in range(n_seg)]
+    for j in range(128):
+        g, gs, ge, w = (int(x) for x in p['enc_dim'][j])
+        assert g == int(p['group_of'][j]) and (w >> 8) == int(p['head_perm'][j])
+        if g >= 0:
+            assert (gs, ge) == (segs[g][1], segs[g][1] + segs[g][2]) and (w & 255) == int(p['seg_identity'][g])
+        else:
+            assert (gs, ge, w & 255) == (0, 0, 0)
+    rng = np.random.default_rng(5)
+    codes = np.zeros(128, dtype=np.int64)
+    for bw, s0, ln in segs:
+        codes[s0:s0 + ln] = rng.integers(0, 1 << bw, ln)
+
+    def assemble(layout, n_bytes):
+        out = np.zeros(n_bytes, dtype=np.uint8)
+        for j in range(n_bytes):
+            w0, first = (int(x) for x in p['enc_byte'][layout, j])
+            mode, bw, skip, n = w0 & 3, (w0 >> 2) & 15, (w0 >> 6) & 3, w0 >> 8
+            if mode == 1:
+                acc = 0
+                for i in range(n):
+                    acc |= int(codes[first + i]) << (i * bw)
+                out[j] = (acc >> skip) & 255
+            elif mode == 2:
+                out[j] = codes[first]
+        return out
+
+    want = np.zeros(int(p['k_row_bytes']), dtype=np.uint8)
+    for s, (bw, s0, ln) in enumerate(segs):
+        off = int(p['seg_pack_off'][s])
+        if bw >= 5:
+            want[off:off + ln] = codes[s0:s0 + ln]
+        else:
+            padded = np.zeros((ln + 7) // 8 * 8 if bw == 3 else ln, dtype=np.int64)
+            padded[:ln] = codes[s0:s0 + ln]
+            b = stream_pack(padded[None], bw)[0]
+            want[off:off + len(b)] = b
+    assert np.array_equal(assemble(P.K_BITPACKED, len(want)), want)
+    z, nps, npl = int(p['n_zero_dims']), int(p['nopack_start']), int(p['nopack_len'])
+    wantm = np.concatenate([stream_pack(codes[None, z:nps], 4)[0], codes[nps:nps + npl].astype(np.uint8)])
+    assert len(wantm) == int(p['k_mixed_bytes']) and np.array_equal(assemble(P.K_MIXED, len(wantm)), wantm)
+    assert not p['enc_byte'][P.K_BITPACKED, len(want):].any() and not p['enc_byte'][P.K_MIXED, len(wantm):].any()
+
+    rot = p['k_rot_T'].reshape(128, 128)
+    short = all(ln <= P.ROT_COL or int(p['seg_identity'][s]) for s, (_, _, ln) in enumerate(segs))
+    assert int(p['rot_compact'][0]) == int(short)
+    for s, (bw, s0, ln) in enumerate(segs):
+        if int(p['seg_identity'][s]) or ln > P.ROT_COL:
+            continue
+        for j in range(s0, s0 + ln):
+            assert np.array_equal(p['k_rot_cols'][j][:ln], rot[s0:s0 + ln, j]) and not p['k_rot_cols'][j][ln:].any()
+
+
 # ---------------------------------------------------------------- V packing
 @pytest.mark.parametrize("bits", [1, 2, 3, 4])
 def test_v_packing_matches_a_plain_bit_stream(bits):
