@@ -144,7 +144,7 @@ template <int ROWS, bool IS_V>
 __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, const int h,
                                             const int64_t n_tiles, const int tile_stride,
                                             float* rot_s) {
-    __shared__ __align__(16) float xs[ROWS][D];
+    __shared__ __align__(16) float xs[ROWS + 1][D];     // (one more row of zeros: the compact rotation reads up to BGTQ_ROT_COL values past a segment's start)
     __shared__ float nrm[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ float nrm_out[ROWS][BGTQ_MAX_SEGMENTS];
     __shared__ uint8_t cds[ROWS][D];
@@ -172,6 +172,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             sp.centroids[e] = P.k_centroids[e >> 5][e & 31];
         }
     }
+    xs[ROWS][j] = 0.f;
     uint16_t xr[ROWS];                 // raw rows of the tile about to be processed
     int tp[2];         // decode append: their cache positions, fetched with them
     auto fetch_rows = [&](int64_t tile) {
@@ -322,24 +323,23 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         for (int r = 0; r < ROWS; r++) y[r] = 0.f;
         if constexpr (STAGED) {
             if (compact) {
-                // the column is in registers: the row values of a batch are read ahead of the chain
+                // The column is in registers and is zero past the segment's end, so the chain runs over
+                // BGTQ_ROT_COL terms for every dim without a length test: a term x * 0 leaves the sum as it
+                // is (the row is followed by zeros, so every x read is finite).  The row values of a batch
+                // are read ahead of the chain.
                 constexpr int CB = 16;
 #pragma unroll
                 for (int i0 = 0; i0 < RC; i0 += CB) {
-                    if (gs + i0 < ge) {
-                        float xv[ROWS][CB];
+                    float xv[ROWS][CB];
 #pragma unroll
-                        for (int i = 0; i < CB; i++)
+                    for (int i = 0; i < CB; i++)
 #pragma unroll
-                            for (int r = 0; r < ROWS; r++) xv[r][i] = xs[r][min(gs + i0 + i, ge - 1)];
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int r = 0; r < ROWS; r++) xv[r][i] = (&xs[r][0])[gs + i0 + i];
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                        for (int i = 0; i < CB; i++)
-                            if (gs + i0 + i < ge) {
+                    for (int i = 0; i < CB; i++)
 #pragma unroll
-                                for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xv[r][i], rc[i0 + i], y[r]);
-                            }
-                    }
+                        for (int r = 0; r < ROWS; r++) y[r] = __builtin_fmaf(xv[r][i], rc[i0 + i], y[r]);
                 }
             } else
             // column j of the parked rotation against the rows, the LDS reads a batch ahead of
