@@ -602,24 +602,31 @@ template <int QG>
 __device__ __forceinline__ void rotate_q_group(const RotQArgs& a, const int64_t row, const int h,
                                                const int h_first, float* rot_s) {
     __shared__ uint16_t qraw[QG][D];
-    __shared__ float xs[QG][D];
+    __shared__ float xs[QG + 1][D];                 // (one more row of zeros, see the compact chain below)
     const int j = threadIdx.x;
     const bgtq_head_plan& P = a.plans[h];
+    // what thread j needs of the segment table comes ready-made (enc_dim), and so does its column of
+    // the rotation where the plan holds it by columns (no rotated segment longer than BGTQ_ROT_COL)
+    const int4 dim = *(const int4*)P.enc_dim[j];
+    const int g = dim.x, s = dim.y, e = dim.z, ident = dim.w & 0xFF, src = dim.w >> 8;
+    const bool compact = P.rot_compact[0] != 0;      // (uniform)
     rot_piece rst[D / 4];
-    fetch_rotation(P.k_rot_T, j, rst);
-    const int src = P.head_perm[j];
-    const int g = P.group_of[j];
-    int s = 0, e = 0, ident = 0;
+    float rc[BGTQ_ROT_COL];
+    if (compact) {
 #pragma unroll
-    for (int k = 0; k < BGTQ_MAX_SEGMENTS; k++) {
-        const int ks = P.seg_start[k], kl = P.seg_len[k], ki = P.seg_identity[k];
-        if (k == g) { s = ks; e = ks + kl; ident = ki; }
+        for (int i = 0; i < BGTQ_ROT_COL / 4; i++) {
+            const float4 v = *(const float4*)&P.k_rot_cols[j][4 * i];
+            rc[4 * i] = v.x; rc[4 * i + 1] = v.y; rc[4 * i + 2] = v.z; rc[4 * i + 3] = v.w;
+        }
+    } else {
+        fetch_rotation(P.k_rot_T, j, rst);
     }
     const int gqa = a.gqa;
 #pragma unroll
     for (int r = 0; r < QG; r++)
         qraw[r][j] = h_first + r < gqa ? a.q[row * a.q_sr + (int64_t)(h * gqa + h_first + r) * a.q_sh + j] : (uint16_t)0;
-    park_rotation(rot_s, j, rst);
+    xs[QG][j] = 0.f;
+    if (!compact) park_rotation(rot_s, j, rst);
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < QG; r++) xs[r][j] = bgtq_h2f(qraw[r][src]);
@@ -631,6 +638,23 @@ __device__ __forceinline__ void rotate_q_group(const RotQArgs& a, const int64_t 
         if (ident) {
 #pragma unroll
             for (int r = 0; r < QG; r++) acc[r] = xs[r][j];
+        } else if (compact) {
+            // the column is zero past the segment's end: BGTQ_ROT_COL terms for every dim, no length test
+            // (a term x * 0 leaves the sum as it is; the values read past the row are finite)
+            constexpr int CB = QG == 1 ? 16 : 8;
+#pragma unroll
+            for (int i0 = 0; i0 < BGTQ_ROT_COL; i0 += CB) {
+                float xv[QG][CB];
+#pragma unroll
+                for (int i = 0; i < CB; i++)
+#pragma unroll
+                    for (int r = 0; r < QG; r++) xv[r][i] = (&xs[r][0])[s + i0 + i];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < CB; i++)
+#pragma unroll
+                    for (int r = 0; r < QG; r++) acc[r] = __builtin_fmaf(xv[r][i], rc[i0 + i], acc[r]);
+            }
         } else {
             constexpr int CB = QG == 1 ? 16 : 8;    // LDS reads a batch ahead of the chains
             for (int k0 = s; k0 < e; k0 += CB) {
