@@ -44,24 +44,10 @@ struct EncodeArgs {
     int corrected;              // K codes path: emit corrected norms
 };
 
-// Byte `idx` of the LSB-first stream of bw-bit codes (bw <= 4) covers the codes
-// first .. first + n - 1, the first of them from its bit `skip` on.  None of this depends
-// on the row, so a thread works it out once and reuses it for every row of the tile.
+// One byte of the LSB-first stream of bw-bit codes (bw <= 4) covers the codes first .. first + n - 1,
+// the first of them from its bit `skip` on.  None of this depends on the row: the plan holds it per
+// record byte (enc_byte, enc_vbyte).
 struct StreamSlot { int first, n, skip; };
-__device__ inline StreamSlot stream_slot(int len, int bw, int idx) {
-    const int bit0 = idx * 8;
-    int first, skip;
-    switch (bw) {                               // constant divisors: no integer division at run time
-    case 1: first = bit0; skip = 0; break;
-    case 2: first = bit0 >> 1; skip = 0; break;
-    case 3: first = bit0 / 3; skip = bit0 - first * 3; break;
-    default: first = bit0 >> 2; skip = 0; break;
-    }
-    int last = (bit0 + 7) / (bw == 3 ? 3 : 1);
-    if (bw != 3) last = (bit0 + 7) >> (bw == 1 ? 0 : bw == 2 ? 1 : 2);
-    last = min(last, len - 1);
-    return {first, last - first + 1, skip};
-}
 __device__ inline unsigned stream_byte(const uint8_t* codes, StreamSlot s, int bw) {
     unsigned w = 0;
     for (int i = 0; i < s.n; i++) w |= (unsigned)codes[s.first + i] << (i * bw);
@@ -200,8 +186,10 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         k_byte = *(const uint2*)P.enc_byte[a.layout == BGTQ_K_MIXED ? 1 : 0][j];
         k_lut_off = P.lut_offset[j];
         k_lut_scale = P.lut_inv_scale[j];
+    } else if (j < D / 2) {
+        k_byte = *(const uint2*)P.enc_vbyte[a.layout == BGTQ_V_NIBBLE ? 1 : 0][j];
     }
-    // Decode append (2-row tiles) is latency bound.  K: the whole rotation matrix is requested now,
+    // Decode append (tiles of one or two rows) is latency bound.  K: the whole rotation matrix is requested now,
     // before anything else is known (which rows a thread needs is only known once the plan is in
     // LDS), 16 bytes a lane and contiguous across the wave (32 loads a thread), and parked in LDS
     // (rot_s) ahead of the rotation, which then reads its column from there.  16-row tiles fetch
@@ -231,18 +219,18 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
     }
     if constexpr (PF > 0) {
+        // (the plan holds v_rot_T four rows interleaved: 16-byte loads, contiguous across the threads)
 #pragma unroll
-        for (int i = 0; i < PF; i++) rpre[i] = RT[i * D + j];
+        for (int i = 0; i < PF / 4; i++) {
+            const float4 v = *(const float4*)P.v_rot_T4[i][j];
+            rpre[4 * i] = v.x; rpre[4 * i + 1] = v.y; rpre[4 * i + 2] = v.z; rpre[4 * i + 3] = v.w;
+        }
     }
     __syncthreads();
 
-    // ---- per-thread static data: K threads read theirs ready-made from the plan (requested in the
-    // first burst), V needs none -------------------------------------------
+    // ---- per-thread static data, read ready-made from the plan (requested in the first burst) ----
     int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
     float lut_off_j = 0.f, lut_scale_j = 0.f;          // K: this dim's cell-search parameters
-    int mode = 0;        // output byte j: 0: zero fill, 1: bit stream, 2: raw byte copy
-    int c0 = 0, clen = 0, bw = 1, idx = 0;
-    StreamSlot slot{0, 0, 0};
     if constexpr (!IS_V) {
         lut_off_j = k_lut_off;
         lut_scale_j = k_lut_scale;
@@ -252,15 +240,12 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         ge = k_dim.z;
         ident = k_dim.w & 0xFF;
         src_dim = k_dim.w >> 8;
-        mode = (int)(k_byte.x & 3u);
-        bw = (int)((k_byte.x >> 2) & 15u);
-        slot = StreamSlot{0, (int)(k_byte.x >> 8), (int)((k_byte.x >> 6) & 3u)};
-        c0 = (int)k_byte.y;                             // (the slot's first code is folded into the base)
-    } else {
-        bw = (a.layout == BGTQ_V_NIBBLE) ? 4 : sp.v_bits;
-        if (j < bgtq_seg_bytes(bw, D)) { mode = 1; c0 = 0; clen = D; idx = j; }
-        if (mode == 1) slot = stream_slot(clen, bw, idx);
     }
+    // output byte j: 0: zero fill, 1: bit stream, 2: raw byte copy
+    const int mode = (int)(k_byte.x & 3u);
+    const int bw = (int)((k_byte.x >> 2) & 15u);
+    const StreamSlot slot{0, (int)(k_byte.x >> 8), (int)((k_byte.x >> 6) & 3u)};
+    const int c0 = (int)k_byte.y;                       // (the slot's first code is folded into the base)
 
     for (int64_t tile = bx; tile < n_tiles; tile += tile_stride) {
     const int64_t row0 = tile * ROWS;

@@ -40,6 +40,7 @@ PLAN_DTYPE = np.dtype([
     ('v_centroids', '<f4', (16,)), ('v_boundaries', '<f4', (16,)),
     ('v_lut_f16', '<u2', (16,)),
     ('v_rot_T', '<f4', (_D * _D,)), ('v_rot', '<f4', (_D * _D,)),
+    ('v_rot_T4', '<f4', (_D // 4, _D, 4)), ('enc_vbyte', '<u4', (2, _D // 2, 2)),
     ('n_units', '<i4', (2,)), ('n_pair_units', '<i4', (2,)),
     ('kend', '<u4', (2,)), ('kfirst', '<u4', (2, 2)), ('reserved1', '<u4', (2,)),
     ('kprog', '<u4', (2, MAX_UNITS, 8)), ('kunit', '<u4', (2, MAX_UNITS)),
@@ -333,6 +334,14 @@ def build_head_plan(quantizer) -> np.ndarray:
     p['v_lut_f16'][:nv] = vc.astype(np.float16).view(np.uint16)
     p['v_rot_T'] = q._v_rot_T.detach().cpu().numpy().astype(np.float32).reshape(-1)
     p['v_rot'] = q._v_rot.detach().cpu().numpy().astype(np.float32).reshape(-1)
+    p['v_rot_T4'] = p['v_rot_T'].reshape(HEAD_DIM // 4, 4, HEAD_DIM).transpose(0, 2, 1)
+    p['enc_vbyte'][...] = 0
+    for layout, bw in ((V_BITPACKED, int(q._v_bits)), (V_NIBBLE, 4)):
+        for j in range(HEAD_DIM * bw // 8):
+            first = j * 8 // bw
+            skip = j * 8 - first * bw
+            n = min((j * 8 + 7) // bw, HEAD_DIM - 1) - first + 1
+            p['enc_vbyte'][layout, j] = [1 | (bw << 2) | (skip << 6) | (n << 8), first]
     fill_decode_steps(p)
     return p.reshape(1)
 

@@ -128,6 +128,13 @@ typedef struct bgtq_head_plan {
     uint16_t v_lut_f16[16];
     float    v_rot_T[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];  /* encode: y = vhat @ v_rot_T */
     float    v_rot[BGTQ_HEAD_DIM * BGTQ_HEAD_DIM];    /* decode: out = acc @ v_rot */
+    /* v_rot_T once more, four rows interleaved: v_rot_T4[q][j][c] = v_rot_T[(4 q + c) * 128 + j], so that
+     * the single-row append's thread j reads its column with 32 loads of 16 bytes that are contiguous
+     * across the threads */
+    float    v_rot_T4[BGTQ_HEAD_DIM / 4][BGTQ_HEAD_DIM][4];
+    /* what the V encoder's thread j needs as writer of record byte j (one table per V layout), in the
+     * format of enc_byte */
+    uint32_t enc_vbyte[2][BGTQ_HEAD_DIM / 2][2];
     /*
      * Decode schedule of the K record for the MFMA attention kernel, one per K
      * layout (index BGTQ_K_BITPACKED / BGTQ_K_MIXED).  A "unit" is 8 consecutive

@@ -633,3 +633,29 @@ def test_bench_allocations_follow_calibration_on_drawn_tensors():
             identical += int((diff == 0).all())
             total += 1
     assert identical >= total * 2 // 3, (identical, total)
+
+
+@pytest.mark.parametrize('v_bits', [2, 3, 4])
+def test_v_encoder_tables(v_bits):
+    """`enc_vbyte` assembles, byte by byte, the V record that the independent LSB-first bit-stream writer
+    writes (both layouts); `v_rot_T4` is `v_rot_T` with four rows interleaved."""
+    from blockgtq_amd import plan as P
+    q, _ = make_quantizer(seed=29, v_bits=v_bits)
+    p = q.plan()[0]
+    codes = np.random.default_rng(v_bits).integers(0, 1 << v_bits, 128)
+    for layout, bw in ((P.V_BITPACKED, v_bits), (P.V_NIBBLE, 4)):
+        n_bytes = 16 * bw
+        out = np.zeros(n_bytes, dtype=np.uint8)
+        for j in range(n_bytes):
+            w0, first = (int(x) for x in p['enc_vbyte'][layout, j])
+            mode, w, skip, n = w0 & 3, (w0 >> 2) & 15, (w0 >> 6) & 3, w0 >> 8
+            assert (mode, w) == (1, bw)
+            acc = 0
+            for i in range(n):
+                acc |= int(codes[first + i]) << (i * bw)
+            out[j] = (acc >> skip) & 255
+        assert np.array_equal(out, stream_pack(codes[None], bw)[0])
+        assert not p['enc_vbyte'][layout, n_bytes:].any()
+    vt = p['v_rot_T'].reshape(128, 128)
+    for r in (0, 1, 5, 66, 127):
+        assert np.array_equal(p['v_rot_T4'][r // 4, :, r % 4], vt[r])
