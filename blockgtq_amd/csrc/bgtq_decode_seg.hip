@@ -308,12 +308,19 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         return ((uint64_t)(uint32_t)b * (uint32_t)sb + (uint64_t)(uint32_t)h * (uint32_t)sh) * (uint32_t)elem;
     };
     const uint16_t* q_src = (const uint16_t*)((const uint8_t*)a.q + ((uint64_t)(uint32_t)b * (uint32_t)a.q_sb + (uint64_t)(uint32_t)(h * a.gqa_all + a.head0) * (uint32_t)a.q_sh) * 2u);
-    const int n_walk = min((int)P.n_walk[kl], BGTQ_MAX_WALK);
 
-    // ---- set-up jobs: job j < (HEADS + 1) * MAX_UNITS fills one 16-byte query slot (head j / MAX_UNITS, the
+    // ---- first requests.  The loads of the set-up are written as instructions of their own, so that a
+    // wait can leave the loads issued behind it in flight (the compiler would wait for all of them).
+    // Lane s < BGTQ_MAX_WALK of every wave keeps the words of step s of the record walk (read back with
+    // v_readlane; the steps past the last are zero in the plan, word 1 of a step in use is never zero).
+    uint4v seg_w = {0, 0, 0, 0};
+    {   // (every lane loads, so that no lane keeps an older value: the lanes behind the table repeat its last step)
+        const uint32_t* src = &P.swalk[kl][min(lane, BGTQ_MAX_WALK - 1)][0];
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(seg_w) : "v"(src) : "memory");
+    }
+    // Set-up jobs: job j < (HEADS + 1) * MAX_UNITS fills one 16-byte query slot (head j / MAX_UNITS, the
     // last struct is the zero row) from the plan's unit map: a slot holds the unit's up to 8 query values,
-    // zero where the unit has no dim.  The first N_QJOBS threads take one job each; their loads are written
-    // as instructions of their own, so that the wait for them can leave the tile loads issued later in flight.
+    // zero where the unit has no dim.  The first N_QJOBS threads take one job each.
     constexpr int N_QJOBS = (HEADS + 1) * MAX_UNITS;
     auto job_slot = [&](int j) -> uint32_t { const int jh = j / MAX_UNITS; return QS_OFF + jh * QSTRUCT + (j - jh * MAX_UNITS) * 16; };
     auto job_mask = [&](uint4v w, int len) -> uint4v {
@@ -323,53 +330,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     };
     const bool job_wave = wave * 64 < N_QJOBS;               // (uniform)
     uint32_t job_dsc = 0;
-    if (job_wave) {                                           // (every lane of the wave loads: no lane keeps an older value)
+    if (job_wave) {                                           // (every lane of the wave loads)
         const uint32_t* src = &P.sunit[kl][tid % MAX_UNITS];
         asm volatile("global_load_dword %0, %1, off" : "=v"(job_dsc) : "v"(src) : "memory");
     }
-    // segment words: lane s of every wave keeps the two words of segment s (read back with v_readlane)
-    uint32_t seg_w0 = 0, seg_w1 = 0, seg_w2 = 0;
-    if (lane < BGTQ_MAX_WALK) {                            // (steps past the last are zero in the plan: no wait for the count)
-        seg_w0 = P.swalk[kl][lane][0];
-        seg_w1 = P.swalk[kl][lane][1];
-        seg_w2 = P.swalk[kl][lane][2];
-    }
-
-    // the query words of this thread's job: requested as soon as the unit's dims are known
-    uint4v job_w = {0, 0, 0, 0};
-    int job_len = 0;
-    if (job_wave) {
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(job_dsc) :: "memory");
-        const int jh = tid / MAX_UNITS, d0 = (int)(job_dsc & 0xFF);
-        job_len = (tid < N_QJOBS && jh < gqa && jh < HEADS) ? (int)(job_dsc >> 8) : 0;
-        {   // every lane loads (a lane without a job reads the first head's row and masks everything out)
-            const uint32_t* row = (const uint32_t*)(q_src + (job_len > 0 ? jh : 0) * a.q_sh + d0);     // d0 is even
-            const int last = (D - d0) / 2 - 1;                                        // (a unit's words past the row's end repeat its last one: masked out below)
-            const uint32_t *r1 = row + min(1, last), *r2 = row + min(2, last), *r3 = row + min(3, last);
-            asm volatile("global_load_dword %0, %4, off\n\tglobal_load_dword %1, %5, off\n\t"
-                         "global_load_dword %2, %6, off\n\tglobal_load_dword %3, %7, off"
-                         : "=&v"(job_w[0]), "=&v"(job_w[1]), "=&v"(job_w[2]), "=&v"(job_w[3]) : "v"(row), "v"(r1), "v"(r2), "v"(r3) : "memory");
-        }
-    }
-
-    // ---- tables by DMA: V table at LDS offset 0, K tables behind it; the chunks are dealt round-robin
-    // to the first four waves (the others go straight on to their first tile)
     const uint32_t voff = (uint32_t)lane * 16;
-    const int tab_waves = min(nw, 4);
-    if (wave < tab_waves) {
-        const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
-        const uint8_t* kimg_src = (const uint8_t*)P.lut_image[kl];
-        const int vbytes = vlut_bytes(VBW, vnib), kbytes = P.n_walk[2 + kl] ? BGTQ_LUT_K5PEND : kimg_bytes(kl);
-        const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
-        for (int cc = wave; cc < vch + kch; cc += tab_waves) {
-            const uint8_t* src;
-            uint32_t dst;
-            int left;
-            if (cc < vch) { src = vimg + cc * 1024; dst = cc * 1024; left = vbytes - cc * 1024; }
-            else { src = kimg_src + (cc - vch) * 1024; dst = VTAB_BYTES + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
-            dma16(voff, src, __builtin_amdgcn_readfirstlane(dst), __builtin_amdgcn_ballot_w64((int)voff < left));
-        }
-    }
 
     // ---- per-wave buffers and streaming sources: 16-byte aligned bases and phases (constant per tile) ----
     const int wave_bytes = a.wave_bytes;
@@ -446,14 +411,59 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         voff_v += v_step;
         return n_loads;
     };
-    int tile = t0 + wave * MT;
-    int tile_loads = 0;
-    if (tile < t1) { tile_loads = issue_k(tile); tile_loads += issue_v(tile); }        // the wave's first tile: K and V travel together
-    bool v_issued = true, fresh = true;                    // (fresh: the wave has no sums yet)
+    // ---- tables by DMA: V table at LDS offset 0, the K image of the record layout behind it (all of it:
+    // what a plan does not use costs a few loads that the L2 serves, knowing it would cost a round trip);
+    // the 1 KB chunks are dealt round-robin to the waves from the last one down (the first ones have the
+    // query slots to fill)
+    int tab_loads = 0;
+    {
+        const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
+        const uint8_t* kimg_src = (const uint8_t*)P.lut_image[kl];
+        constexpr int vbytes_max = BGTQ_VLUT_BYTES;
+        const int vbytes = vlut_bytes(VBW, vnib), kbytes = BGTQ_LUT_IMAGE_BYTES;
+        static_assert(vbytes_max % 1024 == 0 && BGTQ_LUT_IMAGE_BYTES % 512 == 0, "");
+        const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
+        for (int cc = nw - 1 - wave; cc < vch + kch; cc += nw) {
+            const uint8_t* src;
+            uint32_t dst;
+            int left;
+            if (cc < vch) { src = vimg + cc * 1024; dst = cc * 1024; left = vbytes - cc * 1024; }
+            else { src = kimg_src + (cc - vch) * 1024; dst = VTAB_BYTES + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
+            dma16(voff, src, __builtin_amdgcn_readfirstlane(dst), __builtin_amdgcn_ballot_w64((int)voff < left));
+            tab_loads++;
+        }
+    }
 
-    // ---- the set-up slots.  The wait covers this wave's table chunks and query words and leaves its
-    // first tile in flight: the tile is waited for where it is used, by this wave alone
-    wait_loads(tile_loads);
+    // the query words of this thread's job: requested as soon as the unit's dims are known
+    uint4v job_w = {0, 0, 0, 0};
+    int job_len = 0;
+    if (job_wave) {
+        wait_loads(tab_loads);
+        asm volatile("" : "+v"(job_dsc) :: "memory");
+        const int jh = tid / MAX_UNITS, d0 = (int)(job_dsc & 0xFF);
+        job_len = (tid < N_QJOBS && jh < gqa && jh < HEADS) ? (int)(job_dsc >> 8) : 0;
+        {   // every lane loads (a lane without a job reads the first head's row and masks everything out)
+            const uint32_t* row = (const uint32_t*)(q_src + (job_len > 0 ? jh : 0) * a.q_sh + d0);     // d0 is even
+            const int last = (D - d0) / 2 - 1;                                        // (a unit's words past the row's end repeat its last one: masked out below)
+            const uint32_t *r1 = row + min(1, last), *r2 = row + min(2, last), *r3 = row + min(3, last);
+            asm volatile("global_load_dword %0, %4, off\n\tglobal_load_dword %1, %5, off\n\t"
+                         "global_load_dword %2, %6, off\n\tglobal_load_dword %3, %7, off"
+                         : "=&v"(job_w[0]), "=&v"(job_w[1]), "=&v"(job_w[2]), "=&v"(job_w[3]) : "v"(row), "v"(r1), "v"(r2), "v"(r3) : "memory");
+        }
+    }
+
+    // ---- the K records and norms of the wave's first tile.  The barrier below does not wait for them: a wave
+    // waits for its own tile where it uses it (the V records of a tile are requested when its K records are there)
+    int tile = t0 + wave * MT;
+    int k_loads = 0;
+    if (tile < t1) k_loads = issue_k(tile);
+    bool fresh = true;                                     // (the wave has no sums yet)
+
+    // ---- the set-up slots.  The wait covers the walk words, the wave's table chunks and query words
+    wait_loads(k_loads);
+    asm volatile("" : "+v"(seg_w) :: "memory");
+    const uint32_t seg_w0 = seg_w[0], seg_w1 = seg_w[1], seg_w2 = seg_w[2];
+    const int n_walk = __builtin_popcountll(__builtin_amdgcn_ballot_w64(lane < BGTQ_MAX_WALK && seg_w1 != 0));
     if (job_wave) {
         asm volatile("" : "+v"(job_w[0]), "+v"(job_w[1]), "+v"(job_w[2]), "+v"(job_w[3]) :: "memory");
         if (tid < N_QJOBS) lds_put<uint4v>(job_slot(tid), job_mask(job_w, job_len));
@@ -507,12 +517,11 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     for (; tile < t1; tile += step_tiles) {
         const int nt = min(MT, t1 - tile);
         const bool more = tile + step_tiles < t1;
-        // Streaming order: the V tile is requested when the K tile has arrived and the K tile of the
-        // wave's next tile when the V tile has, so every wait is for all loads in flight.
+        // Streaming order behind the first tile: the V tile is requested when the K tile has arrived and
+        // the K tile of the wave's next tile when the V tile has, so every wait is for all loads in flight.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // K records and norms of this tile are in LDS
         __builtin_amdgcn_wave_barrier();
-        if (!v_issued) issue_v(tile);                        // (the V buffer's last readers were the products of the previous tile)
-        v_issued = false;
+        issue_v(tile);                                       // (the V buffer's last readers were the products of the previous tile)
         const uint32_t vraw = lds_at<uint16_t>(vn_l);
 
         // ---- scores of this lane's token, HEADS heads, in log2 units ----------------------------------
