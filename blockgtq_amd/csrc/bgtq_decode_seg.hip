@@ -701,28 +701,29 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     // the head's reference over all waves, this wave's factor 2^(m_wave - m) and that factor times the
     // wave's denominator, left in LDS where the query rows were.  Step 2, one thread per (head, output):
     // the 16 scaled sums, the denominator, one store.
-    constexpr uint32_t F_OFF = QS_OFF, FL_OFF = QS_OFF + 8 * MAX_WAVES * 4, M_OFF = QS_OFF + 16 * MAX_WAVES * 4;
-    static_assert((HEADS + 1) * QSTRUCT >= 16 * MAX_WAVES * 4 + 32, "the fold's factors take the place of the query rows");
+    constexpr int FW = (MAX_WAVES + 3) & ~3;                 // factors per head, padded to whole 16-byte reads
+    constexpr uint32_t F_OFF = QS_OFF, FL_OFF = QS_OFF + 8 * FW * 4, M_OFF = QS_OFF + 16 * FW * 4;
+    static_assert((HEADS + 1) * QSTRUCT >= 16 * FW * 4 + 32, "the fold's factors take the place of the query rows");
     auto wave_base = [&](int w) -> uint32_t { return WAVES_OFF + (uint32_t)(min(w, nw - 1) * wave_bytes); };
-    for (int i = tid; i < 8 * MAX_WAVES; i += nthr) {
+    for (int i = tid; i < 8 * FW; i += nthr) {
         const int hh = i & 7, w = i >> 3;
         float m = -INFINITY;
 #pragma unroll
         for (int x = 0; x < MAX_WAVES; x++) m = fmaxf(m, lds_at<float>(wave_base(x) + hh * 4));     // (waves past the last repeat it)
         const float mine = lds_at<float>(wave_base(w) + hh * 4), l = lds_at<float>(wave_base(w) + 32 + hh * 4);
         const float f = (w < nw && mine != -INFINITY) ? __builtin_amdgcn_exp2f(mine - m) : 0.f;
-        lds_put<float>(F_OFF + (hh * MAX_WAVES + w) * 4, f);
-        lds_put<float>(FL_OFF + (hh * MAX_WAVES + w) * 4, f * l);
+        lds_put<float>(F_OFF + (hh * FW + w) * 4, f);
+        lds_put<float>(FL_OFF + (hh * FW + w) * 4, f * l);
         if (w == 0) lds_put<float>(M_OFF + hh * 4, m);
     }
     __syncthreads();
     for (int i = tid; i < gqa * 128; i += nthr) {
         const int hq = i >> 7, e = i & 127;                    // e = (li * 2 + (lg >> 1)) * 4 + jb
-        float4v f4[MAX_WAVES / 4], fl4[MAX_WAVES / 4];
+        float4v f4[FW / 4], fl4[FW / 4];
 #pragma unroll
-        for (int x = 0; x < MAX_WAVES / 4; x++) {
-            f4[x] = lds_at<float4v>(F_OFF + (hq * MAX_WAVES + 4 * x) * 4);
-            fl4[x] = lds_at<float4v>(FL_OFF + (hq * MAX_WAVES + 4 * x) * 4);
+        for (int x = 0; x < FW / 4; x++) {
+            f4[x] = lds_at<float4v>(F_OFF + (hq * FW + 4 * x) * 4);
+            fl4[x] = lds_at<float4v>(FL_OFF + (hq * FW + 4 * x) * 4);
         }
         float o[MAX_WAVES];
 #pragma unroll
