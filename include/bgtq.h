@@ -192,7 +192,8 @@ typedef struct bgtq_head_plan {
      * bit-packed codes of w bits; w = 4: a byte holds a code pair as nibbles, which is every
      * segment of up to 4 bits in BGTQ_K_MIXED), BGTQ_STEP_RAW5 + (units - 1) for 5-bit codes stored one
      * per byte and BGTQ_STEP_RAW + (units - 1) for wider codes stored one per byte.  n_walk[l] steps;
-     * all zero past the last.
+     * all zero past the last (the decode kernel counts the steps by their table word, which is never
+     * zero for a step in use, and copies all BGTQ_LUT_IMAGE_BYTES of lut_image[l]).
      * sunit[l][u] = first packed dim of unit u | number of real dims (1..8) << 8, units numbered
      * through the segments in order with no empty units between them; 0 past the last unit.
      */
