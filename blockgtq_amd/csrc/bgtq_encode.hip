@@ -453,8 +453,11 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     __syncthreads();
 
     // ---- 6. norms to store (raw or divided by ||centroids[codes]||) ---------
-    if (j < ROWS * BGTQ_MAX_SEGMENTS) {
-        int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
+    // Single-row tiles give this chain to the second wave: the first one packs the record meanwhile
+    // (neither needs anything of the other: the barrier between them is left out below).
+    const int jn = ROWS == 1 ? j - 64 : j;
+    if (jn >= 0 && jn < ROWS * BGTQ_MAX_SEGMENTS) {
+        int r = jn / BGTQ_MAX_SEGMENTS, gg = jn % BGTQ_MAX_SEGMENTS;
         float out = 0.f;
         if (gg < n_seg) {
             float n = nrm[r][gg];
@@ -477,7 +480,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
         }
         nrm_out[r][gg] = out;
     }
-    __syncthreads();
+    if (ROWS > 1 || a.codes_out) __syncthreads();       // (uniform; the cache norms below are stored by the thread that made them)
 
     // ---- 7a. unpacked outputs (codes path) ------------------------------------
     if (a.codes_out) {
@@ -497,8 +500,8 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     }
 
     // ---- 7b. cache norms --------------------------------------------------------
-    if (!a.codes_out && j < ROWS * BGTQ_MAX_SEGMENTS) {
-        int r = j / BGTQ_MAX_SEGMENTS, gg = j % BGTQ_MAX_SEGMENTS;
+    if (!a.codes_out && jn >= 0 && jn < ROWS * BGTQ_MAX_SEGMENTS) {
+        int r = jn / BGTQ_MAX_SEGMENTS, gg = jn % BGTQ_MAX_SEGMENTS;
         int64_t n = row0 + r;
         int width = IS_V ? 1 : a.norm_width;
         if (n < N && gg < width) {
