@@ -226,7 +226,7 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
             rpre[4 * i] = v.x; rpre[4 * i + 1] = v.y; rpre[4 * i + 2] = v.z; rpre[4 * i + 3] = v.w;
         }
     }
-    __syncthreads();
+    if constexpr (!IS_V) __syncthreads();     // (K reads the staged header next; V's staged tables are first read three barriers on)
 
     // ---- per-thread static data, read ready-made from the plan (requested in the first burst) ----
     int n_seg = 1, g = 0, gs = 0, ge = D, ident = 0, src_dim = j;
@@ -252,12 +252,18 @@ __device__ __forceinline__ void encode_rows(const EncodeArgs& a, const int bx, c
     int tcur[2] = {0, 0};              // this tile's positions (the prefetch below overwrites tp)
     if (ROWS <= 2) { tcur[0] = tp[0]; tcur[1] = tp[ROWS == 2 ? 1 : 0]; }
     // ---- 1. rows to LDS, next tile's rows on their way, gather by head_perm (K) -------------
+    if constexpr (IS_V) {              // (no gather: a thread converts its own value)
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) xraw[r][j] = xr[r];
-    __syncthreads();
-    if (tile + tile_stride < n_tiles) fetch_rows(tile + tile_stride);
+        for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xr[r]);
+        if (tile + tile_stride < n_tiles) fetch_rows(tile + tile_stride);
+    } else {
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xraw[r][src_dim]);
+        for (int r = 0; r < ROWS; r++) xraw[r][j] = xr[r];
+        __syncthreads();
+        if (tile + tile_stride < n_tiles) fetch_rows(tile + tile_stride);
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) xs[r][j] = bgtq_h2f(xraw[r][src_dim]);
+    }
     __syncthreads();
 
     // ---- 2. group norms: thread (r, grp) runs one sequential chain ---------
