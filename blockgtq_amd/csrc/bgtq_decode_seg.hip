@@ -69,11 +69,6 @@ constexpr int PBUF_BYTES = 4 * PROW;                             // P of a tile:
 constexpr int MERGE_BYTES = 64 + 8 * 32 * 16;                    // what a wave leaves for the merge: m, l, 8 heads x 128 floats
 
 __host__ __device__ constexpr int waves_off(int heads) { return QS_OFF + (heads + 1) * QSTRUCT; }
-__host__ __device__ constexpr int kimg_bytes(int k_layout) { return k_layout == BGTQ_K_MIXED ? BGTQ_LUTM_KEND : BGTQ_LUT_KEND; }
-__host__ __device__ constexpr int vlut_bytes(int vbw, bool nibble) {
-    return (nibble || vbw == 4) ? 1024 : (1 << (2 * vbw)) * 128;
-}
-
 __host__ __device__ inline TileLayout tile_layout(int krow, int vrow, int kn_st) {
     TileLayout t;
     t.kt = (MT * krow + 32 + 15) & ~15;
@@ -411,25 +406,23 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
         voff_v += v_step;
         return n_loads;
     };
-    // ---- tables by DMA: V table at LDS offset 0, the K image of the record layout behind it (all of it:
-    // what a plan does not use costs a few loads that the L2 serves, knowing it would cost a round trip);
+    // ---- tables by DMA: V table image at LDS offset 0, the K image of the record layout behind it (all of
+    // both: what a plan does not use costs a few loads that the L2 serves, knowing it would cost a round trip);
     // the 1 KB chunks are dealt round-robin to the waves from the last one down (the first ones have the
     // query slots to fill)
     int tab_loads = 0;
     {
+        // (chunk cc of the table area lies at LDS offset 1024 cc whichever image it belongs to: the V image
+        // takes the first BGTQ_VLUT_BYTES of the area whole, and both images are copied whole)
+        constexpr int VCH = BGTQ_VLUT_BYTES / 1024, NCH = VCH + (BGTQ_LUT_IMAGE_BYTES + 1023) / 1024;
+        constexpr int LAST_PIECES = (BGTQ_LUT_IMAGE_BYTES - (NCH - VCH - 1) * 1024) / 16;
+        static_assert(BGTQ_VLUT_BYTES % 1024 == 0 && VTAB_BYTES == BGTQ_VLUT_BYTES && LAST_PIECES >= 1 && LAST_PIECES <= 64, "");
         const uint8_t* vimg = (const uint8_t*)P.vlut_image[vnib ? 1 : 0];
-        const uint8_t* kimg_src = (const uint8_t*)P.lut_image[kl];
-        constexpr int vbytes_max = BGTQ_VLUT_BYTES;
-        const int vbytes = vlut_bytes(VBW, vnib), kbytes = BGTQ_LUT_IMAGE_BYTES;
-        static_assert(vbytes_max % 1024 == 0 && BGTQ_LUT_IMAGE_BYTES % 512 == 0, "");
-        const int vch = (vbytes + 1023) >> 10, kch = (kbytes + 1023) >> 10;
-        for (int cc = nw - 1 - wave; cc < vch + kch; cc += nw) {
-            const uint8_t* src;
-            uint32_t dst;
-            int left;
-            if (cc < vch) { src = vimg + cc * 1024; dst = cc * 1024; left = vbytes - cc * 1024; }
-            else { src = kimg_src + (cc - vch) * 1024; dst = VTAB_BYTES + (cc - vch) * 1024; left = kbytes - (cc - vch) * 1024; }
-            dma16(voff, src, __builtin_amdgcn_readfirstlane(dst), __builtin_amdgcn_ballot_w64((int)voff < left));
+        const uint8_t* kimg_m = (const uint8_t*)P.lut_image[kl] - VCH * 1024;
+        for (int cc = nw - 1 - wave; cc < NCH; cc += nw) {
+            const uint8_t* src = (cc < VCH ? vimg : kimg_m) + cc * 1024;
+            const uint64_t lanes = cc == NCH - 1 ? (LAST_PIECES >= 64 ? ~0ull : (1ull << LAST_PIECES) - 1ull) : ~0ull;
+            dma16(voff, src, (uint32_t)cc * 1024u, lanes);
             tab_loads++;
         }
     }
