@@ -161,8 +161,8 @@ __device__ __forceinline__ uint4v raw_unit_words(uint32_t xp, uint32_t tb) {
     return w;
 }
 
-// A run of NU units of W-bit codes read through pair tables (W = 1..3 bit-packed, 4: nibbles), as
-// straight-line code.  The run starts m bytes behind the 4-byte aligned LDS address a0 of this lane's
+// A run of NU units of W-bit codes read through pair tables (W = 3 bit-packed, 4: nibbles) or through
+// tables of four codes an entry (W = 1, 2 bit-packed), as straight-line code.  The run starts m bytes behind the 4-byte aligned LDS address a0 of this lane's
 // record; its bytes are read as aligned dwords and brought to bit 0 by one byte funnel each, after
 // which every field position is a constant: a field reaches its table-index position (bit SH up)
 // with one shift, or one bit funnel where it straddles two dwords.  A rows come from qa + 16 * unit.
@@ -174,8 +174,9 @@ __device__ __forceinline__ void step_pairs(float (&S)[8], float n, uint32_t a0, 
     constexpr int ND = (NU * W + 3) / 4;
     // (bit-packed codes of 1..3 bits: the table sits at a fixed place of the table area; nibble tables are one per
     // segment and their address comes with the step)
-    constexpr uint32_t FIXED = VTAB_BYTES + (W == 1 ? BGTQ_LUT_K1 : W == 2 ? BGTQ_LUT_K2 : BGTQ_LUT_K3);
-    const uint32_t tb = W == 4 ? tab : (rep | FIXED);
+    constexpr uint32_t FIXED = VTAB_BYTES + (W == 1 ? BGTQ_LUT_K1Q : W == 2 ? BGTQ_LUT_K2Q : BGTQ_LUT_K3);
+    static_assert((VTAB_BYTES + BGTQ_LUT_K1Q) % 128 == 0 && (VTAB_BYTES + BGTQ_LUT_K2Q) % 2048 == 0, "index bits are OR-ed into the table address");
+    const uint32_t tb = W == 4 ? tab : W == 3 ? (rep | FIXED) : FIXED;
     uint32_t r[ND + 1], e[ND];
 #pragma unroll
     for (int i = 0; i <= ND; i++) r[i] = lds_at<uint32_t>(a0 + 4 * i);      // (the last one may lie past the run: inside the tile buffer's slack)
@@ -186,19 +187,38 @@ __device__ __forceinline__ void step_pairs(float (&S)[8], float n, uint32_t a0, 
     uint4v w[NU];
 #pragma unroll
     for (int k = 0; k < NU; k++) {
-        uint32_t ad[4];
+        if constexpr (W <= 2) {
+            // 1- and 2-bit codes: four codes index an 8-byte entry of an unreplicated table (16 entries on 16
+            // bank pairs; 256 entries): two reads a unit instead of four
+            constexpr uint32_t QMASK = ((1u << (4 * W)) - 1u) << 3;
+            uint32_t ad[2];
 #pragma unroll
-        for (int p = 0; p < 4; p++) {
-            const int pos = 8 * W * k + 2 * W * p, i = pos >> 5, b = pos & 31;
-            uint32_t x;
-            if (b + 2 * W > 32) x = __builtin_amdgcn_alignbit(e[i + 1 < ND ? i + 1 : i], e[i], b - SH);
-            else if (b > SH) x = e[i] >> (b - SH);
-            else if (b < SH) x = e[i] << (SH - b);
-            else x = e[i];
-            ad[p] = and_or(x, MASK, tb);
+            for (int p = 0; p < 2; p++) {
+                const int pos = 8 * W * k + 4 * W * p, i = pos >> 5, b = pos & 31;     // (a field of 4 or 8 bits never straddles two dwords)
+                const uint32_t x = b > 3 ? e[i] >> (b - 3) : b < 3 ? e[i] << (3 - b) : e[i];
+                ad[p] = and_or(x, QMASK, tb);
+            }
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+                const uint2v r = lds_at<uint2v>(ad[p]);
+                w[k][2 * p] = r.x;
+                w[k][2 * p + 1] = r.y;
+            }
+        } else {
+            uint32_t ad[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const int pos = 8 * W * k + 2 * W * p, i = pos >> 5, b = pos & 31;
+                uint32_t x;
+                if (b + 2 * W > 32) x = __builtin_amdgcn_alignbit(e[i + 1 < ND ? i + 1 : i], e[i], b - SH);
+                else if (b > SH) x = e[i] >> (b - SH);
+                else if (b < SH) x = e[i] << (SH - b);
+                else x = e[i];
+                ad[p] = and_or(x, MASK, tb);
+            }
+#pragma unroll
+            for (int p = 0; p < 4; p++) w[k][p] = lds_at<uint32_t>(ad[p]);
         }
-#pragma unroll
-        for (int p = 0; p < 4; p++) w[k][p] = lds_at<uint32_t>(ad[p]);
         a[k] = lds_at<half8>(qa + 16 * k);
         // the MFMA of the unit before this one goes out while this unit's table words are on their way
         if (k == 1) acc.mma0(a[0], __builtin_bit_cast(half8, w[0]));

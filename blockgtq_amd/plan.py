@@ -45,12 +45,13 @@ PLAN_DTYPE = np.dtype([
     ('kend', '<u4', (2,)), ('kfirst', '<u4', (2, 2)), ('reserved1', '<u4', (2,)),
     ('kprog', '<u4', (2, MAX_UNITS, 8)), ('kunit', '<u4', (2, MAX_UNITS)),
     ('swalk', '<u4', (2, MAX_WALK, 4)), ('n_walk', '<u4', (4,)), ('sunit', '<u4', (2, MAX_UNITS)),
-    ('lut_image', '<u4', (2, 17920 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
+    ('lut_image', '<u4', (2, 20480 // 4)), ('vlut_image', '<u4', (2, 8192 // 4)),
 ], align=True)
 
 # byte offsets inside lut_image[K_BITPACKED] / lut_image[K_MIXED] (BGTQ_LUT_* / BGTQ_LUTM_* of include/bgtq.h)
 LUT_K = {3: 0, 2: 8192, 4: 10240, 1: 11264}    # each on a multiple of its size once VLUT_BYTES is added
-LUT_KRAW, LUT_K5P, LUT_IMAGE_BYTES = 11776, 13824, 17920
+LUT_KRAW, LUT_K5P, LUT_IMAGE_BYTES = 11776, 13824, 20480
+LUT_KQ = {1: 17920, 2: 18432}                  # four codes per 8-byte entry (decode kernel, bit-packed image)
 LUTM_KRAW = 4096
 VLUT_BYTES = 8192          # the kernel's table area starts with the V table; the K image follows it
 
@@ -88,6 +89,14 @@ def _byte_pair_table(cb16: np.ndarray, bw: int) -> np.ndarray:
     ok = (lo < (1 << bw)) & (hi < (1 << bw))
     pairs = cb16[np.where(ok, lo, 0)].astype(np.uint32) | (cb16[np.where(ok, hi, 0)].astype(np.uint32) << 16)
     return np.where(ok, pairs, 0).astype(np.uint32)
+
+
+def _quad_table(cb16: np.ndarray, bw: int) -> np.ndarray:
+    """Entry i = c0 | c1 << bw | c2 << 2 bw | c3 << 3 bw -> two words: (cb[c0] | cb[c1] << 16, cb[c2] | cb[c3] << 16)."""
+    i = np.arange(1 << (4 * bw))
+    m = (1 << bw) - 1
+    c = [cb16[(i >> (k * bw)) & m].astype(np.uint32) for k in range(4)]
+    return np.stack([c[0] | (c[1] << 16), c[2] | (c[3] << 16)], axis=1).reshape(-1)
 
 
 def _raw_table(cb16: np.ndarray, bw: int) -> np.ndarray:
@@ -212,6 +221,9 @@ def fill_decode_steps(p) -> None:
                     t = _byte_pair_table(cb, bw)
                     n_ptab += 1
                 img[table // 4:table // 4 + t.size] = t
+                if layout == K_BITPACKED and bw in LUT_KQ:
+                    q = _quad_table(cb, bw)
+                    img[LUT_KQ[bw] // 4:LUT_KQ[bw] // 4 + q.size] = q
                 row = [(pw * i - tsh) % 32 for i in range(4)] + [((1 << pw) - 1) << tsh, VLUT_BYTES + table, rep_mask]
                 n_pair += n_u
             else:

@@ -50,7 +50,12 @@ extern "C" {
 #define BGTQ_LUT_K5P     13824                   /* either image: 1024 entries (c0 | c1 << 5) for the 5-bit codebook, not
                                                   * replicated; present when n_walk[2 + layout] is non-zero */
 #define BGTQ_LUT_K5PEND  17920
-#define BGTQ_LUT_IMAGE_BYTES 17920               /* room for either K image */
+/* bit-packed image only, for the decode kernel: four codes per entry (index c0 | c1 << bw | c2 << 2 bw | c3 << 3 bw,
+ * 8 bytes = their four fp16 centroids), not replicated: 16 entries of 1-bit codes (every entry on a bank pair of its
+ * own) and 256 entries of 2-bit codes (on a multiple of its size in the kernel's table area) */
+#define BGTQ_LUT_K1Q     17920
+#define BGTQ_LUT_K2Q     18432
+#define BGTQ_LUT_IMAGE_BYTES 20480               /* room for either K image */
 /* how a segment's units are unpacked */
 #define BGTQ_PATH_B1     1   /* bit-packed 1-bit codes: a unit is 1 byte, pair table of 4 entries x 32 replicas */
 #define BGTQ_PATH_B2     2   /* bit-packed 2-bit codes: 2 bytes, 16 entries x 32 replicas */
