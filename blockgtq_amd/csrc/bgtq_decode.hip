@@ -799,8 +799,8 @@ int bgtq_window_swap(void* kbuf, void* vbuf, int64_t w_sb, int64_t w_sh, int64_t
 }
 
 size_t bgtq_plan_sizeof(void) { return sizeof(bgtq_head_plan); }
-int bgtq_abi_version(void) { return 6; }
-int bgtq_decode_kernel_revision(void) { return 6; }
+int bgtq_abi_version(void) { return 7; }
+int bgtq_decode_kernel_revision(void) { return 7; }
 
 const char* bgtq_strerror(int code) {
     switch (code) {

@@ -21,7 +21,8 @@
 //        per dword brings them to bit 0, and from there every field position is a constant:
 //        {shift, and-or, 4-byte table read} per code pair.  Tables of at most 64 entries are
 //        replicated 32 times (entry stride 128 bytes): LDS serves the 32 lanes of a half-wave
-//        together and the replicas put them on 32 different banks.
+//        together and the replicas put them on 32 different banks.  1- and 2-bit codes go four
+//        at a time through 8-byte entries of unreplicated tables (16 and 256 entries).
 //        One MFMA per unit: B = dequantised K (one token per lane), A = the unit's rotated
 //        queries, zero outside the lane's own lane group ("block diagonal"), so every lane
 //        receives the scores of its own token for all heads: v_mfma_f32_32x32x16_f16 for up

@@ -302,6 +302,10 @@ def test_decode_schedule_and_tables_cover_the_record(seed, min_bits, max_bits, b
                 for c1 in range(1 << bw):
                     assert int(t[c0 | (c1 << bw), 0]) == int(cb[c0]) | (int(cb[c1]) << 16)
                     assert int(tm[c0 | (c1 << 4)]) == int(cb[c0]) | (int(cb[c1]) << 16)
+            if bw in P.LUT_KQ:        # four codes an entry: the halves of its two words in code order
+                tq = img[P.LUT_KQ[bw] // 4:][:2 << (4 * bw)].view(np.uint16).reshape(-1, 4)
+                for i in range(1 << (4 * bw)):
+                    assert [int(x) for x in tq[i]] == [int(cb[(i >> (k * bw)) & ((1 << bw) - 1)]) for k in range(4)]
         else:
             for im, base in ((img, P.LUT_KRAW), (imgm, P.LUTM_KRAW)):
                 raw = im[(base + (bw - 5) * 512) // 4:][:128].view(np.uint16)
