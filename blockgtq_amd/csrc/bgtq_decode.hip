@@ -265,23 +265,28 @@ int launch_generic(const DecodeArgs& a, hipStream_t st) {
 }
 
 // ---- partition merge + V un-rotation ------------------------------------------
-// One work-group per (batch row, query head).  Its loads are 16 bytes a lane and
-// contiguous across the wave: thread t holds columns 4(t & 31) .. +3 of the rows
-// r = t >> 5 (mod 4) of the partial vectors and of the un-rotation, sums over its own
-// rows, and the four row classes are added through LDS (in a fixed order, so the result
+// One work-group of NTHR threads per (batch row, query head).  Its loads are 16 bytes a lane
+// and contiguous across the wave: thread t holds columns 4(t & 31) .. +3 of the rows
+// r = t >> 5 (mod NTHR / 32) of the partial vectors and of the un-rotation, sums over its own
+// rows, and the NTHR / 32 row classes are added through LDS (in a fixed order, so the result
 // does not depend on timing).  Every load that does not depend on a computed value
-// (the first 16 partial vectors, the whole un-rotation) is issued up front, so the
-// kernel pays for about one memory round trip of 36 wide loads a thread.
+// (the first round of partial vectors, the whole un-rotation) is issued up front, so the
+// kernel pays for about one memory round trip.  512 threads (16 classes: 8 rows of the
+// un-rotation a thread instead of 32) where the launch has at most one work-group per compute
+// unit, 128 threads where work-groups queue up.
 static_assert(offsetof(bgtq_head_plan, v_rot) % 16 == 0 && sizeof(bgtq_head_plan) % 16 == 0,
               "the un-rotation is read 16 bytes at a time");
-__global__ __launch_bounds__(D) void lse_reduce_kernel(
+template <int RT_THREADS>
+__global__ __launch_bounds__(RT_THREADS) void lse_reduce_kernel(
     const bgtq_head_plan* plans, const float* part_out, const float* part_lse, int n_splits,
     const float* extra_out, const float* extra_lse, int n_extra,
     int n_q, int gqa, int unrotate, uint16_t* out, int64_t o_sb, int64_t o_sh, float* lse_out) {
-    __shared__ __align__(16) float cls_sum[4][D];
+    constexpr int RT_CLASSES = RT_THREADS / 32;
+    __shared__ __align__(16) float cls_sum[RT_CLASSES][D];
     __shared__ float vec[D];
     __shared__ float wgt[BGTQ_MAX_SPLITS];
-    __shared__ float red[4];
+    __shared__ float red[RT_THREADS / 64];
+    __shared__ float dsum[RT_CLASSES];
     const int j = threadIdx.x;
     const int cls = j >> 5, c4 = (j & 31) * 4;
     const int hq = blockIdx.x, b = blockIdx.y;
@@ -294,31 +299,33 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     // loads land in issue order: the partitions' log-sum-exps go first, so that the maximum and
     // the weights are worked out while the vectors and the un-rotation are still on their way
     const float l_first = j < n_splits ? pl[j] : -INFINITY;
-    constexpr int NB = 4;                      // rounds of 4 partial vectors fetched before anything else
+    constexpr int NB = 16 / RT_CLASSES;        // rounds of partial vectors fetched before anything else (16 vectors)
     float4 pv[NB];
 #pragma unroll
-    for (int i = 0; i < NB; i++) pv[i] = *(const float4*)(po + (size_t)min(4 * i + cls, n_splits - 1) * D);
-    float4 rv[D / 4];                          // rows 4i + cls of the un-rotation, this thread's four columns
+    for (int i = 0; i < NB; i++) pv[i] = *(const float4*)(po + (size_t)min(RT_CLASSES * i + cls, n_splits - 1) * D);
+    float4 rv[D / RT_CLASSES];                 // rows 16 i + cls of the un-rotation, this thread's four columns
     if (unrotate) {
 #pragma unroll
-        for (int i = 0; i < D / 4; i++) rv[i] = *(const float4*)(R + (4 * i + cls) * D + c4);
+        for (int i = 0; i < D / RT_CLASSES; i++) rv[i] = *(const float4*)(R + (RT_CLASSES * i + cls) * D + c4);
     }
 
     float m = l_first;
     if (j < n_splits) wgt[j] = l_first;
-    for (int c = j + D; c < n_splits; c += D) { float l = pl[c]; wgt[c] = l; m = fmaxf(m, l); }
-    for (int c = j; c < n_extra; c += D) m = fmaxf(m, el[c]);
+    for (int c = j + RT_THREADS; c < n_splits; c += RT_THREADS) { float l = pl[c]; wgt[c] = l; m = fmaxf(m, l); }
+    for (int c = j; c < n_extra; c += RT_THREADS) m = fmaxf(m, el[c]);
     m = wave_max(m);
     if ((j & 63) == 0) red[j >> 6] = m;
     __syncthreads();
-    m = fmaxf(red[0], red[1]);
+    m = red[0];
+#pragma unroll
+    for (int i = 1; i < RT_THREADS / 64; i++) m = fmaxf(m, red[i]);
     if (m == -INFINITY) {                      // nothing visible at all
-        out[b * o_sb + hq * o_sh + j] = 0;
+        if (j < D) out[b * o_sb + hq * o_sh + j] = 0;
         if (lse_out && j == 0) lse_out[row] = -INFINITY;
         return;
     }
     // weights: exp(lse - m), 0 for empty partitions (their vectors are undefined)
-    for (int c = j; c < n_splits; c += D) { float l = wgt[c]; wgt[c] = (l == -INFINITY) ? 0.f : __expf(l - m); }
+    for (int c = j; c < n_splits; c += RT_THREADS) { float l = wgt[c]; wgt[c] = (l == -INFINITY) ? 0.f : __expf(l - m); }
     __syncthreads();
     float dcl = 0.f;                           // weight sum of this thread's row class
     float4 a4 = {0.f, 0.f, 0.f, 0.f};
@@ -328,36 +335,60 @@ __global__ __launch_bounds__(D) void lse_reduce_kernel(
     };
 #pragma unroll
     for (int i = 0; i < NB; i++)
-        if (4 * i + cls < n_splits) add(wgt[4 * i + cls], pv[i]);
-    for (int c = 4 * NB + cls; c < n_splits; c += 4) add(wgt[c], *(const float4*)(po + (size_t)c * D));
+        if (RT_CLASSES * i + cls < n_splits) add(wgt[RT_CLASSES * i + cls], pv[i]);
+    for (int c = RT_CLASSES * NB + cls; c < n_splits; c += RT_CLASSES) add(wgt[c], *(const float4*)(po + (size_t)c * D));
     *(float4*)&cls_sum[cls][c4] = a4;
-    if ((j & 31) == 0) red[cls] = dcl;         // (the maxima in red were read before the last barrier)
+    if ((j & 31) == 0) dsum[cls] = dcl;
     float acce = 0.f, den = 0.f;
-    for (int e = 0; e < n_extra; e++) {
-        float l = el[e];
-        if (l == -INFINITY) continue;
-        float w = __expf(l - m);
-        den += w;
-        acce += w * extra_out[(row * n_extra + e) * D + j];
-    }
+    if (j < D)
+        for (int e = 0; e < n_extra; e++) {
+            float l = el[e];
+            if (l == -INFINITY) continue;
+            float w = __expf(l - m);
+            den += w;
+            acce += w * extra_out[(row * n_extra + e) * D + j];
+        }
     __syncthreads();
-    den += (red[0] + red[1]) + (red[2] + red[3]);
-    float res = (cls_sum[0][j] + cls_sum[1][j]) + (cls_sum[2][j] + cls_sum[3][j]);
+    // the classes are added pairwise in a fixed order
+    auto fold = [&](const float (*t)[D], int col) {
+        float s[RT_CLASSES];
+#pragma unroll
+        for (int i = 0; i < RT_CLASSES; i++) s[i] = t[i][col];
+#pragma unroll
+        for (int w = RT_CLASSES / 2; w >= 1; w >>= 1)
+#pragma unroll
+            for (int i = 0; i < w; i++) s[i] = s[2 * i] + s[2 * i + 1];
+        return s[0];
+    };
+    float res = 0.f;
+    if (j < D) {
+        float ds[RT_CLASSES];
+#pragma unroll
+        for (int i = 0; i < RT_CLASSES; i++) ds[i] = dsum[i];
+#pragma unroll
+        for (int w = RT_CLASSES / 2; w >= 1; w >>= 1)
+#pragma unroll
+            for (int i = 0; i < w; i++) ds[i] = ds[2 * i] + ds[2 * i + 1];
+        den += ds[0];
+        res = fold(cls_sum, j);
+    }
     if (unrotate) {
-        vec[j] = res;
+        if (j < D) vec[j] = res;
         __syncthreads();                       // also: every read of cls_sum above is done
         float4 r4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < D / 4; i++) {
-            const float x = vec[4 * i + cls];
+        for (int i = 0; i < D / RT_CLASSES; i++) {
+            const float x = vec[RT_CLASSES * i + cls];
             r4.x += x * rv[i].x; r4.y += x * rv[i].y; r4.z += x * rv[i].z; r4.w += x * rv[i].w;
         }
         *(float4*)&cls_sum[cls][c4] = r4;
         __syncthreads();
-        res = (cls_sum[0][j] + cls_sum[1][j]) + (cls_sum[2][j] + cls_sum[3][j]);
+        if (j < D) res = fold(cls_sum, j);
     }
-    out[b * o_sb + hq * o_sh + j] = bgtq_f2h((res + acce) / den);
-    if (lse_out && j == 0) lse_out[row] = m + __logf(den);
+    if (j < D) {
+        out[b * o_sb + hq * o_sh + j] = bgtq_f2h((res + acce) / den);
+        if (lse_out && j == 0) lse_out[row] = m + __logf(den);
+    }
 }
 
 
@@ -710,10 +741,16 @@ int bgtq_lse_reduce(const bgtq_head_plan* plans,
     if (n_splits > BGTQ_MAX_SPLITS) return BGTQ_ELIMIT;
     if (B == 0 || n_kv == 0) return BGTQ_OK;
     dim3 grid((unsigned)(n_kv * gqa), (unsigned)B);
-    hipLaunchKernelGGL(lse_reduce_kernel, grid, dim3(D), 0, (hipStream_t)stream,
-                       plans, partial_out, partial_lse, n_splits,
-                       n_extra ? extra_out : nullptr, n_extra ? extra_lse : nullptr, n_extra,
-                       n_kv * gqa, gqa, unrotate, (uint16_t*)out, o_sb, o_sh, lse_out);
+    if ((int64_t)B * n_kv * gqa <= 256)
+        hipLaunchKernelGGL(lse_reduce_kernel<512>, grid, dim3(512), 0, (hipStream_t)stream,
+                           plans, partial_out, partial_lse, n_splits,
+                           n_extra ? extra_out : nullptr, n_extra ? extra_lse : nullptr, n_extra,
+                           n_kv * gqa, gqa, unrotate, (uint16_t*)out, o_sb, o_sh, lse_out);
+    else
+        hipLaunchKernelGGL(lse_reduce_kernel<128>, grid, dim3(128), 0, (hipStream_t)stream,
+                           plans, partial_out, partial_lse, n_splits,
+                           n_extra ? extra_out : nullptr, n_extra ? extra_lse : nullptr, n_extra,
+                           n_kv * gqa, gqa, unrotate, (uint16_t*)out, o_sb, o_sh, lse_out);
     return bgtq_launch_status();
 }
 
