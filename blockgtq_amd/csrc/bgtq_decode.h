@@ -23,6 +23,7 @@ struct DecodeArgs {
     int k_row_width;       // widest K record over the heads (LDS sizing)
     int v_row_width;
     int nw;                // MFMA kernel: waves per work-group
+    int nw_tiles;          // MFMA kernel: how many of them own tiles and tile buffers (the first ones)
     int p_over_k;          // MFMA kernel: the P tile lies over the K tile (no buffer of its own)
     TileLayout tl;
     int wave_bytes;        // MFMA kernel: LDS bytes of one wave's buffers

@@ -295,7 +295,8 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nw = a.nw, nthr = nw * 64;
+    const int nw = a.nw, nthr = nw * 64;                 // waves launched; the first nwt of them own tiles and tile buffers,
+    const int nwt = a.nw_tiles;                          // the others help with the set-up and the merge of short partitions
     const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const bgtq_head_plan& P = a.plans[h];
     const int gqa = a.gqa;
@@ -384,7 +385,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     const uint32_t knbuf = kbuf + tl.kt, vnbuf = knbuf + tl.knr;
     const DmaTail tail_k = tail_of(k_al, kbuf, full_k), tail_kn = tail_of(kn_al, knbuf, full_kn);
     const DmaTail tail_vn = tail_of(vn_al, vnbuf, full_vn), tail_v = tail_of(v_al, vbuf, full_v);
-    const int step_tiles = nw * MT;
+    const int step_tiles = nwt * MT;
     const uint32_t first = (uint32_t)(t0 + wave * MT);          // (a (row, head) slice is below 4 GB: checked by the launcher)
     // a lane's byte offset from the aligned base of each range, for the wave's current tile
     uint32_t voff_k = voff + first * (uint32_t)krow, voff_kn = voff + first * (uint32_t)(kn_st * 2);
@@ -468,7 +469,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
 
     // ---- the K records and norms of the wave's first tile.  The barrier below does not wait for them: a wave
     // waits for its own tile where it uses it (the V records of a tile are requested when its K records are there)
-    int tile = t0 + wave * MT;
+    int tile = wave < nwt ? t0 + wave * MT : t1;
     int k_loads = 0;
     if (tile < t1) k_loads = issue_k(tile);
     bool fresh = true;                                     // (the wave has no sums yet)
@@ -693,7 +694,7 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     // (dead by now), in the order the merging threads read them: [m 8][l 8][head 8][li 16][lg >> 1][jb 4].
     // After one barrier thread t of the first gqa * 32 owns head t / 32 and the four dims
     // 8 li + (lg >> 1) + {0, 2, 4, 6} with (li, lg >> 1) = t % 32 and folds the waves in a fixed order.
-    {
+    if (wave < nwt) {
         float lt[8];
 #pragma unroll
         for (int hh = 0; hh < 8; hh++) lt[hh] = l_part[hh];
@@ -718,43 +719,48 @@ __global__ __launch_bounds__(MAX_WAVES * 64) void decode_seg_kernel(DecodeArgs a
     constexpr int FW = (MAX_WAVES + 3) & ~3;                 // factors per head, padded to whole 16-byte reads
     constexpr uint32_t F_OFF = QS_OFF, FL_OFF = QS_OFF + 8 * FW * 4, M_OFF = QS_OFF + 16 * FW * 4;
     static_assert((HEADS + 1) * QSTRUCT >= 16 * FW * 4 + 32, "the fold's factors take the place of the query rows");
-    auto wave_base = [&](int w) -> uint32_t { return WAVES_OFF + (uint32_t)(min(w, nw - 1) * wave_bytes); };
+    auto wave_base = [&](int w) -> uint32_t { return WAVES_OFF + (uint32_t)(min(w, nwt - 1) * wave_bytes); };
     for (int i = tid; i < 8 * FW; i += nthr) {
         const int hh = i & 7, w = i >> 3;
         float m = -INFINITY;
 #pragma unroll
         for (int x = 0; x < MAX_WAVES; x++) m = fmaxf(m, lds_at<float>(wave_base(x) + hh * 4));     // (waves past the last repeat it)
         const float mine = lds_at<float>(wave_base(w) + hh * 4), l = lds_at<float>(wave_base(w) + 32 + hh * 4);
-        const float f = (w < nw && mine != -INFINITY) ? __builtin_amdgcn_exp2f(mine - m) : 0.f;
+        const float f = (w < nwt && mine != -INFINITY) ? __builtin_amdgcn_exp2f(mine - m) : 0.f;
         lds_put<float>(F_OFF + (hh * FW + w) * 4, f);
         lds_put<float>(FL_OFF + (hh * FW + w) * 4, f * l);
         if (w == 0) lds_put<float>(M_OFF + hh * 4, m);
     }
     __syncthreads();
-    for (int i = tid; i < gqa * 128; i += nthr) {
-        const int hq = i >> 7, e = i & 127;                    // e = (li * 2 + (lg >> 1)) * 4 + jb
-        float4v f4[FW / 4], fl4[FW / 4];
+    // (the sums of at most 4 waves where no more own tiles: short partitions)
+    auto fold = [&](auto nwf_c) {
+        constexpr int NWF = decltype(nwf_c)::value;
+        for (int i = tid; i < gqa * 128; i += nthr) {
+            const int hq = i >> 7, e = i & 127;                    // e = (li * 2 + (lg >> 1)) * 4 + jb
+            float4v f4[NWF / 4], fl4[NWF / 4];
 #pragma unroll
-        for (int x = 0; x < FW / 4; x++) {
-            f4[x] = lds_at<float4v>(F_OFF + (hq * FW + 4 * x) * 4);
-            fl4[x] = lds_at<float4v>(FL_OFF + (hq * FW + 4 * x) * 4);
+            for (int x = 0; x < NWF / 4; x++) {
+                f4[x] = lds_at<float4v>(F_OFF + (hq * FW + 4 * x) * 4);
+                fl4[x] = lds_at<float4v>(FL_OFF + (hq * FW + 4 * x) * 4);
+            }
+            float o[NWF];
+#pragma unroll
+            for (int w = 0; w < NWF; w++) o[w] = lds_at<float>(wave_base(w) + 64 + (hq * 128 + e) * 4);
+            float num = 0.f, den = 0.f;
+#pragma unroll
+            for (int w = 0; w < NWF; w++) {                       // (a wave past the last has factor 0)
+                num = fmaf(f4[w >> 2][w & 3], o[w], num);
+                den += fl4[w >> 2][w & 3];
+            }
+            const bool any = t1 > t0;
+            const float inv = any ? 1.f / den : 0.f;
+            const size_t row = ((size_t)b * a.n_kv * a.gqa_all + (size_t)h * a.gqa_all + a.head0 + hq) * a.n_splits + c;
+            const int x = e >> 2;
+            a.part_out[row * D + (x >> 1) * 8 + (e & 3) * 2 + (x & 1)] = num * inv;
+            if (e == 0) a.part_lse[row] = any ? (lds_at<float>(M_OFF + hq * 4) + log2f(den)) * 0.69314718055994530942f : -INFINITY;
         }
-        float o[MAX_WAVES];
-#pragma unroll
-        for (int w = 0; w < MAX_WAVES; w++) o[w] = lds_at<float>(wave_base(w) + 64 + (hq * 128 + e) * 4);
-        float num = 0.f, den = 0.f;
-#pragma unroll
-        for (int w = 0; w < MAX_WAVES; w++) {                 // (a wave past the last has factor 0)
-            num = fmaf(f4[w >> 2][w & 3], o[w], num);
-            den += fl4[w >> 2][w & 3];
-        }
-        const bool any = t1 > t0;
-        const float inv = any ? 1.f / den : 0.f;
-        const size_t row = ((size_t)b * a.n_kv * a.gqa_all + (size_t)h * a.gqa_all + a.head0 + hq) * a.n_splits + c;
-        const int x = e >> 2;
-        a.part_out[row * D + (x >> 1) * 8 + (e & 3) * 2 + (x & 1)] = num * inv;
-        if (e == 0) a.part_lse[row] = any ? (lds_at<float>(M_OFF + hq * 4) + log2f(den)) * 0.69314718055994530942f : -INFINITY;
-    }
+    };
+    if (nwt <= 4) fold(std::integral_constant<int, 4>{}); else fold(std::integral_constant<int, FW>{});
 }
 
 template <int HEADS>
@@ -775,7 +781,9 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
     while (nw > 1 && seg_smem_bytes<HEADS>(a.tl, nw, over) > (size_t)LDS_LIMIT) nw--;
     const size_t smem = seg_smem_bytes<HEADS>(a.tl, nw, over);
     if (smem > (size_t)LDS_LIMIT) return BGTQ_EUNSUPPORTED;
-    a.nw = nw;
+    // short partitions: more waves than own tiles share the table copies, the query slots and the merge
+    a.nw_tiles = nw;
+    a.nw = nw < 8 ? 8 : nw;
     a.p_over_k = over ? 1 : 0;
     a.wave_bytes = wave_lds_bytes(a.tl, over);
     {
@@ -809,7 +817,7 @@ int launch_kernel(DecodeArgs a, hipStream_t st) {
     }
     if (ready.load(std::memory_order_acquire) < 0) return BGTQ_EUNSUPPORTED;
     dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv, (unsigned)a.B);
-    hipLaunchKernelGGL(kern, grid, dim3(nw * 64), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(a.nw * 64), smem, st, a);
     return bgtq_launch_status();
 }
 
