@@ -699,18 +699,18 @@ __global__ __launch_bounds__(NT) void rotate_q_kernel(RotQArgs a) {
 constexpr int PREP_ROWS = 1;       // rows of a work-group in the one-launch preparation
 
 // ---- decode-step preparation: append-encode K and V and rotate the queries, one launch ----
-// Work-groups [0, nk) encode one K row each, [nk, nk + nv) one V row each, the rest rotate one or
-// four query heads each.
+// Work-groups [0, nv) encode one V row each (the longest chain of the three goes out first),
+// [nv, nv + nk) one K row each, the rest rotate one or four query heads each.
 __global__ __launch_bounds__(NT) void prepare_kernel(EncodeArgs ak, EncodeArgs av, RotQArgs aq,
                                                      int k_tiles, int v_tiles) {
     __shared__ __align__(16) float rot_s[D * D];       // the work-group's rotation, whatever its role
     int bid = blockIdx.x;
     const int nk = k_tiles * ak.n_kv, nv = v_tiles * av.n_kv;
-    if (bid < nk) {
-        encode_rows<PREP_ROWS, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles, rot_s);
-    } else if (bid < nk + nv) {
-        bid -= nk;
+    if (bid < nv) {
         encode_rows<PREP_ROWS, true>(av, bid % v_tiles, bid / v_tiles, v_tiles, v_tiles, rot_s);
+    } else if (bid < nk + nv) {
+        bid -= nv;
+        encode_rows<PREP_ROWS, false>(ak, bid % k_tiles, bid / k_tiles, k_tiles, k_tiles, rot_s);
     } else {
         rotate_q_block(aq, bid - (nk + nv), rot_s);
     }
